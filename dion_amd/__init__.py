@@ -1,0 +1,22 @@
+"""MI355X-native Muon / NorMuon / Dion2 optimizer-step kernels behind the microsoft/dion API."""
+from .newton_schulz import (  # noqa: F401
+    gram_newton_schulz,
+    newton_schulz_triton,
+    ns_line_1,
+    ns_line_2,
+    ns_line_3,
+    polar_express,
+    polar_express_triton,
+    zeropower_via_newtonschulz5,
+)
+
+__all__ = [
+    "gram_newton_schulz",
+    "newton_schulz_triton",
+    "ns_line_1",
+    "ns_line_2",
+    "ns_line_3",
+    "polar_express",
+    "polar_express_triton",
+    "zeropower_via_newtonschulz5",
+]

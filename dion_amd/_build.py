@@ -1,0 +1,56 @@
+"""Compile the HIP sources under dion_amd/csrc into dion_amd/libdion_hip.so (gfx950 only)."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_PATH = os.path.join(HERE, "libdion_hip.so")
+SOURCES = ["gemm_nt.hip", "elementwise.hip", "capi.hip"]
+
+# -packed-fp32-ops off: keep hipcc from forming v_pk_*_f32 out of scalar float code.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def hipcc_path() -> str:
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cand = os.path.join(rocm, "bin", "hipcc")
+    return cand if os.path.exists(cand) else "hipcc"
+
+
+def build(verbose: bool = True) -> str:
+    """Compile every source and link the shared library. Always recompiles."""
+    objs = []
+    procs = []
+    for src in SOURCES:
+        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        cmd = [hipcc_path(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+    for src, proc in procs:
+        out, _ = proc.communicate()
+        lines = [l for l in out.splitlines() if "packed-fp32-ops" not in l]
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n" + "\n".join(lines))
+        if verbose and lines:
+            print("\n".join(lines))
+    cmd = [hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()
+    print(LIB_PATH)
+    sys.exit(0)

@@ -1,0 +1,445 @@
+// extern "C" surface of libdion_hip.so (declared in include/dion_hip.h) and the host-side
+// Newton-Schulz driver that strings the GEMM launches together.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/dion_hip.h"
+#include "elementwise.h"
+
+using namespace dion;
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static int hip_fail(hipError_t e, const char* what) {
+  return fail(DION_E_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr, what)                     \
+  do {                                          \
+    hipError_t _e = (expr);                     \
+    if (_e != hipSuccess) return hip_fail(_e, what); \
+  } while (0)
+
+static inline int round_up(int v, int g) { return (v + g - 1) / g * g; }
+static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
+
+extern "C" const char* dion_last_error(void) { return g_err; }
+extern "C" int dion_abi_version(void) { return 1; }
+
+// ---------------------------------------------------------------------------------------------
+// Kernel-level GEMMs
+// ---------------------------------------------------------------------------------------------
+static int check_gemm_dims(const char* who, int batch, int m, int n) {
+  if (batch < 0 || m < 0 || n < 0) return fail(DION_E_INVALID, "%s: negative extent", who);
+  if (m % 128 || n % 128)
+    return fail(DION_E_INVALID, "%s: extents (%d, %d) must be multiples of 128", who, m, n);
+  return DION_OK;
+}
+
+extern "C" int dion_ns_line_1(const void* X, void* A, int batch, int m, int k, void* stream) {
+  if (int rc = check_gemm_dims("dion_ns_line_1", batch, m, k)) return rc;
+  if (batch == 0 || m == 0) return DION_OK;
+  if (k == 0) return fail(DION_E_INVALID, "dion_ns_line_1: k == 0");
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.P = p.Q = (const bf16_t*)X;
+  p.C = p.Ct = (bf16_t*)A;
+  p.strideP = p.strideQ = (int64_t)m * k;
+  p.strideC = p.strideCt = (int64_t)m * m;
+  p.ldp = p.ldq = k;
+  p.ldc = p.ldct = m;
+  p.M = p.N = p.Mst = p.Nst = m;
+  p.K = k;
+  p.batch = batch;
+  p.tri = 1;
+  p.alpha = 1.0f;
+  HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_1");
+  return DION_OK;
+}
+
+extern "C" int dion_ns_line_2(const void* A, void* B, int batch, int m, float alpha, float beta,
+                              void* stream) {
+  if (int rc = check_gemm_dims("dion_ns_line_2", batch, m, m)) return rc;
+  if (batch == 0 || m == 0) return DION_OK;
+  if (A == B) return fail(DION_E_INVALID, "dion_ns_line_2: in-place not supported");
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.P = p.Q = p.D = (const bf16_t*)A;
+  p.C = p.Ct = (bf16_t*)B;
+  p.strideP = p.strideQ = p.strideD = p.strideC = p.strideCt = (int64_t)m * m;
+  p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = m;
+  p.M = p.N = p.K = p.Mst = p.Nst = m;
+  p.batch = batch;
+  p.tri = 1;
+  p.alpha = alpha;
+  p.beta = beta;
+  HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_2");
+  return DION_OK;
+}
+
+extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void* C, void* Ct,
+                              int batch, int m, int n, float a, void* stream) {
+  if (int rc = check_gemm_dims("dion_ns_line_3", batch, m, n)) return rc;
+  if (batch == 0 || m == 0 || n == 0) return DION_OK;
+  if (!C && !Ct) return fail(DION_E_INVALID, "dion_ns_line_3: no output");
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.P = (const bf16_t*)B;
+  p.Q = (const bf16_t*)Xt;
+  p.D = (const bf16_t*)X;
+  p.C = (bf16_t*)C;
+  p.Ct = (bf16_t*)Ct;
+  p.strideP = (int64_t)m * m;
+  p.strideQ = p.strideD = p.strideC = p.strideCt = (int64_t)m * n;
+  p.ldp = m;
+  p.ldq = m;
+  p.ldd = n;
+  p.ldc = n;
+  p.ldct = m;
+  p.M = p.Mst = m;
+  p.N = p.Nst = n;
+  p.K = m;
+  p.batch = batch;
+  p.tri = 0;
+  p.alpha = 1.0f;
+  p.beta = a;
+  HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_3");
+  return DION_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Whole orthogonalization
+// ---------------------------------------------------------------------------------------------
+namespace {
+struct NsPlan {
+  int m, n, mp, np, tall, nblk;
+  size_t x_bytes, a_bytes, partial_bytes, inv_bytes, total;
+};
+
+NsPlan make_plan(int batch, int rows, int cols, int flags) {
+  NsPlan pl;
+  pl.tall = rows > cols;
+  pl.m = pl.tall ? cols : rows;
+  pl.n = pl.tall ? rows : cols;
+  const int g = gemm_pad_granule(pl.m, pl.n, batch);
+  pl.mp = round_up(pl.m, g);
+  pl.np = round_up(pl.n, g);
+  const int64_t numel = (int64_t)rows * cols;
+  int64_t nb = numel / (256 * 16);
+  if (nb < 1) nb = 1;
+  if (nb > 256) nb = 256;
+  pl.nblk = (int)nb;
+  pl.x_bytes = align256((size_t)batch * pl.mp * pl.np * 2);
+  pl.a_bytes = align256((size_t)batch * pl.mp * pl.mp * 2);
+  pl.partial_bytes = align256((size_t)batch * pl.nblk * 4);
+  pl.inv_bytes = align256((size_t)batch * 4);
+  // X, Xt ping-pong pairs; A, B (+ Q, Z, T for the Gram recurrence)
+  const int n_sq = (flags & DION_NS_GRAM) ? 6 : 2;
+  pl.total = 4 * pl.x_bytes + n_sq * pl.a_bytes + pl.partial_bytes + pl.inv_bytes;
+  return pl;
+}
+}  // namespace
+
+extern "C" size_t dion_ns_workspace_bytes(int batch, int rows, int cols, int flags) {
+  if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
+  return make_plan(batch, rows, cols, flags).total;
+}
+
+extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, int rows,
+                                     int cols, const float* coeffs, int n_iters, float norm_scale,
+                                     float eps, int flags, int gram_reset, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+  if (batch < 0 || rows < 0 || cols < 0 || n_iters < 0)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize: negative extent");
+  if (in_dtype != DION_BF16 && in_dtype != DION_F32)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize: in_dtype %d", in_dtype);
+  if (batch == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!in || !out || (n_iters > 0 && !coeffs))
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize: null argument");
+  if (flags & ~DION_NS_GRAM) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
+  if (flags & DION_NS_GRAM) return fail(DION_E_INVALID, "dion_ns_orthogonalize: Gram recurrence not built");
+  (void)gram_reset;
+  const NsPlan pl = make_plan(batch, rows, cols, flags);
+  if (!workspace || workspace_bytes < pl.total)
+    return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize: workspace %zu < %zu bytes", workspace_bytes,
+                pl.total);
+  if (((uintptr_t)workspace & 255) != 0)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize: workspace not 256-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+
+  char* w = (char*)workspace;
+  bf16_t* X[2];
+  bf16_t* Xt[2];
+  X[0] = (bf16_t*)w; w += pl.x_bytes;
+  X[1] = (bf16_t*)w; w += pl.x_bytes;
+  Xt[0] = (bf16_t*)w; w += pl.x_bytes;
+  Xt[1] = (bf16_t*)w; w += pl.x_bytes;
+  bf16_t* A = (bf16_t*)w; w += pl.a_bytes;
+  bf16_t* Bm = (bf16_t*)w; w += pl.a_bytes;
+  float* partial = (float*)w; w += pl.partial_bytes;
+  float* inv = (float*)w; w += pl.inv_bytes;
+
+  const int mp = pl.mp, np = pl.np;
+  HIP_TRY(launch_frobenius_inv(in, in_dtype, batch, (int64_t)rows * cols, norm_scale, eps, partial,
+                               pl.nblk, inv, st),
+          "frobenius norm");
+  if (pl.tall)
+    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, Xt[0], np, mp, X[0], st), "prepare");
+  else
+    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, X[0], mp, np, Xt[0], st), "prepare");
+
+  const bool direct = (mp == pl.m && np == pl.n);
+  int cur = 0;
+  for (int it = 0; it < n_iters; ++it) {
+    const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
+    GemmParams p;
+    // A = X X^T
+    memset(&p, 0, sizeof(p));
+    p.P = p.Q = X[cur];
+    p.C = p.Ct = A;
+    p.strideP = p.strideQ = (int64_t)mp * np;
+    p.strideC = p.strideCt = (int64_t)mp * mp;
+    p.ldp = p.ldq = np;
+    p.ldc = p.ldct = mp;
+    p.M = p.N = p.Mst = p.Nst = mp;
+    p.K = np;
+    p.batch = batch;
+    p.tri = 1;
+    p.alpha = 1.0f;
+    HIP_TRY(launch_gemm_nt(p, -1, st), "A = X X^T");
+    // B = c A A + b A
+    memset(&p, 0, sizeof(p));
+    p.P = p.Q = p.D = A;
+    p.C = p.Ct = Bm;
+    p.strideP = p.strideQ = p.strideD = p.strideC = p.strideCt = (int64_t)mp * mp;
+    p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = mp;
+    p.M = p.N = p.K = p.Mst = p.Nst = mp;
+    p.batch = batch;
+    p.tri = 1;
+    p.alpha = c;
+    p.beta = b;
+    HIP_TRY(launch_gemm_nt(p, -1, st), "B = c A A + b A");
+    // X' = a X + B X   (and its transpose)
+    memset(&p, 0, sizeof(p));
+    p.P = Bm;
+    p.Q = Xt[cur];
+    p.D = X[cur];
+    p.strideP = (int64_t)mp * mp;
+    p.strideQ = p.strideD = (int64_t)mp * np;
+    p.ldp = mp;
+    p.ldq = mp;
+    p.ldd = np;
+    p.M = p.Mst = mp;
+    p.N = p.Nst = np;
+    p.K = mp;
+    p.batch = batch;
+    p.alpha = 1.0f;
+    p.beta = a;
+    const bool last = (it == n_iters - 1);
+    if (last && direct) {
+      if (pl.tall) {
+        p.Ct = (bf16_t*)out;
+        p.strideCt = (int64_t)mp * np;
+        p.ldct = mp;
+      } else {
+        p.C = (bf16_t*)out;
+        p.strideC = (int64_t)mp * np;
+        p.ldc = np;
+      }
+    } else {
+      p.C = X[cur ^ 1];
+      p.Ct = Xt[cur ^ 1];
+      p.strideC = p.strideCt = (int64_t)mp * np;
+      p.ldc = np;
+      p.ldct = mp;
+    }
+    HIP_TRY(launch_gemm_nt(p, -1, st), "X = a X + B X");
+    cur ^= 1;
+  }
+  if (!(direct && n_iters > 0)) {
+    if (pl.tall)
+      HIP_TRY(launch_unpad(Xt[cur], (int64_t)mp * np, mp, (bf16_t*)out, batch, rows, cols, st), "unpad");
+    else
+      HIP_TRY(launch_unpad(X[cur], (int64_t)mp * np, np, (bf16_t*)out, batch, rows, cols, st), "unpad");
+  }
+  return DION_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Memory-bound kernels
+// ---------------------------------------------------------------------------------------------
+static bool table_aligned(const uint64_t* t, int n) {
+  for (int i = 0; i < n; ++i)
+    if (!aligned16(t[i])) return false;
+  return true;
+}
+
+static void fill_tab(PtrTab& tab, const uint64_t* src, int n) {
+  memset(&tab, 0, sizeof(tab));
+  memcpy(tab.p, src, (size_t)n * sizeof(uint64_t));
+}
+
+extern "C" int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, void* U,
+                             int n, int64_t numel, float mu, int nesterov, void* stream) {
+  if (n < 0 || numel < 0) return fail(DION_E_INVALID, "dion_muon_pre: negative size");
+  if (g_dtype != DION_BF16 && g_dtype != DION_F32) return fail(DION_E_INVALID, "dion_muon_pre: g_dtype");
+  if (n == 0 || numel == 0) return DION_OK;
+  if (!G_ptrs || !M_ptrs || !U) return fail(DION_E_INVALID, "dion_muon_pre: null argument");
+  const bool vec = (numel % 8 == 0) && table_aligned(G_ptrs, n) && table_aligned(M_ptrs, n) &&
+                   aligned16((uint64_t)U);
+  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
+    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+    PtrTab g, m;
+    fill_tab(g, G_ptrs + i0, c);
+    fill_tab(m, M_ptrs + i0, c);
+    HIP_TRY(launch_muon_pre(g, g_dtype, m, (bf16_t*)U + (int64_t)i0 * numel, c, numel, mu, nesterov,
+                            vec, (hipStream_t)stream),
+            "dion_muon_pre");
+  }
+  return DION_OK;
+}
+
+extern "C" int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype, int n,
+                              int64_t numel, int cols, const float* row_scale, const float* lr_dev,
+                              float adj_ratio, const float* wd_dev, float wd_host, int cautious,
+                              void* stream) {
+  if (n < 0 || numel < 0 || cols <= 0) return fail(DION_E_INVALID, "dion_muon_post: bad size");
+  if (u_dtype != DION_BF16 && u_dtype != DION_F32) return fail(DION_E_INVALID, "dion_muon_post: u_dtype");
+  if (n == 0 || numel == 0) return DION_OK;
+  if (numel % cols) return fail(DION_E_INVALID, "dion_muon_post: numel %% cols != 0");
+  if (!X_ptrs || !U || !lr_dev) return fail(DION_E_INVALID, "dion_muon_post: null argument");
+  const size_t usz = u_dtype == DION_BF16 ? 2 : 4;
+  const bool vec = (numel % 8 == 0) && (cols % 8 == 0) && table_aligned(X_ptrs, n) &&
+                   aligned16((uint64_t)U);
+  const int64_t rows = numel / cols;
+  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
+    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+    PtrTab x;
+    fill_tab(x, X_ptrs + i0, c);
+    HIP_TRY(launch_muon_post(x, (const char*)U + (size_t)i0 * numel * usz, u_dtype, c, numel, cols,
+                             row_scale ? row_scale + (int64_t)i0 * rows : nullptr, lr_dev, adj_ratio,
+                             wd_dev, wd_host, cautious, vec, (hipStream_t)stream),
+            "dion_muon_post");
+  }
+  return DION_OK;
+}
+
+extern "C" int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr,
+                                  int rows, int cols, float beta2, float* row_scale, float* scratch,
+                                  void* stream) {
+  (void)scratch;
+  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0)
+    return fail(DION_E_INVALID, "dion_normuon_stats: bad size");
+  if (n == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!U || !V_ptrs || !row_scale) return fail(DION_E_INVALID, "dion_normuon_stats: null argument");
+  const float w = 1.0f - beta2;
+  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
+    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+    PtrTab v;
+    fill_tab(v, V_ptrs + i0, c);
+    const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
+    HIP_TRY(launch_normuon_stats((const bf16_t*)U + mat0 * rows * cols, v, c * mats_per_ptr, 0,
+                                 mats_per_ptr, rows, cols, w, row_scale + mat0 * rows,
+                                 (hipStream_t)stream),
+            "dion_normuon_stats");
+  }
+  return DION_OK;
+}
+
+static int check_select_dim(const char* who, int select_dim) {
+  if (select_dim != -2 && select_dim != -1)
+    return fail(DION_E_INVALID, "%s: select_dim must be -2 or -1, got %d", who, select_dim);
+  return DION_OK;
+}
+
+extern "C" int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs,
+                                     int n, int mats_per_ptr, int rows, int cols, int select_dim,
+                                     float* norms, void* stream) {
+  if (int rc = check_select_dim("dion_dion2_accumulate", select_dim)) return rc;
+  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0)
+    return fail(DION_E_INVALID, "dion_dion2_accumulate: bad size");
+  if (g_dtype != DION_BF16 && g_dtype != DION_F32)
+    return fail(DION_E_INVALID, "dion_dion2_accumulate: g_dtype");
+  if (n == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!G_ptrs || !M_ptrs || !norms) return fail(DION_E_INVALID, "dion_dion2_accumulate: null argument");
+  const int dim = select_dim == -2 ? rows : cols;
+  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
+    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+    PtrTab g, m;
+    fill_tab(g, G_ptrs + i0, c);
+    fill_tab(m, M_ptrs + i0, c);
+    HIP_TRY(launch_dion2_accumulate(g, g_dtype, m, c * mats_per_ptr, mats_per_ptr, rows, cols,
+                                    select_dim == -2, norms + (int64_t)i0 * mats_per_ptr * dim,
+                                    (hipStream_t)stream),
+            "dion_dion2_accumulate");
+  }
+  return DION_OK;
+}
+
+extern "C" int dion_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
+                               int32_t* map, void* stream) {
+  if (n_mat < 0 || dim < 0 || k < 0 || k > dim) return fail(DION_E_INVALID, "dion_dion2_topk: bad size");
+  if (n_mat == 0 || dim == 0) return DION_OK;
+  if ((size_t)dim * 4 + 128 > 160 * 1024 - 256)
+    return fail(DION_E_INVALID, "dion_dion2_topk: dim %d exceeds the LDS-resident limit", dim);
+  if (!norms || !idx || !map) return fail(DION_E_INVALID, "dion_dion2_topk: null argument");
+  HIP_TRY(launch_dion2_topk(norms, n_mat, dim, k, idx, map, (hipStream_t)stream), "dion_dion2_topk");
+  return DION_OK;
+}
+
+extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr, int rows, int cols,
+                                 int select_dim, const int32_t* idx, int k, float ef_decay,
+                                 void* U_sel, void* stream) {
+  if (int rc = check_select_dim("dion_dion2_gather", select_dim)) return rc;
+  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || k < 0)
+    return fail(DION_E_INVALID, "dion_dion2_gather: bad size");
+  if (n == 0 || rows == 0 || cols == 0 || k == 0) return DION_OK;
+  if (!M_ptrs || !idx || !U_sel) return fail(DION_E_INVALID, "dion_dion2_gather: null argument");
+  const int64_t sel_numel = select_dim == -2 ? (int64_t)k * cols : (int64_t)rows * k;
+  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
+    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+    PtrTab m;
+    fill_tab(m, M_ptrs + i0, c);
+    const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
+    HIP_TRY(launch_dion2_gather(m, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
+                                idx + mat0 * k, k, ef_decay, (bf16_t*)U_sel + mat0 * sel_numel,
+                                (hipStream_t)stream),
+            "dion_dion2_gather");
+  }
+  return DION_OK;
+}
+
+extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, int cols,
+                               int select_dim, const void* U_sel, int k, const int32_t* map,
+                               const float* lr_dev, float adj_ratio, const float* wd_dev,
+                               float wd_host, void* stream) {
+  if (int rc = check_select_dim("dion_dion2_post", select_dim)) return rc;
+  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || k < 0)
+    return fail(DION_E_INVALID, "dion_dion2_post: bad size");
+  if (n == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!X_ptrs || !map || !lr_dev || (k > 0 && !U_sel))
+    return fail(DION_E_INVALID, "dion_dion2_post: null argument");
+  const int dim = select_dim == -2 ? rows : cols;
+  const int64_t sel_numel = select_dim == -2 ? (int64_t)k * cols : (int64_t)rows * k;
+  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
+    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+    PtrTab x;
+    fill_tab(x, X_ptrs + i0, c);
+    const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
+    HIP_TRY(launch_dion2_post(x, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
+                              (const bf16_t*)U_sel + mat0 * sel_numel, k, map + mat0 * dim, lr_dev,
+                              adj_ratio, wd_dev, wd_host, (hipStream_t)stream),
+            "dion_dion2_post");
+  }
+  return DION_OK;
+}

@@ -1,0 +1,58 @@
+// Shared declarations for the gfx950 kernels behind the C-ABI in include/dion_hip.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dion {
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits in memory
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// Round-to-nearest-even float -> bf16 (hardware v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, b);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2 v;
+  v[0] = (__bf16)lo;
+  v[1] = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// One batched C = alpha * P * Q^T + beta * D problem, all operands row-major bf16 with the
+// reduction dimension contiguous ("NT" GEMM).  M, N, K are the computed extents and must be
+// multiples of the tile the launcher picks; Mst/Nst bound the stores (<= M, N) so the last
+// GEMM of a chain can write into an unpadded destination.
+struct GemmParams {
+  const bf16_t* P;   // [batch][M][K], leading dimension ldp
+  const bf16_t* Q;   // [batch][N][K], leading dimension ldq (== P when tri)
+  const bf16_t* D;   // optional [batch][M][N] addend, leading dimension ldd
+  bf16_t* C;         // optional [batch][Mst][Nst]
+  bf16_t* Ct;        // optional [batch][Nst][Mst] (transposed copy; == C when tri -> mirror)
+  int64_t strideP, strideQ, strideD, strideC, strideCt;  // batch strides in elements
+  int ldp, ldq, ldd, ldc, ldct;
+  int M, N, K;
+  int Mst, Nst;
+  int batch;
+  int tri;           // 1: Q == P, only tiles with tile_row <= tile_col are computed, Ct mirrors
+  float alpha, beta;
+};
+
+// Returns hipSuccess or the launch error.  variant < 0 picks by shape.
+hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream);
+// Tile edge (128 or 256) launch_gemm_nt would use for a problem whose padded short/long
+// dims are given; workspaces are padded to this.
+int gemm_pad_granule(int m, int n, int batch);
+
+}  // namespace dion

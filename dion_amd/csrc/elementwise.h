@@ -1,0 +1,45 @@
+// Launchers for the memory-bound kernels in elementwise.hip (internal; the public surface is
+// include/dion_hip.h).
+#pragma once
+#include "common.h"
+
+namespace dion {
+
+// Up to kMaxPtrs device pointers passed by value in the kernel-argument segment: the
+// list-of-parameters of one shape group reaches the GPU without a host->device copy.
+constexpr int kMaxPtrs = 64;
+struct PtrTab {
+  uint64_t p[kMaxPtrs];
+};
+
+hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t numel,
+                                float norm_scale, float eps, float* partial, int nblk,
+                                float* inv_norm, hipStream_t st);
+hipError_t launch_ns_prepare(const void* in, int in_dtype, int batch, int R, int C,
+                             const float* inv_norm, bf16_t* same, int Rp, int Cp, bf16_t* trans,
+                             hipStream_t st);
+hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* dst, int batch, int R,
+                        int C, hipStream_t st);
+hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, bf16_t* U, int n,
+                           int64_t numel, float mu, int nesterov, bool vec, hipStream_t st);
+hipError_t launch_muon_post(const PtrTab& X, const void* U, int u_dtype, int n, int64_t numel,
+                            int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
+                            const float* wd_dev, float wd_host, int cautious, bool vec,
+                            hipStream_t st);
+hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int n_mat, int mat0,
+                                int mats_per_ptr, int rows, int cols, float w, float* row_scale,
+                                hipStream_t st);
+hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int n_mat,
+                                   int mats_per_ptr, int rows, int cols, int select_rows,
+                                   float* norms, hipStream_t st);
+hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
+                             int32_t* map, hipStream_t st);
+hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int rows, int cols,
+                               int select_rows, const int32_t* idx, int k, float ef_decay, bf16_t* U,
+                               hipStream_t st);
+hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
+                             int select_rows, const bf16_t* U, int k, const int32_t* map,
+                             const float* lr_dev, float adj_ratio, const float* wd_dev,
+                             float wd_host, hipStream_t st);
+
+}  // namespace dion

@@ -1,0 +1,623 @@
+// Memory-bound kernels of the Muon / NorMuon / Dion2 step for gfx950: everything around the
+// Newton-Schulz GEMMs.  All of them are single-pass over their big operands, use 16-byte
+// per-lane accesses where alignment allows, and reduce in a fixed order (no float atomics) so a
+// step is bit-reproducible run to run.
+#include "elementwise.h"
+
+namespace dion {
+
+static __device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Block-wide sum in a fixed order; result valid in every thread.  red: >= 16 floats of LDS.
+static __device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int i = 0; i < nw; ++i) s += red[i];
+  return s;
+}
+
+template <typename T>
+static __device__ __forceinline__ float load_as_bf16_f32(const T* p, int64_t i);
+template <>
+__device__ __forceinline__ float load_as_bf16_f32<bf16_t>(const bf16_t* p, int64_t i) {
+  return bf16_to_f32(p[i]);
+}
+template <>
+__device__ __forceinline__ float load_as_bf16_f32<float>(const float* p, int64_t i) {
+  return bf16_to_f32(f32_to_bf16(p[i]));
+}
+
+// ------------------------------------------------------------------------------------------
+// Frobenius pre-normalisation:  partial sums of squares of bf16(in), then 1/(||.||*s + eps).
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void sumsq_partial_kernel(const T* __restrict__ in, int64_t numel,
+                                                            int nblk, float* __restrict__ partial) {
+  __shared__ float red[16];
+  const int b = blockIdx.y;
+  const T* src = in + (int64_t)b * numel;
+  const int64_t per = (numel + nblk - 1) / nblk;
+  const int64_t lo = (int64_t)blockIdx.x * per;
+  int64_t hi = lo + per;
+  if (hi > numel) hi = numel;
+  float s = 0.f;
+  for (int64_t i = lo + threadIdx.x; i < hi; i += 256) {
+    const float v = load_as_bf16_f32<T>(src, i);
+    s += v * v;
+  }
+  s = block_sum(s, red);
+  if (threadIdx.x == 0) partial[(int64_t)b * nblk + blockIdx.x] = s;
+}
+
+__global__ __launch_bounds__(64) void norm_finalize_kernel(const float* __restrict__ partial, int nblk,
+                                                           float norm_scale, float eps,
+                                                           float* __restrict__ inv_norm) {
+  const int b = blockIdx.x;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < nblk; i += 64) s += partial[(int64_t)b * nblk + i];
+  s = wave_sum(s);
+  if (threadIdx.x == 0) inv_norm[b] = 1.0f / (sqrtf(s) * norm_scale + eps);
+}
+
+// in [B,R,C] -> same [B,Rp,Cp] (scaled, zero padded) and trans [B,Cp,Rp] = same^T, both bf16.
+// 64x64 tiles through LDS so both stores are row-contiguous.
+template <typename T>
+__global__ __launch_bounds__(256) void ns_prepare_kernel(const T* __restrict__ in, int R, int C,
+                                                         const float* __restrict__ inv_norm,
+                                                         bf16_t* __restrict__ same, int Rp, int Cp,
+                                                         bf16_t* __restrict__ trans) {
+  __shared__ bf16_t tile[64][66];
+  const int b = blockIdx.z;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const float sc = inv_norm[b];
+  const T* src = in + (int64_t)b * R * C;
+  bf16_t* ds = same + (int64_t)b * Rp * Cp;
+  bf16_t* dt = trans + (int64_t)b * Rp * Cp;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll 4
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i, c = c0 + tx;
+    bf16_t v = 0;
+    if (r < R && c < C) v = f32_to_bf16(load_as_bf16_f32<T>(src, (int64_t)r * C + c) * sc);
+    tile[i][tx] = v;
+    ds[(int64_t)r * Cp + c] = v;
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (int i = ty; i < 64; i += 4) {
+    // trans row (c0 + i), column (r0 + tx)
+    dt[(int64_t)(c0 + i) * Rp + r0 + tx] = tile[tx][i];
+  }
+}
+
+// Dense [B,R,C] <- padded [B,*,ld] (drops padding).
+__global__ __launch_bounds__(256) void unpad_kernel(const bf16_t* __restrict__ src, int64_t src_stride,
+                                                    int ld, bf16_t* __restrict__ dst, int R, int C) {
+  const int b = blockIdx.z;
+  const int r = blockIdx.y;
+  const bf16_t* s = src + (int64_t)b * src_stride + (int64_t)r * ld;
+  bf16_t* d = dst + ((int64_t)b * R + r) * C;
+  for (int c = blockIdx.x * 256 + threadIdx.x; c < C; c += gridDim.x * 256) d[c] = s[c];
+}
+
+hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t numel,
+                                float norm_scale, float eps, float* partial, int nblk,
+                                float* inv_norm, hipStream_t st) {
+  if (in_dtype == 0)
+    hipLaunchKernelGGL(sumsq_partial_kernel<bf16_t>, dim3(nblk, batch), dim3(256), 0, st,
+                       (const bf16_t*)in, numel, nblk, partial);
+  else
+    hipLaunchKernelGGL(sumsq_partial_kernel<float>, dim3(nblk, batch), dim3(256), 0, st,
+                       (const float*)in, numel, nblk, partial);
+  hipLaunchKernelGGL(norm_finalize_kernel, dim3(batch), dim3(64), 0, st, partial, nblk, norm_scale,
+                     eps, inv_norm);
+  return hipGetLastError();
+}
+
+hipError_t launch_ns_prepare(const void* in, int in_dtype, int batch, int R, int C,
+                             const float* inv_norm, bf16_t* same, int Rp, int Cp, bf16_t* trans,
+                             hipStream_t st) {
+  dim3 grid(Cp / 64, Rp / 64, batch);
+  if (in_dtype == 0)
+    hipLaunchKernelGGL(ns_prepare_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)in, R, C,
+                       inv_norm, same, Rp, Cp, trans);
+  else
+    hipLaunchKernelGGL(ns_prepare_kernel<float>, grid, dim3(256), 0, st, (const float*)in, R, C,
+                       inv_norm, same, Rp, Cp, trans);
+  return hipGetLastError();
+}
+
+hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* dst, int batch, int R,
+                        int C, hipStream_t st) {
+  int gx = (C + 255) / 256;
+  if (gx > 64) gx = 64;
+  hipLaunchKernelGGL(unpad_kernel, dim3(gx, R, batch), dim3(256), 0, st, src, src_stride, ld, dst, R,
+                     C);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// Muon pre: momentum + Nesterov + bf16 cast, list-of-parameters in, one arena out.
+// ------------------------------------------------------------------------------------------
+template <typename GT, bool VEC>
+__global__ __launch_bounds__(256) void muon_pre_kernel(PtrTab G, PtrTab M, bf16_t* __restrict__ U,
+                                                       int64_t numel, float mu, int nesterov) {
+  const int p = blockIdx.y;
+  const GT* __restrict__ g = (const GT*)G.p[p];
+  float* __restrict__ m = (float*)M.p[p];
+  bf16_t* __restrict__ u = U + (int64_t)p * numel;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  if (VEC) {
+    const int64_t nv = numel >> 3;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nv; i += stride) {
+      float gv[8];
+      if (sizeof(GT) == 2) {
+        const uint4 raw = ((const uint4*)g)[i];
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          gv[2 * e] = __uint_as_float(w[e] << 16);
+          gv[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+        }
+      } else {
+        const float4 a = ((const float4*)g)[2 * i], b = ((const float4*)g)[2 * i + 1];
+        gv[0] = a.x; gv[1] = a.y; gv[2] = a.z; gv[3] = a.w;
+        gv[4] = b.x; gv[5] = b.y; gv[6] = b.z; gv[7] = b.w;
+      }
+      float4 m0 = ((float4*)m)[2 * i], m1 = ((float4*)m)[2 * i + 1];
+      float mv[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
+      float uv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        mv[e] = __fadd_rn(__fmul_rn(mv[e], mu), gv[e]);
+        uv[e] = nesterov ? __fadd_rn(__fmul_rn(mv[e], mu), gv[e]) : mv[e];
+      }
+      ((float4*)m)[2 * i] = make_float4(mv[0], mv[1], mv[2], mv[3]);
+      ((float4*)m)[2 * i + 1] = make_float4(mv[4], mv[5], mv[6], mv[7]);
+      uint4 o;
+      o.x = pack_bf16x2(uv[0], uv[1]);
+      o.y = pack_bf16x2(uv[2], uv[3]);
+      o.z = pack_bf16x2(uv[4], uv[5]);
+      o.w = pack_bf16x2(uv[6], uv[7]);
+      ((uint4*)u)[i] = o;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
+      const float gv = sizeof(GT) == 2 ? bf16_to_f32(((const bf16_t*)g)[i]) : ((const float*)g)[i];
+      const float mv = __fadd_rn(__fmul_rn(m[i], mu), gv);
+      m[i] = mv;
+      u[i] = f32_to_bf16(nesterov ? __fadd_rn(__fmul_rn(mv, mu), gv) : mv);
+    }
+  }
+}
+
+static int ew_blocks(int64_t work_items) {
+  int64_t b = (work_items + 255) / 256;
+  if (b > 2048) b = 2048;
+  if (b < 1) b = 1;
+  return (int)b;
+}
+
+hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, bf16_t* U, int n,
+                           int64_t numel, float mu, int nesterov, bool vec, hipStream_t st) {
+  if (vec) {
+    dim3 grid(ew_blocks(numel >> 3), n);
+    if (g_dtype == 0)
+      hipLaunchKernelGGL((muon_pre_kernel<bf16_t, true>), grid, dim3(256), 0, st, G, M, U, numel, mu,
+                         nesterov);
+    else
+      hipLaunchKernelGGL((muon_pre_kernel<float, true>), grid, dim3(256), 0, st, G, M, U, numel, mu,
+                         nesterov);
+  } else {
+    dim3 grid(ew_blocks(numel), n);
+    if (g_dtype == 0)
+      hipLaunchKernelGGL((muon_pre_kernel<bf16_t, false>), grid, dim3(256), 0, st, G, M, U, numel, mu,
+                         nesterov);
+    else
+      hipLaunchKernelGGL((muon_pre_kernel<float, false>), grid, dim3(256), 0, st, G, M, U, numel, mu,
+                         nesterov);
+  }
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// Muon / NorMuon post: decoupled weight decay (plain or cautious) + scaled update.
+// ------------------------------------------------------------------------------------------
+static __device__ __forceinline__ float post_one(float x, float u, float a, float coeff, float b,
+                                                 int cautious) {
+  if (cautious) {
+    // mask = min(sign(x*u) + 1, 1): 0 only where x*u < 0  (dion/muon.py:333-340)
+    const float mask = (x * u < 0.f) ? 0.f : 1.f;
+    x = __fsub_rn(x, __fmul_rn(__fmul_rn(x, mask), coeff));
+  } else {
+    x = __fmul_rn(x, a);
+  }
+  return __fsub_rn(x, __fmul_rn(u, b));
+}
+
+template <typename UT, bool VEC>
+__global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __restrict__ U,
+                                                        int64_t numel, int cols,
+                                                        const float* __restrict__ row_scale,
+                                                        const float* __restrict__ lr_dev,
+                                                        float adj_ratio,
+                                                        const float* __restrict__ wd_dev,
+                                                        float wd_host, int cautious) {
+  const int p = blockIdx.y;
+  float* __restrict__ x = (float*)X.p[p];
+  const UT* __restrict__ u = U + (int64_t)p * numel;
+  const float lr = *lr_dev;
+  const float wd = wd_dev ? *wd_dev : wd_host;
+  const float coeff = __fmul_rn(lr, wd);
+  const float a = __fsub_rn(1.0f, coeff);
+  const float b = __fmul_rn(lr, adj_ratio);
+  const int64_t rows = numel / cols;
+  const float* rs = row_scale ? row_scale + (int64_t)p * rows : nullptr;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  if (VEC) {
+    const int64_t nv = numel >> 3;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nv; i += stride) {
+      float uv[8];
+      if (sizeof(UT) == 2) {
+        const uint4 raw = ((const uint4*)u)[i];
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          uv[2 * e] = __uint_as_float(w[e] << 16);
+          uv[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+        }
+      } else {
+        const float4 q0 = ((const float4*)u)[2 * i], q1 = ((const float4*)u)[2 * i + 1];
+        uv[0] = q0.x; uv[1] = q0.y; uv[2] = q0.z; uv[3] = q0.w;
+        uv[4] = q1.x; uv[5] = q1.y; uv[6] = q1.z; uv[7] = q1.w;
+      }
+      if (rs) {  // cols % 8 == 0 on this path, so the 8 elements share a row
+        const float s = rs[(i << 3) / cols];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) uv[e] = __fmul_rn(uv[e], s);
+      }
+      float4 x0 = ((float4*)x)[2 * i], x1 = ((float4*)x)[2 * i + 1];
+      float xv[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xv[e] = post_one(xv[e], uv[e], a, coeff, b, cautious);
+      ((float4*)x)[2 * i] = make_float4(xv[0], xv[1], xv[2], xv[3]);
+      ((float4*)x)[2 * i + 1] = make_float4(xv[4], xv[5], xv[6], xv[7]);
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
+      float uv = sizeof(UT) == 2 ? bf16_to_f32(((const bf16_t*)u)[i]) : ((const float*)u)[i];
+      if (rs) uv = __fmul_rn(uv, rs[i / cols]);
+      x[i] = post_one(x[i], uv, a, coeff, b, cautious);
+    }
+  }
+}
+
+hipError_t launch_muon_post(const PtrTab& X, const void* U, int u_dtype, int n, int64_t numel,
+                            int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
+                            const float* wd_dev, float wd_host, int cautious, bool vec,
+                            hipStream_t st) {
+  dim3 grid(ew_blocks(vec ? (numel >> 3) : numel), n);
+#define POST_LAUNCH(UT, V)                                                                        \
+  hipLaunchKernelGGL((muon_post_kernel<UT, V>), grid, dim3(256), 0, st, X, (const UT*)U, numel,   \
+                     cols, row_scale, lr_dev, adj_ratio, wd_dev, wd_host, cautious)
+  if (u_dtype == 0) {
+    if (vec) POST_LAUNCH(bf16_t, true); else POST_LAUNCH(bf16_t, false);
+  } else {
+    if (vec) POST_LAUNCH(float, true); else POST_LAUNCH(float, false);
+  }
+#undef POST_LAUNCH
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// NorMuon: per-row second moment EMA and the Frobenius-preserving row scales.
+// ------------------------------------------------------------------------------------------
+// Pass 1: one wavefront per row.  V <- lerp(V, mean(u^2), w);  tmp[row] = sum(u^2).
+__global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restrict__ U, PtrTab V,
+                                                           int mats_per_ptr, int rows, int cols,
+                                                           float w, float* __restrict__ rowsq) {
+  const int mat = blockIdx.y;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const bf16_t* u = U + ((int64_t)mat * rows + row) * cols;
+  float s = 0.f;
+  if ((cols & 7) == 0 && (((uintptr_t)u) & 15) == 0) {
+    for (int c = lane * 8; c < cols; c += 512) {
+      const uint4 raw = *(const uint4*)(u + c);
+      const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __uint_as_float(wv[e] << 16), hi = __uint_as_float(wv[e] & 0xffff0000u);
+        s += lo * lo;
+        s += hi * hi;
+      }
+    }
+  } else {
+    for (int c = lane; c < cols; c += 64) {
+      const float v = bf16_to_f32(u[c]);
+      s += v * v;
+    }
+  }
+  s = wave_sum(s);
+  if (lane == 0) {
+    float* v = (float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows + row;
+    const float mean = s / (float)cols;
+    const float vo = *v;
+    *v = vo + w * (mean - vo);  // torch.lerp for weight < 0.5
+    rowsq[(int64_t)mat * rows + row] = s;
+  }
+}
+
+// Pass 2: one block per matrix.  scale[row] = (1/d) * sqrt(S1) / max(sqrt(S2), 1e-8) with
+// d = sqrt(V)+1e-8, S1 = sum rowsq, S2 = sum rowsq/d^2.  In place over rowsq.
+__global__ __launch_bounds__(1024) void normuon_scale_kernel(PtrTab V, int mats_per_ptr, int rows,
+                                                             float* __restrict__ scale) {
+  __shared__ float red[16];
+  const int mat = blockIdx.x;
+  const float* v = (const float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows;
+  float* sc = scale + (int64_t)mat * rows;
+  float s1 = 0.f, s2 = 0.f;
+  for (int r = threadIdx.x; r < rows; r += 1024) {
+    const float q = sc[r];
+    const float inv = 1.0f / (sqrtf(v[r]) + 1e-8f);
+    s1 += q;
+    s2 += q * inv * inv;
+  }
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  const float ratio = sqrtf(s1) / fmaxf(sqrtf(s2), 1e-8f);
+  __syncthreads();
+  for (int r = threadIdx.x; r < rows; r += 1024) {
+    const float inv = 1.0f / (sqrtf(v[r]) + 1e-8f);
+    sc[r] = inv * ratio;
+  }
+}
+
+hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int n_mat, int mat0,
+                                int mats_per_ptr, int rows, int cols, float w, float* row_scale,
+                                hipStream_t st) {
+  // U / row_scale are offset to matrix mat0 by the caller; V is the table chunk covering them.
+  (void)mat0;
+  hipLaunchKernelGGL(normuon_rows_kernel, dim3((rows + 3) / 4, n_mat), dim3(256), 0, st, U, V,
+                     mats_per_ptr, rows, cols, w, row_scale);
+  hipLaunchKernelGGL(normuon_scale_kernel, dim3(n_mat), dim3(1024), 0, st, V, mats_per_ptr, rows,
+                     row_scale);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// Dion2: accumulate + slice L1 norms, top-k, gather with error-feedback decay, fused post.
+// ------------------------------------------------------------------------------------------
+template <typename GT>
+static __device__ __forceinline__ float g_load(const GT* g, int64_t i) {
+  return sizeof(GT) == 2 ? bf16_to_f32(((const bf16_t*)g)[i]) : ((const float*)g)[i];
+}
+
+// select rows: one wavefront per row, norms[mat][row] = sum_j |M+G|.
+template <typename GT>
+__global__ __launch_bounds__(256) void dion2_acc_rows_kernel(PtrTab G, PtrTab M, int mats_per_ptr,
+                                                             int rows, int cols,
+                                                             float* __restrict__ norms) {
+  const int mat = blockIdx.y;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t base = ((int64_t)(mat % mats_per_ptr) * rows + row) * cols;
+  const GT* g = (const GT*)G.p[mat / mats_per_ptr] + base;
+  float* m = (float*)M.p[mat / mats_per_ptr] + base;
+  float s = 0.f;
+  for (int c = lane; c < cols; c += 64) {
+    const float v = __fadd_rn(m[c], g_load<GT>(g, c));
+    m[c] = v;
+    s += fabsf(v);
+  }
+  s = wave_sum(s);
+  if (lane == 0) norms[(int64_t)mat * rows + row] = s;
+}
+
+// select columns: each block owns 64 columns of one matrix and walks all rows (4 rows at a time).
+template <typename GT>
+__global__ __launch_bounds__(256) void dion2_acc_cols_kernel(PtrTab G, PtrTab M, int mats_per_ptr,
+                                                             int rows, int cols,
+                                                             float* __restrict__ norms) {
+  __shared__ float red[4][64];
+  const int mat = blockIdx.y;
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int ry = threadIdx.x >> 6;
+  const int64_t base = (int64_t)(mat % mats_per_ptr) * rows * cols;
+  const GT* g = (const GT*)G.p[mat / mats_per_ptr] + base;
+  float* m = (float*)M.p[mat / mats_per_ptr] + base;
+  float s = 0.f;
+  if (c < cols) {
+    for (int r = ry; r < rows; r += 4) {
+      const int64_t i = (int64_t)r * cols + c;
+      const float v = __fadd_rn(m[i], g_load<GT>(g, i));
+      m[i] = v;
+      s += fabsf(v);
+    }
+  }
+  red[ry][threadIdx.x & 63] = s;
+  __syncthreads();
+  if (ry == 0 && c < cols)
+    norms[(int64_t)mat * cols + c] = (red[0][threadIdx.x] + red[1][threadIdx.x]) +
+                                     (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
+hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int n_mat,
+                                   int mats_per_ptr, int rows, int cols, int select_rows,
+                                   float* norms, hipStream_t st) {
+  if (select_rows) {
+    dim3 grid((rows + 3) / 4, n_mat);
+    if (g_dtype == 0)
+      hipLaunchKernelGGL(dion2_acc_rows_kernel<bf16_t>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
+                         rows, cols, norms);
+    else
+      hipLaunchKernelGGL(dion2_acc_rows_kernel<float>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
+                         rows, cols, norms);
+  } else {
+    dim3 grid((cols + 63) / 64, n_mat);
+    if (g_dtype == 0)
+      hipLaunchKernelGGL(dion2_acc_cols_kernel<bf16_t>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
+                         rows, cols, norms);
+    else
+      hipLaunchKernelGGL(dion2_acc_cols_kernel<float>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
+                         rows, cols, norms);
+  }
+  return hipGetLastError();
+}
+
+// Exact top-k by rank counting (rank = number of entries that beat this one; ties go to the lower
+// index), one block per matrix.  Selected indices come out ascending, which keeps the gather and
+// the scatter walking memory forwards.  NaNs order as +inf like torch.topk.
+__global__ __launch_bounds__(1024) void dion2_topk_kernel(const float* __restrict__ norms, int dim,
+                                                          int k, int32_t* __restrict__ idx,
+                                                          int32_t* __restrict__ map) {
+  extern __shared__ float vals[];  // dim floats + 17 ints
+  int* wave_tot = (int*)(vals + dim);
+  const int mat = blockIdx.x;
+  const float* v = norms + (int64_t)mat * dim;
+  for (int i = threadIdx.x; i < dim; i += 1024) {
+    float x = v[i];
+    if (x != x) x = INFINITY;
+    vals[i] = x;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  int running = 0;  // selected entries before the current chunk (same in every thread)
+  for (int base = 0; base < dim; base += 1024) {
+    const int i = base + threadIdx.x;
+    int sel = 0;
+    if (i < dim) {
+      const float x = vals[i];
+      int rank = 0;
+      for (int j = 0; j < dim; ++j) {
+        const float y = vals[j];
+        rank += (y > x) || (y == x && j < i);
+      }
+      sel = rank < k;
+    }
+    // block-wide exclusive scan of sel
+    const unsigned long long ball = __ballot(sel);
+    const int in_wave = __popcll(ball & ((1ull << lane) - 1ull));
+    __syncthreads();
+    if (lane == 0) wave_tot[w] = __popcll(ball);
+    __syncthreads();
+    int before = 0, total = 0;
+    for (int q = 0; q < 16; ++q) {
+      const int tq = wave_tot[q];
+      if (q < w) before += tq;
+      total += tq;
+    }
+    if (i < dim) {
+      const int pos = running + before + in_wave;
+      if (sel) idx[(int64_t)mat * k + pos] = i;
+      map[(int64_t)mat * dim + i] = sel ? pos : -1;
+    }
+    running += total;
+  }
+}
+
+hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
+                             int32_t* map, hipStream_t st) {
+  const size_t shmem = (size_t)dim * sizeof(float) + 17 * sizeof(int);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)dion2_topk_kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(dion2_topk_kernel, dim3(n_mat), dim3(1024), shmem, st, norms, dim, k, idx, map);
+  return hipGetLastError();
+}
+
+// U_sel = bf16(M[sel]); M[sel] *= ef_decay.
+__global__ __launch_bounds__(256) void dion2_gather_kernel(PtrTab M, int mats_per_ptr, int rows,
+                                                           int cols, int select_rows,
+                                                           const int32_t* __restrict__ idx, int k,
+                                                           float ef_decay, bf16_t* __restrict__ U) {
+  const int mat = blockIdx.y;
+  float* m = (float*)M.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
+  const int32_t* id = idx + (int64_t)mat * k;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  if (select_rows) {
+    bf16_t* u = U + (int64_t)mat * k * cols;
+    const int64_t n = (int64_t)k * cols;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+      const int j = (int)(i / cols), c = (int)(i - (int64_t)j * cols);
+      const int64_t src = (int64_t)id[j] * cols + c;
+      const float v = m[src];
+      u[i] = f32_to_bf16(v);
+      m[src] = __fmul_rn(v, ef_decay);
+    }
+  } else {
+    bf16_t* u = U + (int64_t)mat * rows * k;
+    const int64_t n = (int64_t)rows * k;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+      const int r = (int)(i / k), j = (int)(i - (int64_t)r * k);
+      const int64_t src = (int64_t)r * cols + id[j];
+      const float v = m[src];
+      u[i] = f32_to_bf16(v);
+      m[src] = __fmul_rn(v, ef_decay);
+    }
+  }
+}
+
+hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int rows, int cols,
+                               int select_rows, const int32_t* idx, int k, float ef_decay, bf16_t* U,
+                               hipStream_t st) {
+  const int64_t n = select_rows ? (int64_t)k * cols : (int64_t)rows * k;
+  hipLaunchKernelGGL(dion2_gather_kernel, dim3(ew_blocks(n), n_mat), dim3(256), 0, st, M,
+                     mats_per_ptr, rows, cols, select_rows, idx, k, ef_decay, U);
+  return hipGetLastError();
+}
+
+// x = a*x - b*u[map] on selected slices, x = a*x elsewhere; one rounding of the sum.
+__global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_ptr, int rows,
+                                                         int cols, int select_rows,
+                                                         const bf16_t* __restrict__ U, int k,
+                                                         const int32_t* __restrict__ map,
+                                                         const float* __restrict__ lr_dev,
+                                                         float adj_ratio,
+                                                         const float* __restrict__ wd_dev,
+                                                         float wd_host) {
+  const int mat = blockIdx.y;
+  float* x = (float*)X.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
+  const float lr = *lr_dev;
+  const float wd = wd_dev ? *wd_dev : wd_host;
+  const float a = __fsub_rn(1.0f, __fmul_rn(lr, wd));
+  const float b = __fmul_rn(lr, adj_ratio);
+  const int dim = select_rows ? rows : cols;
+  const int32_t* mp = map + (int64_t)mat * dim;
+  const bf16_t* u = U + (int64_t)mat * (select_rows ? (int64_t)k * cols : (int64_t)rows * k);
+  const int64_t n = (int64_t)rows * cols;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const int r = (int)(i / cols), c = (int)(i - (int64_t)r * cols);
+    const int j = mp[select_rows ? r : c];
+    float uv = 0.f;
+    if (j >= 0) uv = bf16_to_f32(select_rows ? u[(int64_t)j * cols + c] : u[(int64_t)r * k + j]);
+    x[i] = fmaf(a, x[i], -(b * uv));
+  }
+}
+
+hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
+                             int select_rows, const bf16_t* U, int k, const int32_t* map,
+                             const float* lr_dev, float adj_ratio, const float* wd_dev,
+                             float wd_host, hipStream_t st) {
+  hipLaunchKernelGGL(dion2_post_kernel, dim3(ew_blocks((int64_t)rows * cols), n_mat), dim3(256), 0,
+                     st, X, mats_per_ptr, rows, cols, select_rows, U, k, map, lr_dev, adj_ratio,
+                     wd_dev, wd_host);
+  return hipGetLastError();
+}
+
+}  // namespace dion

@@ -1,0 +1,333 @@
+// Batched bf16 "NT" GEMM for gfx950 (CDNA4):  C = alpha * P * Q^T + beta * D, fp32 accumulate.
+//
+// Every GEMM of the Newton-Schulz / Polar-Express iteration is expressed in this one form, with
+// both operands contiguous along the reduction dimension, by carrying X and X^T side by side:
+//   A  = X X^T                     P = Q = X            (tri: upper tiles + mirrored store)
+//   B  = c A A + b A               P = Q = A (A = A^T)  (tri, D = A)
+//   X' = a X + B X                 P = B, Q = X^T, D = X, stores X' and (X')^T
+// This replaces the reference's ns_line_1 / ns_line_2 / ns_line_3
+// (dion/newton_schulz_triton.py:88-157, :206-287, :384-447) and the baddbmm of
+// dion/newton_schulz_triton.py:557-563.
+//
+// Kernel structure: one workgroup per BM x BN output tile, WM x WN wavefronts (64 lanes) each
+// owning a (BM/WM) x (BN/WN) sub-tile as 32x32 MFMA accumulators
+// (v_mfma_f32_32x32x16_bf16).  Operand tiles stream global -> LDS with the direct-to-LDS loads
+// (global_load_lds_dwordx4, no VGPR staging) into an NSTAGE ring; a 16-byte-chunk XOR swizzle
+// keeps both the DMA writes and the ds_read_b128 fragment reads bank-conflict free.
+#include "common.h"
+
+namespace dion {
+
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int NSTAGE_>
+struct TileCfg {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, NSTAGE = NSTAGE_;
+  static constexpr int NT = WM * WN * 64;
+  static constexpr int CPR = BK / 8;            // 16-byte chunks per tile row
+  static constexpr int ROWS_PER_LOAD = NT / CPR; // tile rows covered by one load instruction
+  static constexpr int P_BYTES = BM * BK * 2;
+  static constexpr int Q_BYTES = BN * BK * 2;
+  static constexpr int STAGE_BYTES = P_BYTES + Q_BYTES;
+  static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
+  static constexpr int P_LOADS = BM / ROWS_PER_LOAD;
+  static constexpr int Q_LOADS = BN / ROWS_PER_LOAD;
+  static constexpr int LOADS_PER_STAGE = P_LOADS + Q_LOADS;
+  static constexpr int WTM = BM / WM, WTN = BN / WN;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int KK = BK / 16;
+  static constexpr int SWZ_DIV = 8 / CPR;       // rows sharing one swizzle value
+  static_assert(BM % ROWS_PER_LOAD == 0 && BN % ROWS_PER_LOAD == 0, "tile/threads mismatch");
+  static_assert(CPR == 8 || CPR == 4, "BK must be 64 or 32");
+};
+
+// s_waitcnt with only vmcnt constrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8]
+// | vmcnt_hi[15:14]).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
+}
+
+__device__ __forceinline__ void tri_tile(int t, int T, int& ti, int& tj) {
+  // Row-major enumeration of the upper triangle of a T x T tile grid.
+  float f = (float)(2 * T + 1);
+  int i = (int)((f - sqrtf(f * f - 8.0f * (float)t)) * 0.5f);
+  if (i < 0) i = 0;
+  if (i > T - 1) i = T - 1;
+  while (i + 1 < T && (i + 1) * T - ((i + 1) * i) / 2 <= t) ++i;
+  while (i > 0 && i * T - (i * (i - 1)) / 2 > t) --i;
+  ti = i;
+  tj = i + (t - (i * T - (i * (i - 1)) / 2));
+}
+
+// Workgroup barrier preceded by the counter waits the software pipeline needs: every LDS read
+// this wave issued has returned (the ring slot they read is about to be refilled) and all but the
+// newest VM_LEFT direct-to-LDS loads of this wave have landed.  The "memory" clobber keeps the
+// compiler from moving LDS accesses across it.
+template <int VM_LEFT>
+__device__ __forceinline__ void pipeline_barrier() {
+  static_assert(VM_LEFT >= 0 && VM_LEFT < 64, "vmcnt range");
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("" ::: "memory");
+  // vmcnt = VM_LEFT, lgkmcnt = 0, expcnt unconstrained (gfx9 s_waitcnt encoding).
+  __builtin_amdgcn_s_waitcnt((VM_LEFT & 0xF) | ((VM_LEFT >> 4) << 14) | 0x0070);
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT>
+__global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, KK = Cfg::KK, NSTAGE = Cfg::NSTAGE;
+  constexpr int NM = TM * TN;  // MFMAs per 16-wide k slice
+  constexpr int NR = TM + TN;  // fragment reads per slice
+  constexpr int LPS = Cfg::LOADS_PER_STAGE;
+  static_assert(KK % 2 == 0, "fragment double buffer needs an even slice count per stage");
+  constexpr int RPM = (NR + NM - 1) / NM;    // fragment reads slotted behind each MFMA
+  constexpr int LPM = (LPS + NM - 1) / NM;   // refill loads slotted behind each MFMA
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+
+  // ---- workgroup -> (batch, tile) map.  Hardware deals workgroups round-robin over the 8 XCDs;
+  // give each XCD (own L2) one contiguous run of the tile list so neighbours share operands.
+  const int tilesM = p.M / BM, tilesN = p.N / BN;
+  const int tiles_per_mat = p.tri ? (tilesM * (tilesM + 1)) / 2 : tilesM * tilesN;
+  const int total = gridDim.x;
+  int lt;
+  {
+    const int pid = blockIdx.x;
+    const int xcd = pid & 7, loc = pid >> 3;
+    const int q = total >> 3, r = total & 7;
+    lt = xcd * q + (xcd < r ? xcd : r) + loc;
+  }
+  const int b = lt / tiles_per_mat;
+  const int t = lt - b * tiles_per_mat;
+  int ti, tj;
+  if (p.tri) {
+    tri_tile(t, tilesM, ti, tj);
+  } else {
+    constexpr int GM = 4;
+    const int per_group = GM * tilesN;
+    const int g = t / per_group;
+    const int first = g * GM;
+    const int gsz = (tilesM - first) < GM ? (tilesM - first) : GM;
+    const int tg = t - g * per_group;
+    ti = first + tg % gsz;
+    tj = tg / gsz;
+  }
+
+  // ---- global -> LDS addressing.  Chunk q = j*NT + tid of a tile lands at LDS byte q*16; it holds
+  // logical 16-byte chunk (q % CPR) ^ swz(row) of tile row q / CPR.
+  const int ld_row = tid / Cfg::CPR;
+  const int ld_phys = tid % Cfg::CPR;
+  const int ld_chunk = ld_phys ^ ((ld_row / Cfg::SWZ_DIV) % Cfg::CPR);
+  const char* gP = (const char*)(p.P + (int64_t)b * p.strideP + (int64_t)(ti * BM) * p.ldp);
+  const char* gQ = (const char*)(p.Q + (int64_t)b * p.strideQ + (int64_t)(tj * BN) * p.ldq);
+  const uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
+  const uint32_t offQ = (uint32_t)(ld_row * p.ldq + ld_chunk * 8) * 2u;
+  const uint32_t stepP = (uint32_t)(Cfg::ROWS_PER_LOAD * p.ldp) * 2u;
+  const uint32_t stepQ = (uint32_t)(Cfg::ROWS_PER_LOAD * p.ldq) * 2u;
+  const int KT = p.K / BK;
+
+  // One direct-to-LDS load (index j of the LPS that make up a stage) of k-slab kt into ring
+  // slot buf.  kt past the end re-fetches the last slab (never read): the refill count per stage
+  // stays fixed, which is what the vmcnt bookkeeping in pipeline_barrier relies on.
+  auto issue_load = [&](int kt, int buf, int j) {
+    const int k = kt < KT ? kt : KT - 1;
+    char* l = lds + buf * Cfg::STAGE_BYTES + wave * (64 * 16);
+    if (j < Cfg::P_LOADS) {
+      const char* src = gP + (int64_t)k * (BK * 2) + (offP + j * stepP);
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
+    } else {
+      const int jq = j - Cfg::P_LOADS;
+      const char* src = gQ + (int64_t)k * (BK * 2) + (offQ + jq * stepQ);
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + Cfg::P_BYTES + jq * (Cfg::NT * 16)),
+                                       16, 0, 0);
+    }
+  };
+
+  // ---- LDS -> register fragment addressing (per lane, per 16-wide k slice).
+  const int frow = lane & 31;
+  const int fhalf = lane >> 5;
+  const int fswz = (frow / Cfg::SWZ_DIV) % Cfg::CPR;
+  uint32_t aoff[KK], boff[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    const int chunk = ((kk * 2 + fhalf) ^ fswz) * 16;
+    aoff[kk] = (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + chunk);
+    boff[kk] = (uint32_t)(Cfg::P_BYTES + (wn * Cfg::WTN + frow) * (BK * 2) + chunk);
+  }
+
+  bf16x8 fa[2][TM], fb[2][TN];
+  // Fragment read r (0..NR-1) of slice kk of ring slot buf into fragment set f.
+  auto read_frag = [&](int buf, int kk, int f, int r) {
+    const char* st = lds + buf * Cfg::STAGE_BYTES;
+    if (r < TM) fa[f][r] = *(const bf16x8*)(st + aoff[kk] + r * (32 * BK * 2));
+    else fb[f][r - TM] = *(const bf16x8*)(st + boff[kk] + (r - TM) * (32 * BK * 2));
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  // ---- prologue: fill NSTAGE-1 ring slots, wait for slab 0, read its first fragments, start the
+  // last free slot.
+#pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s)
+#pragma unroll
+    for (int j = 0; j < LPS; ++j) issue_load(s, s, j);
+  pipeline_barrier<(NSTAGE - 2) * LPS>();
+#pragma unroll
+  for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
+#pragma unroll
+  for (int j = 0; j < LPS; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- main loop.  Slices run back to back across slab boundaries: while the MFMAs of one slice
+  // issue, the fragment reads of the next slice (and, on the last slice of a slab, the refill of
+  // the slot that slab occupied) are slotted one behind each MFMA.  sched_barrier pins that order.
+  // KT is a multiple of NSTAGE (launcher checks) so ring slots are compile-time constants.
+  for (int kt0 = 0; kt0 < KT; kt0 += NSTAGE) {
+#pragma unroll
+    for (int s = 0; s < NSTAGE; ++s) {
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        const int cur = kk & 1, nxt = cur ^ 1;
+        const bool last = (kk == KK - 1);
+        if (last) pipeline_barrier<(NSTAGE - 2) * LPS>();  // slab kt+1 landed, slab kt fully read
+#pragma unroll
+        for (int q = 0; q < NM; ++q) {
+          acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              fa[cur][q / TN], fb[cur][q % TN], acc[q / TN][q % TN], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int r = q * RPM; r < (q + 1) * RPM && r < NR; ++r) {
+            if (last) read_frag((s + 1) % NSTAGE, 0, nxt, r);
+            else read_frag(s, kk + 1, nxt, r);
+          }
+          if (last) {
+#pragma unroll
+            for (int j = q * LPM; j < (q + 1) * LPM && j < LPS; ++j)
+              issue_load(kt0 + s + NSTAGE, s, j);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  }
+  wait_vmcnt<0>();  // drain the redundant tail refills before the wave can exit
+
+  // ---- epilogue.  Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4,
+  // column l%32 of its 32x32 tile.  Whole tiles are stored: destinations are padded to the tile.
+  const float alpha = p.alpha, beta = p.beta;
+  const int row_base = ti * BM + wm * Cfg::WTM + 4 * fhalf;
+  const int col_base = tj * BN + wn * Cfg::WTN + frow;
+  const bool mirror = HAS_CT && !(p.tri && ti == tj);  // a diagonal tile is its own mirror
+  const bf16_t* Dp = HAS_D ? p.D + (int64_t)b * p.strideD + (int64_t)row_base * p.ldd + col_base : nullptr;
+  bf16_t* Cp = HAS_C ? p.C + (int64_t)b * p.strideC + (int64_t)row_base * p.ldc + col_base : nullptr;
+  bf16_t* Ctp = HAS_CT ? p.Ct + (int64_t)b * p.strideCt + (int64_t)col_base * p.ldct + row_base : nullptr;
+  const int ldd = p.ldd, ldc = p.ldc, ldct = p.ldct;
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      float v[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) v[r] = alpha * acc[i][j][r];
+      if (HAS_D) {
+        bf16_t d[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          d[r] = Dp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldd + j * 32];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] += beta * bf16_to_f32(d[r]);
+      }
+      if (HAS_C) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          Cp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldc + j * 32] = f32_to_bf16(v[r]);
+      }
+      if (HAS_CT) {
+        if (mirror) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            uint2 pk;
+            pk.x = pack_bf16x2(v[g * 4 + 0], v[g * 4 + 1]);
+            pk.y = pack_bf16x2(v[g * 4 + 2], v[g * 4 + 3]);
+            *(uint2*)(Ctp + (int64_t)(j * 32) * ldct + i * 32 + g * 8) = pk;
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+typedef TileCfg<256, 256, 64, 2, 2, 2> Cfg256;
+typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg128;
+typedef TileCfg<256, 256, 32, 2, 2, 4> Cfg256k32;
+
+template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT>
+static hipError_t launch_epi(const GemmParams& p, hipStream_t stream) {
+  static bool attr_set = false;
+  auto kern = gemm_nt_kernel<Cfg, HAS_D, HAS_C, HAS_CT>;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       Cfg::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  const int tilesM = p.M / Cfg::BM, tilesN = p.N / Cfg::BN;
+  const int64_t per_mat = p.tri ? (int64_t)tilesM * (tilesM + 1) / 2 : (int64_t)tilesM * tilesN;
+  const int64_t total = per_mat * p.batch;
+  if (total <= 0) return hipSuccess;
+  if (total > 0x7fffffff) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  return hipGetLastError();
+}
+
+template <class Cfg>
+static hipError_t launch_cfg(const GemmParams& p, hipStream_t stream) {
+  if (p.M % Cfg::BM || p.N % Cfg::BN || p.K % (Cfg::BK * Cfg::NSTAGE)) return hipErrorInvalidValue;
+  const bool d = p.D != nullptr, c = p.C != nullptr, ct = p.Ct != nullptr;
+  if (!d && c && ct) return launch_epi<Cfg, false, true, true>(p, stream);   // A = X X^T
+  if (d && c && ct) return launch_epi<Cfg, true, true, true>(p, stream);     // B, X' (both layouts)
+  if (d && c && !ct) return launch_epi<Cfg, true, true, false>(p, stream);   // last X'
+  if (d && !c && ct) return launch_epi<Cfg, true, false, true>(p, stream);   // last (X')^T
+  if (!d && c && !ct) return launch_epi<Cfg, false, true, false>(p, stream); // plain product
+  return hipErrorInvalidValue;
+}
+
+int gemm_pad_granule(int m, int n, int batch) {
+  // 256-wide tiles need enough of them to fill 256 CUs; small problems use 128-wide tiles.
+  const int64_t m256 = (m + 255) / 256;
+  const int64_t syrk_tiles = m256 * (m256 + 1) / 2 * batch;
+  (void)n;
+  return syrk_tiles >= 256 ? 256 : 128;
+}
+
+hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) {
+  if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.batch <= 0) return hipSuccess;
+  if (variant < 0) variant = (p.M % 256 == 0 && p.N % 256 == 0) ? 0 : 1;
+  if (p.tri && (p.M != p.N)) return hipErrorInvalidValue;
+  switch (variant) {
+    case 0: return launch_cfg<Cfg256>(p, stream);
+    case 1: return launch_cfg<Cfg128>(p, stream);
+    case 2: return launch_cfg<Cfg256k32>(p, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace dion

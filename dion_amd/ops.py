@@ -1,0 +1,331 @@
+"""Tensor-level wrappers over the C ABI of libdion_hip.so.
+
+Each function takes torch tensors that live on the GPU, validates shapes/dtypes on the host,
+hands raw device pointers and the current stream to the library, and returns torch tensors.
+torch is used for device memory and streams only; all arithmetic happens in the HIP kernels.
+There is no CPU implementation behind these functions: CPU tensors raise.
+"""
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from ._lib import DION_BF16, DION_F32, DION_NS_GRAM, check, ptr_table
+
+
+def _stream_handle(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_gpu(t: Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{name} must be a GPU tensor (got device {t.device}); the dion_amd kernels have no CPU path"
+        )
+
+
+def _dtype_code(t: Tensor, name: str) -> int:
+    if t.dtype == torch.bfloat16:
+        return DION_BF16
+    if t.dtype == torch.float32:
+        return DION_F32
+    raise TypeError(f"{name}: dtype {t.dtype} not supported (bfloat16 or float32)")
+
+
+_workspaces = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> Tensor:
+    """Grow-only scratch buffer per (device, stream); NS calls on one stream reuse it in order."""
+    key = (device.index, _stream_handle(device))
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = None
+        _workspaces.pop(key, None)
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def release_workspaces() -> None:
+    """Drop the cached Newton-Schulz workspaces (they are re-created on demand)."""
+    _workspaces.clear()
+
+
+def _pad128(t: Tensor) -> Tensor:
+    """Zero-pad the last two dims of a 3-D bf16 tensor to multiples of 128 (copy only if needed)."""
+    r, c = t.shape[-2], t.shape[-1]
+    rp, cp = -(-r // 128) * 128, -(-c // 128) * 128
+    if rp == r and cp == c:
+        return t.contiguous()
+    out = torch.zeros(t.shape[0], rp, cp, dtype=t.dtype, device=t.device)
+    out[:, :r, :c] = t
+    return out
+
+
+def _as_batch(t: Tensor, name: str) -> Tuple[Tensor, bool]:
+    if t.ndim == 2:
+        return t.unsqueeze(0), True
+    if t.ndim == 3:
+        return t, False
+    raise ValueError(f"{name} must be a 2D or 3D tensor, got shape {tuple(t.shape)}")
+
+
+def _check_bf16(t: Tensor, name: str) -> None:
+    _require_gpu(t, name)
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name}: the gfx950 kernels take bfloat16 operands, got {t.dtype}")
+
+
+def ns_line_1(A: Tensor, *, out: Optional[Tensor] = None) -> Tensor:
+    """``A @ A.mT`` computing only the upper-triangular tiles and mirroring them.
+
+    Mirrors ``ns_line_1`` of the reference (dion/newton_schulz_triton.py:160-203): 2D or 3D
+    input, optional ``out``; ValueError for other ranks.
+    """
+    _check_bf16(A, "A")
+    A3, squeeze = _as_batch(A, "Input tensor")
+    b, m, k = A3.shape
+    Ap = _pad128(A3)
+    mp, kp = Ap.shape[-2:]
+    res = torch.empty(b, mp, mp, dtype=torch.bfloat16, device=A.device)
+    lib = _lib.load()
+    check(lib.dion_ns_line_1(Ap.data_ptr(), res.data_ptr(), b, mp, kp, _stream_handle(A.device)),
+          "ns_line_1")
+    res = res[:, :m, :m]
+    if squeeze:
+        res = res[0]
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res.contiguous()
+
+
+def ns_line_2(A: Tensor, alpha: float, beta: float, *, out: Optional[Tensor] = None) -> Tensor:
+    """``alpha * A @ A.mT + beta * A`` for symmetric ``A`` (upper tiles + mirror).
+
+    Mirrors ``ns_line_2`` of the reference (dion/newton_schulz_triton.py:290-333).
+    """
+    _check_bf16(A, "A")
+    A3, squeeze = _as_batch(A, "Input tensor")
+    b, m, m2 = A3.shape
+    if m != m2:
+        raise ValueError(f"Input tensor must be square, got shape {tuple(A.shape)}")
+    Ap = _pad128(A3)
+    mp = Ap.shape[-1]
+    res = torch.empty(b, mp, mp, dtype=torch.bfloat16, device=A.device)
+    lib = _lib.load()
+    check(lib.dion_ns_line_2(Ap.data_ptr(), res.data_ptr(), b, mp, float(alpha), float(beta),
+                             _stream_handle(A.device)), "ns_line_2")
+    res = res[:, :m, :m]
+    if squeeze:
+        res = res[0]
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res.contiguous()
+
+
+def ns_line_3(B: Tensor, X: Tensor, a: float, *, out: Optional[Tensor] = None) -> Tensor:
+    """``a * X + B @ X`` for symmetric ``B``.
+
+    Mirrors ``ns_line_3`` of the reference (dion/newton_schulz_triton.py:450-491).  The kernel
+    wants X with the reduction dimension contiguous, so X^T is materialised here; the whole-NS
+    driver keeps both layouts alive instead.
+    """
+    _check_bf16(B, "B")
+    _check_bf16(X, "X")
+    B3, squeeze = _as_batch(B, "B")
+    X3, _ = _as_batch(X, "X")
+    if B3.shape[0] != X3.shape[0] or B3.shape[-1] != B3.shape[-2] or B3.shape[-1] != X3.shape[-2]:
+        raise ValueError(f"shape mismatch: B {tuple(B.shape)} vs X {tuple(X.shape)}")
+    b, m, n = X3.shape
+    Bp = _pad128(B3)
+    Xp = _pad128(X3)
+    Xtp = Xp.transpose(-2, -1).contiguous()
+    mp, np_ = Xp.shape[-2:]
+    res = torch.empty(b, mp, np_, dtype=torch.bfloat16, device=X.device)
+    lib = _lib.load()
+    check(lib.dion_ns_line_3(Bp.data_ptr(), Xp.data_ptr(), Xtp.data_ptr(), res.data_ptr(), None, b, mp,
+                             np_, float(a), _stream_handle(X.device)), "ns_line_3")
+    res = res[:, :m, :n]
+    if squeeze:
+        res = res[0]
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res.contiguous()
+
+
+def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: float, epsilon: float,
+                     gram: bool = False, gram_reset: int = 0) -> Tensor:
+    """Batched Newton-Schulz / Polar-Express orthogonalization of ``G[..., rows, cols]``.
+
+    X0 = bf16(G) / (||bf16(G)||_F * norm_scale + epsilon), then ``len(coeffs)`` quintic
+    iterations on the orientation with rows <= cols; result is bf16 with the shape of ``G``.
+    """
+    _require_gpu(G, "G")
+    if G.ndim < 2:
+        raise ValueError(f"expected a tensor with at least 2 dims, got shape {tuple(G.shape)}")
+    if G.dtype not in (torch.bfloat16, torch.float32):
+        G = G.to(torch.float32)
+    shape = G.shape
+    rows, cols = shape[-2], shape[-1]
+    G3 = G.reshape(-1, rows, cols).contiguous()
+    batch = G3.shape[0]
+    out = torch.empty(batch, rows, cols, dtype=torch.bfloat16, device=G.device)
+    if out.numel() == 0:
+        return out.reshape(shape)
+    flat = [float(v) for abc in coeffs for v in abc]
+    if len(flat) % 3:
+        raise ValueError("coeffs must be (a, b, c) triples")
+    n_iters = len(flat) // 3
+    carr = (_lib.ctypes.c_float * max(1, len(flat)))(*flat)
+    flags = DION_NS_GRAM if gram else 0
+    lib = _lib.load()
+    nbytes = lib.dion_ns_workspace_bytes(batch, rows, cols, flags)
+    ws = _workspace(G.device, nbytes)
+    check(lib.dion_ns_orthogonalize(G3.data_ptr(), _dtype_code(G3, "G"), out.data_ptr(), batch, rows, cols,
+                                    carr, n_iters, float(norm_scale), float(epsilon), flags,
+                                    int(gram_reset), ws.data_ptr(), ws.numel(), _stream_handle(G.device)),
+          "ns_orthogonalize")
+    return out.reshape(shape)
+
+
+# ---------------------------------------------------------------------------------------------
+# optimizer-step kernels on lists of same-shape parameters
+# ---------------------------------------------------------------------------------------------
+def _list_ptrs(ts: List[Tensor], name: str, dtype=None, numel=None):
+    for t in ts:
+        _require_gpu(t, name)
+        if not t.is_contiguous():
+            raise ValueError(f"{name}: tensors must be contiguous")
+        if dtype is not None and t.dtype != dtype:
+            raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+        if numel is not None and t.numel() != numel:
+            raise ValueError(f"{name}: all tensors of a shape group must have {numel} elements")
+    return ptr_table([t.data_ptr() for t in ts])
+
+
+def _scalar_args(lr: Tensor, weight_decay, device):
+    """lr must already be a 0-d fp32 device tensor; weight decay may be one, or a host number."""
+    if not (isinstance(lr, Tensor) and lr.is_cuda and lr.dtype == torch.float32 and lr.numel() == 1):
+        raise TypeError("lr must be a 0-d float32 tensor on the GPU")
+    if isinstance(weight_decay, Tensor) and weight_decay.is_cuda:
+        if weight_decay.dtype != torch.float32 or weight_decay.numel() != 1:
+            raise TypeError("a device weight_decay must be a 0-d float32 tensor")
+        return lr.data_ptr(), weight_decay.data_ptr(), 0.0
+    return lr.data_ptr(), None, float(weight_decay)
+
+
+def muon_pre(G: List[Tensor], M: List[Tensor], momentum: float, nesterov: bool) -> Tensor:
+    """Momentum update of every ``M[i]`` in place; returns the bf16 arena ``[N, *shape]`` holding the
+    orthogonalization inputs.  Mirrors ``muon_update_pre_orthogonalize`` (dion/muon.py:284-311)
+    followed by the ``torch.stack`` of dion/megabatch_base.py:872."""
+    n = len(G)
+    assert n == len(M) and n > 0
+    numel = M[0].numel()
+    gp = _list_ptrs(G, "G", G[0].dtype, numel)
+    mp = _list_ptrs(M, "M", torch.float32, numel)
+    U = torch.empty((n, *M[0].shape), dtype=torch.bfloat16, device=M[0].device)
+    lib = _lib.load()
+    check(lib.dion_muon_pre(gp, _dtype_code(G[0], "G"), mp, U.data_ptr(), n, numel, float(momentum),
+                            int(bool(nesterov)), _stream_handle(U.device)), "muon_pre")
+    return U
+
+
+def muon_post(X: List[Tensor], U: Tensor, lr: Tensor, adj_ratio: float, weight_decay, cautious_wd: bool = False,
+              row_scale: Optional[Tensor] = None) -> None:
+    """In-place weight decay + update of every ``X[i]`` from the arena ``U[i]``.  Mirrors
+    ``muon_update_post_orthogonalize`` (dion/muon.py:315-347); ``row_scale`` folds NorMuon's
+    per-row normalisation into the same pass."""
+    n = len(X)
+    assert n > 0 and U.shape[0] == n
+    numel = X[0].numel()
+    cols = X[0].shape[-1]
+    xp = _list_ptrs(X, "X", torch.float32, numel)
+    if not U.is_contiguous() or U.numel() != n * numel:
+        raise ValueError("U must be a contiguous [N, *shape] arena")
+    lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, U.device)
+    rs_p = None
+    if row_scale is not None:
+        if row_scale.dtype != torch.float32 or row_scale.numel() != n * (numel // cols):
+            raise ValueError("row_scale must be float32 [N, rows]")
+        rs_p = row_scale.data_ptr()
+    lib = _lib.load()
+    check(lib.dion_muon_post(xp, U.data_ptr(), _dtype_code(U, "U"), n, numel, cols, rs_p, lr_p,
+                             float(adj_ratio), wd_p, wd_h, int(bool(cautious_wd)),
+                             _stream_handle(U.device)), "muon_post")
+
+
+def normuon_stats(U: Tensor, V: List[Tensor], beta2: float) -> Tensor:
+    """Updates every ``V[i]`` (``[..., rows, 1]`` fp32) in place from the orthogonalized arena
+    ``U [N, ..., rows, cols]`` and returns the per-row scales ``[n_mat, rows]`` that turn ``U`` into the
+    NorMuon-normalised update.  Mirrors ``normuon_normalization_stacked`` (dion/normuon.py:345-399)."""
+    n = len(V)
+    assert n > 0 and U.shape[0] == n
+    _check_bf16(U, "U")
+    rows, cols = U.shape[-2], U.shape[-1]
+    n_mat = U.numel() // (rows * cols)
+    mats_per_ptr = n_mat // n
+    vp = _list_ptrs(V, "V", torch.float32, mats_per_ptr * rows)
+    scale = torch.empty(n_mat, rows, dtype=torch.float32, device=U.device)
+    lib = _lib.load()
+    check(lib.dion_normuon_stats(U.data_ptr(), vp, n, mats_per_ptr, rows, cols, float(beta2),
+                                 scale.data_ptr(), None, _stream_handle(U.device)), "normuon_stats")
+    return scale
+
+
+def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_decay: float):
+    """``M += G``; pick the ``k`` slices of largest L1 norm along ``select_dim`` of every matrix; return
+    (U_sel bf16 arena, idx int32 [n_mat, k] ascending, map int32 [n_mat, dim]) and decay the selected
+    slices of ``M`` by ``ef_decay``.  Mirrors ``dion2_pre_orthogonalize`` (dion/dion2.py:439-547)."""
+    if select_dim not in (-2, -1):
+        raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
+    n = len(G)
+    assert n == len(M) and n > 0
+    shape = M[0].shape
+    rows, cols = shape[-2], shape[-1]
+    numel = M[0].numel()
+    mats_per_ptr = numel // (rows * cols)
+    n_mat = n * mats_per_ptr
+    gp = _list_ptrs(G, "G", G[0].dtype, numel)
+    mp = _list_ptrs(M, "M", torch.float32, numel)
+    dev = M[0].device
+    dim = rows if select_dim == -2 else cols
+    norms = torch.empty(n_mat, dim, dtype=torch.float32, device=dev)
+    idx = torch.empty(n_mat, k, dtype=torch.int32, device=dev)
+    imap = torch.empty(n_mat, dim, dtype=torch.int32, device=dev)
+    sel_shape = (n, *shape[:-2], k, cols) if select_dim == -2 else (n, *shape[:-2], rows, k)
+    U = torch.empty(sel_shape, dtype=torch.bfloat16, device=dev)
+    lib = _lib.load()
+    st = _stream_handle(dev)
+    check(lib.dion_dion2_accumulate(gp, _dtype_code(G[0], "G"), mp, n, mats_per_ptr, rows, cols, select_dim,
+                                    norms.data_ptr(), st), "dion2_accumulate")
+    check(lib.dion_dion2_topk(norms.data_ptr(), n_mat, dim, k, idx.data_ptr(), imap.data_ptr(), st),
+          "dion2_topk")
+    check(lib.dion_dion2_gather(mp, n, mats_per_ptr, rows, cols, select_dim, idx.data_ptr(), k,
+                                float(ef_decay), U.data_ptr(), st), "dion2_gather")
+    return U, idx, imap
+
+
+def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: float, weight_decay,
+               select_dim: int) -> None:
+    """Fused ``x = (1 - lr*wd)*x - lr*adj_ratio*u[map]`` over every ``X[i]``.  Mirrors
+    ``dion2_post_orthogonalize_triton`` (dion/dion2_triton.py:147-242)."""
+    if select_dim not in (-2, -1):
+        raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
+    n = len(X)
+    assert n > 0
+    shape = X[0].shape
+    rows, cols = shape[-2], shape[-1]
+    numel = X[0].numel()
+    mats_per_ptr = numel // (rows * cols)
+    xp = _list_ptrs(X, "X", torch.float32, numel)
+    _check_bf16(U, "U")
+    k = U.shape[-2] if select_dim == -2 else U.shape[-1]
+    lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, U.device)
+    lib = _lib.load()
+    check(lib.dion_dion2_post(xp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(), k, imap.data_ptr(),
+                              lr_p, float(adj_ratio), wd_p, wd_h, _stream_handle(U.device)), "dion2_post")

