@@ -10,7 +10,12 @@ from .newton_schulz import (  # noqa: F401
     zeropower_via_newtonschulz5,
 )
 
+from .optimizers import Dion2, Muon, NorMuon  # noqa: E402,F401
+
 __all__ = [
+    "Muon",
+    "NorMuon",
+    "Dion2",
     "gram_newton_schulz",
     "newton_schulz_triton",
     "ns_line_1",

@@ -19,6 +19,11 @@ HIPCC_FLAGS = [
 ]
 
 
+# The step kernels keep the reference's separate multiply / add roundings (mul_ then add_), so no
+# FMA contraction there; the GEMM epilogues may contract.
+EXTRA_FLAGS = {"elementwise.hip": ["-ffp-contract=off"]}
+
+
 def hipcc_path() -> str:
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     cand = os.path.join(rocm, "bin", "hipcc")
@@ -31,7 +36,7 @@ def build(verbose: bool = True) -> str:
     procs = []
     for src in SOURCES:
         obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-        cmd = [hipcc_path(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc_path(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

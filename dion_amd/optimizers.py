@@ -1,0 +1,231 @@
+"""Muon, NorMuon and Dion2 with the constructor / param-group / step() / state_dict() contract of
+microsoft/dion (dion/muon.py:20-110, dion/normuon.py:20-133, dion/dion2.py:19-127), executing on
+the hand-written gfx950 kernels.
+
+Per shape group (all parameters of one shape and dtype) a step is:
+  Muon     muon_pre -> orthogonalize -> muon_post
+  NorMuon  muon_pre -> orthogonalize -> normuon_stats -> muon_post(row_scale)
+  Dion2    dion2_select -> orthogonalize(selected slices) -> dion2_post
+where the orthogonalization input/output is one dense bf16 arena ``[N, *shape]`` written and read
+directly by the fused kernels (the reference stacks and unbinds lists of tensors around it,
+dion/megabatch_base.py:870-881).
+"""
+import math
+from typing import Callable, List, Optional, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from . import ops
+from .optim_base import OrthoOptimizer, adjust_lr_ratio, split_lr_scales
+
+
+def _check_common(lr, betas, adjust_lr):
+    if lr < 0.0:
+        raise ValueError(f"Invalid learning rate: {lr}")
+    if len(betas) != 2 or betas[0] < 0.0 or betas[1] < 0.0:
+        raise ValueError(f"Invalid betas: {betas}")
+    if adjust_lr not in ("spectral_norm", "rms_norm", None):
+        raise ValueError(
+            f"Invalid adjust_lr value: {adjust_lr}. Must be 'spectral_norm', 'rms_norm', or None."
+        )
+
+
+def _require_fp32(params: List[Tensor], who: str) -> None:
+    if params[0].dtype != torch.float32:
+        raise NotImplementedError(
+            f"{who}: the gfx950 step kernels keep parameters and optimizer state in float32; "
+            f"got parameter dtype {params[0].dtype}"
+        )
+
+
+class _MomentumOrtho(OrthoOptimizer):
+    """Shared Muon / NorMuon shape-group update (dion/muon.py:194-280, dion/normuon.py:222-341)."""
+
+    _normalize = False
+
+    def _update_shape_group(self, group: dict, params: List[Tensor]) -> None:
+        num_heads = self._resolve_num_heads(group)
+        split_sizes = self._resolve_split_sizes(group)
+        shape = params[0].shape
+        flatten = group["flatten"]
+        split_scales = None
+        if split_sizes is not None:
+            self._validate_split_shape(split_sizes, shape)
+            split_scales = split_lr_scales(split_sizes, shape, group["adjust_lr"])
+        if num_heads is not None:
+            mats, rows, cols = self._head_geometry(num_heads, shape)
+            ratio_shape = (mats, rows, cols)  # the per-head 3D view decides the lr adjustment
+        else:
+            rows, cols = shape[-2], shape[-1]
+            mats = params[0].numel() // (rows * cols)
+            ratio_shape = shape
+        _require_fp32(params, type(self).__name__)
+        n = len(params)
+        X = [p.data for p in params]
+        G = [p.grad.contiguous() for p in params]
+        states = [self._get_or_initialize_state(p, self._algo_name) for p in params]
+        M = [s["momentum"] for s in states]
+        eps = float(group["epsilon"])
+
+        U = ops.muon_pre(G, M, group["mu"], group["nesterov"])  # [n, *shape] bf16
+
+        # shape plumbing of muon_update_newton_schulz (dion/megabatch_base.py:884-908)
+        if split_sizes is not None:
+            O = self._orthogonalize_row_blocks(U, split_sizes, split_scales, eps).contiguous()
+        elif flatten and len(shape) >= 3:
+            O = self._orthogonalize(U.view(n, shape[0], -1), eps)
+        else:
+            O = self._orthogonalize(U.view(n * mats, rows, cols), eps)
+
+        ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
+        row_scale = None
+        if self._normalize:
+            V = [s["variance_neuron"] for s in states]
+            O3 = O.view(n, mats, rows, cols)
+            if split_sizes is not None:
+                # per-block Frobenius-preserving rescale (dion/normuon.py:359-369)
+                scales, off = [], 0
+                for sz in split_sizes:
+                    blk = O3[:, :, off:off + sz, :].contiguous()
+                    vb = [v[off:off + sz] for v in V]
+                    scales.append(ops.normuon_stats(blk, vb, group["muon_beta2"]).view(n, sz))
+                    off += sz
+                row_scale = torch.cat(scales, dim=1).contiguous()
+            else:
+                row_scale = ops.normuon_stats(O3, V, group["muon_beta2"])
+        ops.muon_post(X, O.view(n, -1), group["lr"], ratio, group["weight_decay"],
+                      group["cautious_wd"], row_scale=row_scale)
+
+
+class Muon(_MomentumOrtho):
+    """Muon on one MI355X.  Same arguments as the reference ``Muon`` (dion/muon.py:61-78);
+    ``distributed_mesh`` must be None and ``use_triton`` selects nothing."""
+
+    def __init__(self, params, distributed_mesh=None, lr: float = 0.01, mu: float = 0.95,
+                 betas: Tuple[float, float] = (0.9, 0.95), weight_decay: Union[float, Tensor] = 0.01,
+                 cautious_wd: bool = False, epsilon: float = 1e-8, nesterov: bool = False,
+                 adjust_lr: Optional[str] = "spectral_norm", flatten: bool = False,
+                 use_gram_newton_schulz: bool = False, use_triton: bool = False,
+                 use_polar_express: bool = True, newton_schulz_func: Optional[Callable] = None):
+        _check_common(lr, betas, adjust_lr)
+        if mu < 0.0:
+            raise ValueError(f"Invalid momentum factor (mu): {mu}")
+        defaults = dict(lr=lr, mu=mu, beta1=betas[0], beta2=betas[1], weight_decay=weight_decay,
+                        cautious_wd=cautious_wd, algorithm="muon", step=0, epsilon=epsilon,
+                        nesterov=nesterov, flatten=flatten, adjust_lr=adjust_lr)
+        super().__init__(params, distributed_mesh, "muon", defaults,
+                         use_gram_newton_schulz=use_gram_newton_schulz, use_triton=use_triton,
+                         use_polar_express=use_polar_express, newton_schulz_func=newton_schulz_func)
+
+
+class NorMuon(_MomentumOrtho):
+    """NorMuon on one MI355X.  Same arguments as the reference ``NorMuon``
+    (dion/normuon.py:64-82); adds the ``variance_neuron`` state (dion/normuon.py:119-123)."""
+
+    _normalize = True
+
+    def __init__(self, params, distributed_mesh=None, lr: float = 0.01, mu: float = 0.95,
+                 muon_beta2: float = 0.95, betas: Tuple[float, float] = (0.9, 0.95),
+                 weight_decay: Union[float, Tensor] = 0.01, cautious_wd: bool = False,
+                 epsilon: float = 1e-8, nesterov: bool = False,
+                 adjust_lr: Optional[str] = "spectral_norm", flatten: bool = False,
+                 use_gram_newton_schulz: bool = False, use_triton: bool = False,
+                 use_polar_express: bool = True, newton_schulz_func: Optional[Callable] = None):
+        _check_common(lr, betas, adjust_lr)
+        if mu < 0.0:
+            raise ValueError(f"Invalid momentum factor (mu): {mu}")
+        if muon_beta2 < 0.0:
+            raise ValueError(f"Invalid muon_beta2: {muon_beta2}")
+        defaults = dict(lr=lr, mu=mu, muon_beta2=muon_beta2, beta1=betas[0], beta2=betas[1],
+                        weight_decay=weight_decay, cautious_wd=cautious_wd, algorithm="normuon",
+                        step=0, epsilon=epsilon, nesterov=nesterov, flatten=flatten,
+                        adjust_lr=adjust_lr)
+        super().__init__(params, distributed_mesh, "normuon", defaults,
+                         use_gram_newton_schulz=use_gram_newton_schulz, use_triton=use_triton,
+                         use_polar_express=use_polar_express, newton_schulz_func=newton_schulz_func)
+
+    def _get_or_initialize_state(self, param: Tensor, algo: str) -> dict:
+        state = super()._get_or_initialize_state(param, algo)
+        if algo == self._algo_name and "variance_neuron" not in state:
+            state["variance_neuron"] = torch.zeros_like(param[..., 0:1])
+        return state
+
+
+class Dion2(OrthoOptimizer):
+    """Dion2 on one MI355X.  Same arguments as the reference ``Dion2`` (dion/dion2.py:60-79).
+    ``triton_post_ortho`` is accepted and selects nothing (the fused single-rounding post kernel is
+    the only one); ``selection_scope`` only matters for sharded parameters and is validated only."""
+
+    _printed = set()
+
+    def __init__(self, params, distributed_mesh=None, lr: float = 0.01, fraction: float = 0.25,
+                 ef_decay: float = 0.95, betas: Tuple[float, float] = (0.9, 0.95),
+                 weight_decay: Union[float, Tensor] = 0.01, epsilon: float = 1e-8,
+                 adjust_lr: Optional[str] = "spectral_norm", flatten: bool = False,
+                 use_triton: bool = False, use_polar_express: bool = True,
+                 use_gram_newton_schulz: bool = False, newton_schulz_func: Optional[Callable] = None,
+                 verbose: bool = False, triton_post_ortho: bool = False, selection_scope: str = "local"):
+        if lr < 0.0:
+            raise ValueError(f"Invalid learning rate: {lr}")
+        if not (0.0 < fraction <= 1.0):
+            raise ValueError(f"fraction must be in (0, 1], got {fraction}")
+        if selection_scope not in ("local", "global"):
+            raise ValueError(f"selection_scope must be 'local' or 'global', got {selection_scope!r}")
+        if ef_decay < 0.0:
+            raise ValueError(f"Invalid ef_decay: {ef_decay}")
+        _check_common(lr, betas, adjust_lr)
+        defaults = dict(lr=lr, ef_decay=ef_decay, fraction=float(fraction), beta1=betas[0], beta2=betas[1],
+                        weight_decay=weight_decay, epsilon=epsilon, flatten=flatten, adjust_lr=adjust_lr,
+                        algorithm="dion2", step=0, selection_scope=selection_scope)
+        super().__init__(params, distributed_mesh, "dion2", defaults,
+                         use_gram_newton_schulz=use_gram_newton_schulz, use_triton=use_triton,
+                         use_polar_express=use_polar_express, newton_schulz_func=newton_schulz_func)
+        self.verbose = verbose
+        self._triton_post_ortho = bool(triton_post_ortho)
+
+    def _update_shape_group(self, group: dict, params: List[Tensor]) -> None:
+        num_heads = self._resolve_num_heads(group)
+        if group.get("split_sizes") is not None:
+            raise NotImplementedError("split_sizes is currently supported only by Muon and NorMuon.")
+        shape = params[0].shape
+        flatten = group["flatten"]
+        if num_heads is not None:
+            mats, rows, cols = self._head_geometry(num_heads, shape)
+            ratio_shape = (mats, rows, cols)
+        else:
+            rows, cols = shape[-2], shape[-1]
+            mats = params[0].numel() // (rows * cols)
+            ratio_shape = shape
+        _require_fp32(params, "Dion2")
+        n = len(params)
+        # unsharded: select along the shorter dimension (dion/dion2.py:270-272)
+        select_dim = -2 if rows <= cols else -1
+        dim = rows if select_dim == -2 else cols
+        k = min(max(1, int(math.ceil(group["fraction"] * dim))), dim)
+        if self.verbose:
+            key = (tuple(shape), select_dim)
+            if key not in Dion2._printed:
+                Dion2._printed.add(key)
+                what = "rows" if select_dim == -2 else "columns"
+                print(f"[Dion2] Shape {tuple(shape)}: single GPU, shorter dim ({dim}) -> "
+                      f"select top-{k} {what} by L1 norm")
+
+        X = [p.data.view(mats, rows, cols) for p in params]
+        G = [p.grad.contiguous().view(mats, rows, cols) for p in params]
+        M = [self._get_or_initialize_state(p, self._algo_name)["momentum"].view(mats, rows, cols)
+             for p in params]
+
+        U_sel, _idx, imap = ops.dion2_select(G, M, k, select_dim, group["ef_decay"])
+        sel_rows, sel_cols = U_sel.shape[-2], U_sel.shape[-1]
+        eps = float(group["epsilon"])
+        if flatten and len(shape) >= 3:
+            # leading dim stays, the rest of the selected block is one long row
+            # (dion/megabatch_base.py:903-904)
+            lead = shape[0]
+            O = self._orthogonalize(U_sel.view(n, lead, -1), eps)
+        else:
+            O = self._orthogonalize(U_sel.view(n * mats, sel_rows, sel_cols), eps)
+        ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
+        ops.dion2_post(X, O.view(n, mats, sel_rows, sel_cols), imap, group["lr"], ratio,
+                       group["weight_decay"], select_dim)

@@ -1,0 +1,160 @@
+"""Host-side contract of the optimizers (constructor, param groups, state, validation) -- no GPU.
+Mirrors what the reference pins in tests/test_state_prepopulation.py and the TestValidation class
+of tests/test_optimizers.py."""
+import pytest
+import torch
+
+from dion import Dion2, Muon, NorMuon
+
+
+def _params(shapes):
+    torch.manual_seed(0)
+    return [torch.nn.Parameter(torch.randn(s)) for s in shapes]
+
+
+def test_state_exists_at_construction():
+    p = _params([(16, 32), (32, 16)])
+    for cls, keys in [(Muon, {"momentum"}), (Dion2, {"momentum"}), (NorMuon, {"momentum", "variance_neuron"})]:
+        opt = cls(p, lr=0.01)
+        for q in p:
+            assert set(opt.state[q].keys()) == keys
+            assert torch.equal(opt.state[q]["momentum"], torch.zeros_like(q))
+        if cls is NorMuon:
+            assert opt.state[p[0]]["variance_neuron"].shape == (16, 1)
+
+
+def test_param_group_keys_and_defaults():
+    p = _params([(16, 32)])
+    g = Muon(p).param_groups[0]
+    assert {"lr", "mu", "beta1", "beta2", "weight_decay", "cautious_wd", "algorithm", "step", "epsilon",
+            "nesterov", "flatten", "adjust_lr"} <= set(g)
+    assert g["algorithm"] == "muon" and g["step"] == 0 and g["mu"] == 0.95 and g["adjust_lr"] == "spectral_norm"
+    g = NorMuon(p).param_groups[0]
+    assert g["algorithm"] == "normuon" and g["muon_beta2"] == 0.95
+    g = Dion2(p, fraction=1).param_groups[0]
+    assert g["algorithm"] == "dion2" and g["fraction"] == 1.0 and isinstance(g["fraction"], float)
+    assert g["ef_decay"] == 0.95 and g["selection_scope"] == "local"
+
+
+def test_lr_is_a_persistent_tensor_and_state_dict_is_portable():
+    p = _params([(16, 32)])
+    opt = Muon(p, lr=0.02)
+    lr = opt.param_groups[0]["lr"]
+    assert isinstance(lr, torch.Tensor) and lr.ndim == 0 and lr.dtype == torch.float32
+    sd = opt.state_dict()
+    assert isinstance(sd["param_groups"][0]["lr"], float)
+    assert sd["param_groups"][0]["lr"] == pytest.approx(0.02)
+    # a float assigned by a hand-rolled schedule is copied into the same tensor on sync
+    opt.param_groups[0]["lr"] = 0.05
+    opt._sync_hyperparam_tensors()
+    assert opt.param_groups[0]["lr"] is lr and float(lr) == pytest.approx(0.05)
+    opt2 = Muon(_params([(16, 32)]), lr=0.5)
+    opt2.load_state_dict(sd)
+    assert float(opt2.param_groups[0]["lr"]) == pytest.approx(0.02)
+    # LR schedulers attach like to any torch optimizer
+    sched = torch.optim.lr_scheduler.LambdaLR(opt2, lambda s: 0.5)
+    assert float(opt2.param_groups[0]["lr"]) == pytest.approx(0.01)
+    assert sched is not None
+
+
+def test_weight_decay_tensor_becomes_live():
+    p = _params([(16, 32)])
+    opt = Muon(p, weight_decay=torch.tensor(0.1))
+    wd = opt.param_groups[0]["weight_decay"]
+    assert isinstance(wd, torch.Tensor) and wd.ndim == 0
+    assert isinstance(opt.state_dict()["param_groups"][0]["weight_decay"], float)
+
+
+def test_constructor_validation():
+    p = _params([(16, 32)])
+    with pytest.raises(ValueError):
+        Muon(p, lr=-0.01)
+    with pytest.raises(ValueError):
+        NorMuon(p, mu=-1.0)
+    with pytest.raises(ValueError):
+        NorMuon(p, muon_beta2=-1.0)
+    with pytest.raises(ValueError):
+        Dion2(p, fraction=0.0)
+    with pytest.raises(ValueError):
+        Dion2(p, fraction=1.5)
+    with pytest.raises(ValueError):
+        Dion2(p, selection_scope="shard")
+    with pytest.raises(ValueError):
+        Dion2(p, ef_decay=-0.1)
+    with pytest.raises(ValueError):
+        Muon(p, adjust_lr="invalid")
+    with pytest.raises(ValueError):
+        Muon(p, betas=(0.9,))
+    with pytest.raises(TypeError):
+        Muon(p, newton_schulz_func="not callable")
+    with pytest.raises(TypeError):
+        Muon(p, distributed_mesh="mesh")
+
+
+def test_no_grad_step_is_a_noop_and_counts_steps():
+    p = _params([(16, 32)])
+    before = p[0].data.clone()
+    opt = Muon(p, lr=0.01)
+    opt.step()
+    assert torch.equal(p[0].data, before)
+    assert opt.param_groups[0]["step"] == 1
+
+
+def test_step_validation_on_cpu_params():
+    """Errors raised before any kernel is reached."""
+    w = torch.nn.Parameter(torch.randn(64))
+    w.grad = torch.randn_like(w)
+    with pytest.raises(AssertionError):
+        Muon([{"params": [w]}], lr=0.01).step()
+    for bad in [0, -1, 2.0, "4", True]:
+        w = torch.nn.Parameter(torch.randn(32, 16))
+        w.grad = torch.randn_like(w)
+        with pytest.raises(ValueError, match="num_heads"):
+            Muon([{"params": [w], "num_heads": bad}], lr=0.01).step()
+    w = torch.nn.Parameter(torch.randn(30, 16))
+    w.grad = torch.randn_like(w)
+    with pytest.raises(ValueError, match="num_heads"):
+        Muon([{"params": [w], "num_heads": 4}], lr=0.01).step()
+    w = torch.nn.Parameter(torch.randn(4, 8, 16))
+    w.grad = torch.randn_like(w)
+    with pytest.raises(ValueError, match="2D"):
+        Muon([{"params": [w], "num_heads": 2}], lr=0.01).step()
+    w = torch.nn.Parameter(torch.randn(32, 16))
+    w.grad = torch.randn_like(w)
+    with pytest.raises(ValueError, match="flatten"):
+        Muon([{"params": [w], "num_heads": 4}], lr=0.01, flatten=True).step()
+    for bad in [3, (32,), (32, 0), (32, -1), (32, 2.0), (32, "16"), (32, True)]:
+        w = torch.nn.Parameter(torch.randn(64, 32))
+        w.grad = torch.randn_like(w)
+        with pytest.raises(ValueError, match="split_sizes"):
+            Muon([{"params": [w], "split_sizes": bad}], lr=0.01).step()
+    w = torch.nn.Parameter(torch.randn(60, 32))
+    w.grad = torch.randn_like(w)
+    with pytest.raises(ValueError, match="split_sizes"):
+        Muon([{"params": [w], "split_sizes": (32, 16, 16)}], lr=0.01).step()
+    w = torch.nn.Parameter(torch.randn(64, 32))
+    w.grad = torch.randn_like(w)
+    with pytest.raises(ValueError, match="num_heads"):
+        Muon([{"params": [w], "split_sizes": (32, 16, 16), "num_heads": 4}], lr=0.01).step()
+    with pytest.raises(NotImplementedError, match="split_sizes"):
+        Dion2([{"params": [w], "split_sizes": (32, 16, 16)}], lr=0.01).step()
+    with pytest.raises(ValueError, match="Unknown algorithm"):
+        Muon([{"params": [w], "algorithm": "sgd"}], lr=0.01).step()
+
+
+def test_scalar_groups_run_on_cpu():
+    """adamw / lion groups use stock torch ops and keep their state contract."""
+    b = torch.nn.Parameter(torch.randn(8))
+    c = torch.nn.Parameter(torch.randn(8))
+    opt = Muon([{"params": [b], "algorithm": "adamw"}, {"params": [c], "algorithm": "lion"}], lr=0.01)
+    assert set(opt.state[b].keys()) == {"momentum", "variance", "step_dev"}
+    assert set(opt.state[c].keys()) == {"momentum"}
+    b0, c0 = b.data.clone(), c.data.clone()
+    b.grad = torch.randn(8)
+    c.grad = torch.randn(8)
+    opt.step()
+    assert not torch.equal(b.data, b0) and not torch.equal(c.data, c0)
+    assert float(opt.state[b]["step_dev"]) == 1.0
+    # first AdamW step moves each weight by ~lr in the gradient's direction
+    moved = (b0 * (1 - 0.01 * 0.01) - b.data)
+    assert torch.allclose(moved, 0.01 * torch.sign(b.grad), atol=1e-4)
