@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Benchmark of the Muon optimizer-step hot path on one MI355X.
+
+A "step" is one full ``Muon.step()`` over synthetic parameters of the named model shape list
+(momentum + Nesterov, batched Newton-Schulz orthogonalization, weight decay + update), inputs
+resident in HBM.  ``value`` is the algorithmic Newton-Schulz TFLOP/s of the whole step,
+``5*(4 m^2 n + 2 m^3)`` FLOP per matrix (the reference's benchmark/benchmark_newton_shultz.py:40-49
+convention, not reduced for symmetry) summed over all matrices, divided by the full step time.
+
+Prints ONE JSON line; see --help for the workloads.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+# (name, rows, cols, count) per workload; counts are whole-model totals.
+WORKLOADS = {
+    # Llama-3-8B: 32 layers, d 4096, GQA 32q/8kv, MLP 14336
+    "llama3_8b": [("q_o", 4096, 4096, 64), ("k_v", 1024, 4096, 64), ("gate_up", 14336, 4096, 64),
+                  ("down", 4096, 14336, 32)],
+    # GPT-small 160M: 12 layers, d 768
+    "gpt_small": [("qkv", 2304, 768, 12), ("attn_out", 768, 768, 12), ("fc", 3072, 768, 12),
+                  ("proj", 768, 3072, 12)],
+    # 1.3B: 24 layers, d 2048, MLP 8192
+    "gpt_1p3b": [("qkv", 6144, 2048, 24), ("out", 2048, 2048, 24), ("fc", 8192, 2048, 24),
+                 ("proj", 2048, 8192, 24)],
+    # the headline shape group on its own
+    "ns_4096x14336": [("down", 4096, 14336, 32)],
+}
+
+
+def ns_flops(rows: int, cols: int, iters: int = 5) -> float:
+    m, n = min(rows, cols), max(rows, cols)
+    return iters * (4.0 * m * m * n + 2.0 * m ** 3)
+
+
+def cpu_baseline(ns: str):
+    """Oracle (torch-CPU restatement of the reference's bf16 path) timed on the host cores on a
+    bounded sample: one 4096x14336 matrix, Frobenius normalisation + 5 iterations."""
+    import torch
+
+    from oracle import dion_oracle as oracle
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(1234)
+    G = (torch.randn(4096, 14336, generator=g) * 0.02).to(torch.bfloat16)
+    oracle.ns_bf16(G[:256, :1024].contiguous())  # warm the thread pool
+    t0 = time.perf_counter()
+    if ns == "polar_express":
+        oracle.polar_express_bf16(G, eps=1e-8)
+    else:
+        oracle.ns_bf16(G, oracle.NS5_COEFFS, 1.0, 1e-8)
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(ns_flops(4096, 14336) / dt * 1e-12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"1 of the 32 4096x14336 matrices, Frobenius normalisation + 5 {ns} iterations, "
+                  f"torch-CPU bf16 matmul, {dt:.1f} s",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="llama3_8b", choices=sorted(WORKLOADS))
+    ap.add_argument("--ns", default="ns5", choices=["ns5", "polar_express"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-timing", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build drives one GPU per process and has no multi-GPU path; "
+              "run with --gpus 1 (the step of an N-GPU job is this step on 1/N of each shape group).",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    from dion import Muon
+    from dion_amd import _lib, ops
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    spec = WORKLOADS[args.workload]
+
+    # ---- synthetic model: X ~ N(0, 0.02) fp32, G ~ N(0, 0.02) bf16, momentum fp32 zeros
+    params = []
+    gen = torch.Generator(device=dev).manual_seed(1234)
+    total_flops = 0.0
+    total_elems = 0
+    for _name, rows, cols, count in spec:
+        for _ in range(count):
+            p = torch.nn.Parameter(torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen))
+            p.grad_dtype = None
+            p.grad = torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen).to(torch.bfloat16)
+            params.append(p)
+        total_flops += count * ns_flops(rows, cols)
+        total_elems += count * rows * cols
+    opt = Muon(params, lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, adjust_lr="spectral_norm",
+               use_polar_express=(args.ns == "polar_express"))
+
+    for _ in range(args.warmup):
+        opt.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        opt.step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = total_flops / (ms_per_step * 1e-3) * 1e-12
+
+    result = {
+        "metric": "Newton-Schulz TFLOP/s (% bf16 MFMA peak) + full optimizer-step ms, 1 GPU",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: full Muon.step() (nesterov mu=0.95, {args.ns}, wd 0.01, lr 0.02) over "
+                        + ", ".join(f"{c}x({r}x{k})" for _n, r, k, c in spec),
+            "matrices": sum(c for *_x, c in spec),
+            "elements": total_elems,
+            "ns_flop_per_step": total_flops,
+        },
+        "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
+    }
+
+    # ---- free the model, then time kernels of the headline shape group on their own
+    del opt
+    for p in params:
+        p.grad = None
+    del params
+    ops.release_workspaces()
+    torch.cuda.empty_cache()
+
+    if not args.no_kernel_timing:
+        lib = _lib.load()
+        B, m, n = 32, 4096, 14336
+        if args.workload == "gpt_small":
+            B, m, n = 12, 768, 3072
+        elif args.workload == "gpt_1p3b":
+            B, m, n = 24, 2048, 8192
+        st = torch.cuda.current_stream().cuda_stream
+        X = (torch.randn(B, m, n, device=dev) * 0.01).to(torch.bfloat16)
+        Xt = X.mT.contiguous()
+        Bm = (torch.randn(B, m, m, device=dev) * 0.01)
+        Bm = ((Bm + Bm.mT) * 0.5).to(torch.bfloat16)
+        C = torch.empty_like(X)
+        Ct = torch.empty_like(Xt)
+
+        def time_kernel(fn, iters=10):
+            fn()
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / iters
+
+        # dominant kernel: X' = a X + B X (both layouts), one launch per NS iteration
+        ms3 = time_kernel(lambda: lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), Xt.data_ptr(), C.data_ptr(),
+                                                     Ct.data_ptr(), B, m, n, 1.0, st))
+        flop3 = 2.0 * B * m * m * n
+        achieved = flop3 / (ms3 * 1e-3) * 1e-12
+        result["roofline"] = {
+            "bound": "mfma",
+            "kernel": "gemm_nt_kernel (X' = a X + B X, stores X' and X'^T)",
+            "achieved": round(achieved, 2),
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+            "traffic": None,
+            "launch_ms": round(ms3, 4),
+            "launch_shape": f"{B}x({m}x{m})·({m}x{n})",
+        }
+        # whole NS on the headline group
+        from dion_amd import polar_express, zeropower_via_newtonschulz5
+
+        fn = polar_express if args.ns == "polar_express" else zeropower_via_newtonschulz5
+        del C, Ct, Xt, Bm
+        ms_ns = time_kernel(lambda: fn(X, 1e-8), iters=3)
+        ns_tf = B * ns_flops(m, n) / (ms_ns * 1e-3) * 1e-12
+        result["ns_headline"] = {
+            "shape": f"{B}x({m}x{n})",
+            "ms": round(ms_ns, 3),
+            "tflops": round(ns_tf, 2),
+            "pct_of_bf16_peak": round(100.0 * ns_tf / PEAK_BF16_TFLOPS, 2),
+        }
+        del X
+        torch.cuda.empty_cache()
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.ns)
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -2,6 +2,7 @@
 // Newton-Schulz driver that strings the GEMM launches together.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "../../include/dion_hip.h"
@@ -121,8 +122,20 @@ extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void
 // Whole orthogonalization
 // ---------------------------------------------------------------------------------------------
 namespace {
+// Rows of the workspace matrices are padded by kLdPad elements: a row pitch that is a multiple of
+// 4 KiB sends every row of a tile to the same L2 channel.
+static int ld_pad() {
+  static const int pad = [] {
+    const char* e = getenv("DION_LD_PAD");
+    int v = e ? atoi(e) : 0;
+    return v < 0 ? 0 : (v / 8) * 8;
+  }();
+  return pad;
+}
+
 struct NsPlan {
   int m, n, mp, np, tall, nblk;
+  int ldx, ldxt, lda;  // row pitch (elements) of X [mp][np], X^T [np][mp], A/B [mp][mp]
   size_t x_bytes, a_bytes, partial_bytes, inv_bytes, total;
 };
 
@@ -139,8 +152,13 @@ NsPlan make_plan(int batch, int rows, int cols, int flags) {
   if (nb < 1) nb = 1;
   if (nb > 256) nb = 256;
   pl.nblk = (int)nb;
-  pl.x_bytes = align256((size_t)batch * pl.mp * pl.np * 2);
-  pl.a_bytes = align256((size_t)batch * pl.mp * pl.mp * 2);
+  pl.ldx = pl.np + ld_pad();
+  pl.ldxt = pl.mp + ld_pad();
+  pl.lda = pl.mp + ld_pad();
+  const size_t x_elems = (size_t)pl.mp * pl.ldx > (size_t)pl.np * pl.ldxt ? (size_t)pl.mp * pl.ldx
+                                                                          : (size_t)pl.np * pl.ldxt;
+  pl.x_bytes = align256((size_t)batch * x_elems * 2);
+  pl.a_bytes = align256((size_t)batch * pl.mp * pl.lda * 2);
   pl.partial_bytes = align256((size_t)batch * pl.nblk * 4);
   pl.inv_bytes = align256((size_t)batch * 4);
   // X, Xt ping-pong pairs; A, B (+ Q, Z, T for the Gram recurrence)
@@ -190,13 +208,17 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   float* inv = (float*)w; w += pl.inv_bytes;
 
   const int mp = pl.mp, np = pl.np;
+  const int ldx = pl.ldx, ldxt = pl.ldxt, lda = pl.lda;
+  const int64_t sX = (int64_t)mp * ldx, sXt = (int64_t)np * ldxt, sA = (int64_t)mp * lda;
   HIP_TRY(launch_frobenius_inv(in, in_dtype, batch, (int64_t)rows * cols, norm_scale, eps, partial,
                                pl.nblk, inv, st),
           "frobenius norm");
   if (pl.tall)
-    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, Xt[0], np, mp, X[0], st), "prepare");
+    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, Xt[0], np, mp, ldxt, sXt, X[0], ldx, sX, st),
+            "prepare");
   else
-    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, X[0], mp, np, Xt[0], st), "prepare");
+    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, X[0], mp, np, ldx, sX, Xt[0], ldxt, sXt, st),
+            "prepare");
 
   const bool direct = (mp == pl.m && np == pl.n);
   int cur = 0;
@@ -207,10 +229,10 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     memset(&p, 0, sizeof(p));
     p.P = p.Q = X[cur];
     p.C = p.Ct = A;
-    p.strideP = p.strideQ = (int64_t)mp * np;
-    p.strideC = p.strideCt = (int64_t)mp * mp;
-    p.ldp = p.ldq = np;
-    p.ldc = p.ldct = mp;
+    p.strideP = p.strideQ = sX;
+    p.strideC = p.strideCt = sA;
+    p.ldp = p.ldq = ldx;
+    p.ldc = p.ldct = lda;
     p.M = p.N = p.Mst = p.Nst = mp;
     p.K = np;
     p.batch = batch;
@@ -221,8 +243,8 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     memset(&p, 0, sizeof(p));
     p.P = p.Q = p.D = A;
     p.C = p.Ct = Bm;
-    p.strideP = p.strideQ = p.strideD = p.strideC = p.strideCt = (int64_t)mp * mp;
-    p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = mp;
+    p.strideP = p.strideQ = p.strideD = p.strideC = p.strideCt = sA;
+    p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = lda;
     p.M = p.N = p.K = p.Mst = p.Nst = mp;
     p.batch = batch;
     p.tri = 1;
@@ -234,11 +256,12 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     p.P = Bm;
     p.Q = Xt[cur];
     p.D = X[cur];
-    p.strideP = (int64_t)mp * mp;
-    p.strideQ = p.strideD = (int64_t)mp * np;
-    p.ldp = mp;
-    p.ldq = mp;
-    p.ldd = np;
+    p.strideP = sA;
+    p.strideQ = sXt;
+    p.strideD = sX;
+    p.ldp = lda;
+    p.ldq = ldxt;
+    p.ldd = ldx;
     p.M = p.Mst = mp;
     p.N = p.Nst = np;
     p.K = mp;
@@ -259,18 +282,19 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     } else {
       p.C = X[cur ^ 1];
       p.Ct = Xt[cur ^ 1];
-      p.strideC = p.strideCt = (int64_t)mp * np;
-      p.ldc = np;
-      p.ldct = mp;
+      p.strideC = sX;
+      p.strideCt = sXt;
+      p.ldc = ldx;
+      p.ldct = ldxt;
     }
     HIP_TRY(launch_gemm_nt(p, -1, st), "X = a X + B X");
     cur ^= 1;
   }
   if (!(direct && n_iters > 0)) {
     if (pl.tall)
-      HIP_TRY(launch_unpad(Xt[cur], (int64_t)mp * np, mp, (bf16_t*)out, batch, rows, cols, st), "unpad");
+      HIP_TRY(launch_unpad(Xt[cur], sXt, ldxt, (bf16_t*)out, batch, rows, cols, st), "unpad");
     else
-      HIP_TRY(launch_unpad(X[cur], (int64_t)mp * np, np, (bf16_t*)out, batch, rows, cols, st), "unpad");
+      HIP_TRY(launch_unpad(X[cur], sX, ldx, (bf16_t*)out, batch, rows, cols, st), "unpad");
   }
   return DION_OK;
 }

@@ -16,7 +16,8 @@ hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t
                                 float norm_scale, float eps, float* partial, int nblk,
                                 float* inv_norm, hipStream_t st);
 hipError_t launch_ns_prepare(const void* in, int in_dtype, int batch, int R, int C,
-                             const float* inv_norm, bf16_t* same, int Rp, int Cp, bf16_t* trans,
+                             const float* inv_norm, bf16_t* same, int Rp, int Cp, int ld_same,
+                             int64_t stride_same, bf16_t* trans, int ld_trans, int64_t stride_trans,
                              hipStream_t st);
 hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* dst, int batch, int R,
                         int C, hipStream_t st);

@@ -73,14 +73,16 @@ template <typename T>
 __global__ __launch_bounds__(256) void ns_prepare_kernel(const T* __restrict__ in, int R, int C,
                                                          const float* __restrict__ inv_norm,
                                                          bf16_t* __restrict__ same, int Rp, int Cp,
-                                                         bf16_t* __restrict__ trans) {
+                                                         int ld_same, int64_t stride_same,
+                                                         bf16_t* __restrict__ trans, int ld_trans,
+                                                         int64_t stride_trans) {
   __shared__ bf16_t tile[64][66];
   const int b = blockIdx.z;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   const float sc = inv_norm[b];
   const T* src = in + (int64_t)b * R * C;
-  bf16_t* ds = same + (int64_t)b * Rp * Cp;
-  bf16_t* dt = trans + (int64_t)b * Rp * Cp;
+  bf16_t* ds = same + (int64_t)b * stride_same;
+  bf16_t* dt = trans + (int64_t)b * stride_trans;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
 #pragma unroll 4
   for (int i = ty; i < 64; i += 4) {
@@ -88,13 +90,13 @@ __global__ __launch_bounds__(256) void ns_prepare_kernel(const T* __restrict__ i
     bf16_t v = 0;
     if (r < R && c < C) v = f32_to_bf16(load_as_bf16_f32<T>(src, (int64_t)r * C + c) * sc);
     tile[i][tx] = v;
-    ds[(int64_t)r * Cp + c] = v;
+    ds[(int64_t)r * ld_same + c] = v;
   }
   __syncthreads();
 #pragma unroll 4
   for (int i = ty; i < 64; i += 4) {
     // trans row (c0 + i), column (r0 + tx)
-    dt[(int64_t)(c0 + i) * Rp + r0 + tx] = tile[tx][i];
+    dt[(int64_t)(c0 + i) * ld_trans + r0 + tx] = tile[tx][i];
   }
 }
 
@@ -123,15 +125,16 @@ hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t
 }
 
 hipError_t launch_ns_prepare(const void* in, int in_dtype, int batch, int R, int C,
-                             const float* inv_norm, bf16_t* same, int Rp, int Cp, bf16_t* trans,
+                             const float* inv_norm, bf16_t* same, int Rp, int Cp, int ld_same,
+                             int64_t stride_same, bf16_t* trans, int ld_trans, int64_t stride_trans,
                              hipStream_t st) {
   dim3 grid(Cp / 64, Rp / 64, batch);
   if (in_dtype == 0)
     hipLaunchKernelGGL(ns_prepare_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)in, R, C,
-                       inv_norm, same, Rp, Cp, trans);
+                       inv_norm, same, Rp, Cp, ld_same, stride_same, trans, ld_trans, stride_trans);
   else
     hipLaunchKernelGGL(ns_prepare_kernel<float>, grid, dim3(256), 0, st, (const float*)in, R, C,
-                       inv_norm, same, Rp, Cp, trans);
+                       inv_norm, same, Rp, Cp, ld_same, stride_same, trans, ld_trans, stride_trans);
   return hipGetLastError();
 }
 

@@ -14,6 +14,8 @@
 // (v_mfma_f32_32x32x16_bf16).  Operand tiles stream global -> LDS with the direct-to-LDS loads
 // (global_load_lds_dwordx4, no VGPR staging) into an NSTAGE ring; a 16-byte-chunk XOR swizzle
 // keeps both the DMA writes and the ds_read_b128 fragment reads bank-conflict free.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace dion {
@@ -30,14 +32,22 @@ struct TileCfg {
   static constexpr int P_BYTES = BM * BK * 2;
   static constexpr int Q_BYTES = BN * BK * 2;
   static constexpr int STAGE_BYTES = P_BYTES + Q_BYTES;
-  static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
+  // Epilogue staging of the transposed tile: per wavefront WTN rows of WTM bf16 (+16 B pad).
+  static constexpr int STG_PITCH = (BM / WM_) * 2 + 16;
+  static constexpr int STG_BYTES = (BN / WN_) * STG_PITCH;
+  static constexpr int RING_BYTES = STAGE_BYTES * NSTAGE;
+  static constexpr int LDS_BYTES =
+      RING_BYTES > STG_BYTES * WM_ * WN_ ? RING_BYTES : STG_BYTES * WM_ * WN_;
   static constexpr int P_LOADS = BM / ROWS_PER_LOAD;
   static constexpr int Q_LOADS = BN / ROWS_PER_LOAD;
   static constexpr int LOADS_PER_STAGE = P_LOADS + Q_LOADS;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static constexpr int KK = BK / 16;
-  static constexpr int SWZ_DIV = 8 / CPR;       // rows sharing one swizzle value
+  // gfx950 LDS: 64 banks x 4 B = 256-byte bank rows, and a ds_read_b128 is served 16 lanes at a
+  // time.  16 consecutive tile rows must therefore land in 16 distinct 16-byte slots of a bank
+  // row: the 256/(2*BK) tile rows that share a bank row take one swizzle value.
+  static constexpr int SWZ_DIV = 256 / (BK * 2);
   static_assert(BM % ROWS_PER_LOAD == 0 && BN % ROWS_PER_LOAD == 0, "tile/threads mismatch");
   static_assert(CPR == 8 || CPR == 4, "BK must be 64 or 32");
 };
@@ -50,16 +60,44 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
 }
 
+// Enumeration of the upper triangle (ti <= tj) of a T x T tile grid in super-blocks of SB x SB
+// tiles, so that the ~32 workgroups an XCD runs side by side touch as few distinct operand row
+// blocks as possible (their L2 is what feeds the LDS): a diagonal super-block has SB(SB+1)/2
+// tiles over only SB row blocks; an off-diagonal one is walked in SB x 4 column groups.
 __device__ __forceinline__ void tri_tile(int t, int T, int& ti, int& tj) {
-  // Row-major enumeration of the upper triangle of a T x T tile grid.
-  float f = (float)(2 * T + 1);
-  int i = (int)((f - sqrtf(f * f - 8.0f * (float)t)) * 0.5f);
-  if (i < 0) i = 0;
-  if (i > T - 1) i = T - 1;
-  while (i + 1 < T && (i + 1) * T - ((i + 1) * i) / 2 <= t) ++i;
-  while (i > 0 && i * T - (i * (i - 1)) / 2 > t) --i;
-  ti = i;
-  tj = i + (t - (i * T - (i * (i - 1)) / 2));
+  constexpr int SB = 8;
+  const int nb = (T + SB - 1) / SB;
+  for (int I = 0; I < nb; ++I) {
+    const int r = (T - I * SB) < SB ? (T - I * SB) : SB;  // tile rows in super-row I
+    const int diag = r * (r + 1) / 2;
+    if (t < diag) {
+      // row-major triangle of side r
+      int i = 0, rem = t;
+      while (rem >= r - i) {
+        rem -= r - i;
+        ++i;
+      }
+      ti = I * SB + i;
+      tj = I * SB + i + rem;
+      return;
+    }
+    t -= diag;
+    for (int J = I + 1; J < nb; ++J) {
+      const int c = (T - J * SB) < SB ? (T - J * SB) : SB;
+      const int cnt = r * c;
+      if (t < cnt) {
+        const int per_group = r * 4;
+        const int g = t / per_group;
+        const int gw = (c - g * 4) < 4 ? (c - g * 4) : 4;  // columns in this group
+        const int tg = t - g * per_group;
+        ti = I * SB + tg / gw;
+        tj = J * SB + g * 4 + tg % gw;
+        return;
+      }
+      t -= cnt;
+    }
+  }
+  ti = tj = 0;  // unreachable for t < T(T+1)/2
 }
 
 // Workgroup barrier preceded by the counter waits the software pipeline needs: every LDS read
@@ -140,6 +178,9 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
   // slot buf.  kt past the end re-fetches the last slab (never read): the refill count per stage
   // stays fixed, which is what the vmcnt bookkeeping in pipeline_barrier relies on.
   auto issue_load = [&](int kt, int buf, int j) {
+#ifdef DION_DBG_NO_LOADS
+    if (kt >= NSTAGE) return;
+#endif
     const int k = kt < KT ? kt : KT - 1;
     char* l = lds + buf * Cfg::STAGE_BYTES + wave * (64 * 16);
     if (j < Cfg::P_LOADS) {
@@ -208,6 +249,9 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
         if (last) pipeline_barrier<(NSTAGE - 2) * LPS>();  // slab kt+1 landed, slab kt fully read
 #pragma unroll
         for (int q = 0; q < NM; ++q) {
+#ifdef DION_DBG_NO_MFMA
+          if (q == 0)
+#endif
           acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
               fa[cur][q / TN], fb[cur][q % TN], acc[q / TN][q % TN], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
@@ -226,18 +270,27 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
       }
     }
   }
-  wait_vmcnt<0>();  // drain the redundant tail refills before the wave can exit
+  wait_vmcnt<0>();  // drain the redundant tail refills before LDS is reused / the wave exits
 
   // ---- epilogue.  Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4,
   // column l%32 of its 32x32 tile.  Whole tiles are stored: destinations are padded to the tile.
+  // C goes out straight from registers (32 lanes x 2 B = one 64-byte run per row).  The transposed
+  // copy would be 8-byte pieces scattered over 32 rows per instruction, so it is staged through
+  // LDS ([column][row], this wavefront's private slice) and stored as 16 bytes per lane with
+  // 256-byte runs per row.
   const float alpha = p.alpha, beta = p.beta;
-  const int row_base = ti * BM + wm * Cfg::WTM + 4 * fhalf;
-  const int col_base = tj * BN + wn * Cfg::WTN + frow;
+  const int row_base = ti * BM + wm * Cfg::WTM;
+  const int col_base = tj * BN + wn * Cfg::WTN;
   const bool mirror = HAS_CT && !(p.tri && ti == tj);  // a diagonal tile is its own mirror
-  const bf16_t* Dp = HAS_D ? p.D + (int64_t)b * p.strideD + (int64_t)row_base * p.ldd + col_base : nullptr;
-  bf16_t* Cp = HAS_C ? p.C + (int64_t)b * p.strideC + (int64_t)row_base * p.ldc + col_base : nullptr;
-  bf16_t* Ctp = HAS_CT ? p.Ct + (int64_t)b * p.strideCt + (int64_t)col_base * p.ldct + row_base : nullptr;
+  const bf16_t* Dp = HAS_D ? p.D + (int64_t)b * p.strideD + (int64_t)(row_base + 4 * fhalf) * p.ldd +
+                                 col_base + frow
+                           : nullptr;
+  bf16_t* Cp = HAS_C ? p.C + (int64_t)b * p.strideC + (int64_t)(row_base + 4 * fhalf) * p.ldc +
+                           col_base + frow
+                     : nullptr;
   const int ldd = p.ldd, ldc = p.ldc, ldct = p.ldct;
+  char* stg = lds + wave * Cfg::STG_BYTES;
+  if (HAS_CT) __syncthreads();  // every wavefront is done with the operand ring
 
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -260,15 +313,27 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
           Cp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldc + j * 32] = f32_to_bf16(v[r]);
       }
       if (HAS_CT) {
-        if (mirror) {
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            uint2 pk;
-            pk.x = pack_bf16x2(v[g * 4 + 0], v[g * 4 + 1]);
-            pk.y = pack_bf16x2(v[g * 4 + 2], v[g * 4 + 3]);
-            *(uint2*)(Ctp + (int64_t)(j * 32) * ldct + i * 32 + g * 8) = pk;
-          }
+        for (int g = 0; g < 4; ++g) {
+          uint2 pk;
+          pk.x = pack_bf16x2(v[g * 4 + 0], v[g * 4 + 1]);
+          pk.y = pack_bf16x2(v[g * 4 + 2], v[g * 4 + 3]);
+          *(uint2*)(stg + (j * 32 + frow) * Cfg::STG_PITCH + (i * 32 + g * 8 + 4 * fhalf) * 2) = pk;
         }
+      }
+    }
+  }
+  if (HAS_CT) {
+    if (mirror) {
+      constexpr int CH = Cfg::WTM / 8;  // 16-byte chunks per staged row
+      constexpr int RPI = 64 / CH;      // staged rows per store instruction
+      const int srow = lane / CH, schunk = lane % CH;
+      bf16_t* Ctp = p.Ct + (int64_t)b * p.strideCt + (int64_t)(col_base + srow) * ldct + row_base + schunk * 8;
+      const char* sp = stg + srow * Cfg::STG_PITCH + schunk * 16;
+#pragma unroll 8
+      for (int it = 0; it < Cfg::WTN / RPI; ++it) {
+        const uint4 q = *(const uint4*)(sp + it * RPI * Cfg::STG_PITCH);
+        *(uint4*)(Ctp + (int64_t)(it * RPI) * ldct) = q;
       }
     }
   }
@@ -278,6 +343,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
 typedef TileCfg<256, 256, 64, 2, 2, 2> Cfg256;
 typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg128;
 typedef TileCfg<256, 256, 32, 2, 2, 4> Cfg256k32;
+typedef TileCfg<256, 256, 64, 2, 4, 2> Cfg256w8;   // 8 wavefronts, 128x64 each: two per SIMD
+typedef TileCfg<256, 256, 64, 4, 2, 2> Cfg256w8b;  // 8 wavefronts, 64x128 each
 
 template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT>
 static hipError_t launch_epi(const GemmParams& p, hipStream_t stream) {
@@ -320,12 +387,22 @@ int gemm_pad_granule(int m, int n, int batch) {
 
 hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.batch <= 0) return hipSuccess;
-  if (variant < 0) variant = (p.M % 256 == 0 && p.N % 256 == 0) ? 0 : 1;
+  if (variant < 0) {
+    variant = (p.M % 256 == 0 && p.N % 256 == 0) ? 3 : 1;
+    // Tuning knob: DION_GEMM_VARIANT overrides the 256-wide tile configuration.
+    static const int forced = [] {
+      const char* e = getenv("DION_GEMM_VARIANT");
+      return e ? atoi(e) : -1;
+    }();
+    if (forced >= 0 && variant == 3) variant = forced;
+  }
   if (p.tri && (p.M != p.N)) return hipErrorInvalidValue;
   switch (variant) {
     case 0: return launch_cfg<Cfg256>(p, stream);
     case 1: return launch_cfg<Cfg128>(p, stream);
     case 2: return launch_cfg<Cfg256k32>(p, stream);
+    case 3: return launch_cfg<Cfg256w8>(p, stream);
+    case 4: return launch_cfg<Cfg256w8b>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }
