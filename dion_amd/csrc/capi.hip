@@ -148,9 +148,9 @@ NsPlan make_plan(int batch, int rows, int cols, int flags) {
   pl.mp = round_up(pl.m, g);
   pl.np = round_up(pl.n, g);
   const int64_t numel = (int64_t)rows * cols;
-  int64_t nb = numel / (256 * 16);
+  int64_t nb = numel / (256 * 32);
   if (nb < 1) nb = 1;
-  if (nb > 256) nb = 256;
+  if (nb > 1024) nb = 1024;
   pl.nblk = (int)nb;
   pl.ldx = pl.np + ld_pad();
   pl.ldxt = pl.mp + ld_pad();

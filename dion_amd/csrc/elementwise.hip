@@ -38,20 +38,53 @@ __device__ __forceinline__ float load_as_bf16_f32<float>(const float* p, int64_t
 // ------------------------------------------------------------------------------------------
 // Frobenius pre-normalisation:  partial sums of squares of bf16(in), then 1/(||.||*s + eps).
 // ------------------------------------------------------------------------------------------
+// 8 consecutive elements of `p` (16-byte aligned chunk index i) as bf16-rounded floats.
 template <typename T>
+static __device__ __forceinline__ void load8_as_bf16(const T* p, int64_t i, float v[8]) {
+  if (sizeof(T) == 2) {
+    const uint4 raw = ((const uint4*)p)[i];
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[2 * e] = __uint_as_float(w[e] << 16);
+      v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+    }
+  } else {
+    const float4 a = ((const float4*)p)[2 * i], c = ((const float4*)p)[2 * i + 1];
+    const float f[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = bf16_to_f32(f32_to_bf16(f[e]));
+  }
+}
+
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void sumsq_partial_kernel(const T* __restrict__ in, int64_t numel,
                                                             int nblk, float* __restrict__ partial) {
   __shared__ float red[16];
   const int b = blockIdx.y;
   const T* src = in + (int64_t)b * numel;
-  const int64_t per = (numel + nblk - 1) / nblk;
-  const int64_t lo = (int64_t)blockIdx.x * per;
-  int64_t hi = lo + per;
-  if (hi > numel) hi = numel;
   float s = 0.f;
-  for (int64_t i = lo + threadIdx.x; i < hi; i += 256) {
-    const float v = load_as_bf16_f32<T>(src, i);
-    s += v * v;
+  if (VEC) {
+    const int64_t nv = numel >> 3;
+    const int64_t per = (nv + nblk - 1) / nblk;
+    const int64_t lo = (int64_t)blockIdx.x * per;
+    int64_t hi = lo + per;
+    if (hi > nv) hi = nv;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += 256) {
+      float v[8];
+      load8_as_bf16<T>(src, i, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += v[e] * v[e];
+    }
+  } else {
+    const int64_t per = (numel + nblk - 1) / nblk;
+    const int64_t lo = (int64_t)blockIdx.x * per;
+    int64_t hi = lo + per;
+    if (hi > numel) hi = numel;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += 256) {
+      const float v = load_as_bf16_f32<T>(src, i);
+      s += v * v;
+    }
   }
   s = block_sum(s, red);
   if (threadIdx.x == 0) partial[(int64_t)b * nblk + blockIdx.x] = s;
@@ -100,6 +133,51 @@ __global__ __launch_bounds__(256) void ns_prepare_kernel(const T* __restrict__ i
   }
 }
 
+// Same operation, 16-byte accesses: needs C % 8 == 0, 16-byte aligned input and row pitches.
+template <typename T>
+__global__ __launch_bounds__(256) void ns_prepare_vec_kernel(const T* __restrict__ in, int R, int C,
+                                                             const float* __restrict__ inv_norm,
+                                                             bf16_t* __restrict__ same, int ld_same,
+                                                             int64_t stride_same,
+                                                             bf16_t* __restrict__ trans, int ld_trans,
+                                                             int64_t stride_trans) {
+  __shared__ __attribute__((aligned(16))) bf16_t tile[64][72];
+  const int b = blockIdx.z;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const float sc = inv_norm[b];
+  const T* src = in + (int64_t)b * R * C;
+  bf16_t* ds = same + (int64_t)b * stride_same;
+  bf16_t* dt = trans + (int64_t)b * stride_trans;
+  const int chunk = threadIdx.x & 7, rr = threadIdx.x >> 3;  // 8 chunks x 32 rows per pass
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int i = rr + pass * 32;
+    const int r = r0 + i, c = c0 + chunk * 8;
+    uint4 o = make_uint4(0, 0, 0, 0);
+    if (r < R && c < C) {
+      float v[8];
+      load8_as_bf16<T>(src, ((int64_t)r * C + c) >> 3, v);
+      o.x = pack_bf16x2(v[0] * sc, v[1] * sc);
+      o.y = pack_bf16x2(v[2] * sc, v[3] * sc);
+      o.z = pack_bf16x2(v[4] * sc, v[5] * sc);
+      o.w = pack_bf16x2(v[6] * sc, v[7] * sc);
+    }
+    *(uint4*)&tile[i][chunk * 8] = o;
+    *(uint4*)(ds + (int64_t)r * ld_same + c) = o;
+  }
+  __syncthreads();
+  // transposed: thread -> (trans row = column rr + 32*pass of the tile, 8 consecutive source rows)
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int col = rr + pass * 32;
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      w[e] = (uint32_t)tile[chunk * 8 + 2 * e][col] | ((uint32_t)tile[chunk * 8 + 2 * e + 1][col] << 16);
+    *(uint4*)(dt + (int64_t)(c0 + col) * ld_trans + r0 + chunk * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
 // Dense [B,R,C] <- padded [B,*,ld] (drops padding).
 __global__ __launch_bounds__(256) void unpad_kernel(const bf16_t* __restrict__ src, int64_t src_stride,
                                                     int ld, bf16_t* __restrict__ dst, int R, int C) {
@@ -113,12 +191,16 @@ __global__ __launch_bounds__(256) void unpad_kernel(const bf16_t* __restrict__ s
 hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t numel,
                                 float norm_scale, float eps, float* partial, int nblk,
                                 float* inv_norm, hipStream_t st) {
-  if (in_dtype == 0)
-    hipLaunchKernelGGL(sumsq_partial_kernel<bf16_t>, dim3(nblk, batch), dim3(256), 0, st,
-                       (const bf16_t*)in, numel, nblk, partial);
-  else
-    hipLaunchKernelGGL(sumsq_partial_kernel<float>, dim3(nblk, batch), dim3(256), 0, st,
-                       (const float*)in, numel, nblk, partial);
+  const bool vec = (numel % 8 == 0) && (((uintptr_t)in) & 15) == 0;
+#define SUMSQ_LAUNCH(T, V)                                                                      \
+  hipLaunchKernelGGL((sumsq_partial_kernel<T, V>), dim3(nblk, batch), dim3(256), 0, st, (const T*)in, \
+                     numel, nblk, partial)
+  if (in_dtype == 0) {
+    if (vec) SUMSQ_LAUNCH(bf16_t, true); else SUMSQ_LAUNCH(bf16_t, false);
+  } else {
+    if (vec) SUMSQ_LAUNCH(float, true); else SUMSQ_LAUNCH(float, false);
+  }
+#undef SUMSQ_LAUNCH
   hipLaunchKernelGGL(norm_finalize_kernel, dim3(batch), dim3(64), 0, st, partial, nblk, norm_scale,
                      eps, inv_norm);
   return hipGetLastError();
@@ -129,6 +211,18 @@ hipError_t launch_ns_prepare(const void* in, int in_dtype, int batch, int R, int
                              int64_t stride_same, bf16_t* trans, int ld_trans, int64_t stride_trans,
                              hipStream_t st) {
   dim3 grid(Cp / 64, Rp / 64, batch);
+  const bool vec = (C % 8 == 0) && (((uintptr_t)in) & 15) == 0 && (ld_same % 8 == 0) &&
+                   (ld_trans % 8 == 0) && (stride_same % 8 == 0) && (stride_trans % 8 == 0) &&
+                   (((uintptr_t)same) & 15) == 0 && (((uintptr_t)trans) & 15) == 0;
+  if (vec) {
+    if (in_dtype == 0)
+      hipLaunchKernelGGL(ns_prepare_vec_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)in, R, C,
+                         inv_norm, same, ld_same, stride_same, trans, ld_trans, stride_trans);
+    else
+      hipLaunchKernelGGL(ns_prepare_vec_kernel<float>, grid, dim3(256), 0, st, (const float*)in, R, C,
+                         inv_norm, same, ld_same, stride_same, trans, ld_trans, stride_trans);
+    return hipGetLastError();
+  }
   if (in_dtype == 0)
     hipLaunchKernelGGL(ns_prepare_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)in, R, C,
                        inv_norm, same, Rp, Cp, ld_same, stride_same, trans, ld_trans, stride_trans);
