@@ -114,6 +114,9 @@ extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void
   p.tri = 0;
   p.alpha = 1.0f;
   p.beta = a;
+#ifdef DION_DBG_EPILOGUE
+  if (getenv("DION_DBG_NOD")) p.D = nullptr;
+#endif
   HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_3");
   return DION_OK;
 }
@@ -250,24 +253,21 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     p.tri = 1;
     p.alpha = c;
     p.beta = b;
-    HIP_TRY(launch_gemm_nt(p, -1, st), "B = c A A + b A");
-    // X' = a X + B X   (and its transpose)
+    p.diag = a;  // a*I folded into B: the next GEMM needs no addend (one fewer pass over X)
+    HIP_TRY(launch_gemm_nt(p, -1, st), "B = c A A + b A + a I");
+    // X' = (c A A + b A + a I) X   (and its transpose)
     memset(&p, 0, sizeof(p));
     p.P = Bm;
     p.Q = Xt[cur];
-    p.D = X[cur];
     p.strideP = sA;
     p.strideQ = sXt;
-    p.strideD = sX;
     p.ldp = lda;
     p.ldq = ldxt;
-    p.ldd = ldx;
     p.M = p.Mst = mp;
     p.N = p.Nst = np;
     p.K = mp;
     p.batch = batch;
     p.alpha = 1.0f;
-    p.beta = a;
     const bool last = (it == n_iters - 1);
     if (last && direct) {
       if (pl.tall) {
@@ -287,7 +287,7 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
       p.ldc = ldx;
       p.ldct = ldxt;
     }
-    HIP_TRY(launch_gemm_nt(p, -1, st), "X = a X + B X");
+    HIP_TRY(launch_gemm_nt(p, -1, st), "X = B X");
     cur ^= 1;
   }
   if (!(direct && n_iters > 0)) {

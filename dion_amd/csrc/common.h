@@ -47,6 +47,7 @@ struct GemmParams {
   int batch;
   int tri;           // 1: Q == P, only tiles with tile_row <= tile_col are computed, Ct mirrors
   float alpha, beta;
+  float diag;        // added to C[i][i] (global diagonal); used with tri to fold a*I into B
 };
 
 // Returns hipSuccess or the launch error.  variant < 0 picks by shape.

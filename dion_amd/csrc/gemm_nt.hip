@@ -3,8 +3,8 @@
 // Every GEMM of the Newton-Schulz / Polar-Express iteration is expressed in this one form, with
 // both operands contiguous along the reduction dimension, by carrying X and X^T side by side:
 //   A  = X X^T                     P = Q = X            (tri: upper tiles + mirrored store)
-//   B  = c A A + b A               P = Q = A (A = A^T)  (tri, D = A)
-//   X' = a X + B X                 P = B, Q = X^T, D = X, stores X' and (X')^T
+//   B  = c A A + b A + a I         P = Q = A (A = A^T)  (tri, D = A, a on the diagonal)
+//   X' = B X  (= a X + (B - aI) X)  P = B, Q = X^T, stores X' and (X')^T
 // This replaces the reference's ns_line_1 / ns_line_2 / ns_line_3
 // (dion/newton_schulz_triton.py:88-157, :206-287, :384-447) and the baddbmm of
 // dion/newton_schulz_triton.py:557-563.
@@ -290,6 +290,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
                      : nullptr;
   const int ldd = p.ldd, ldc = p.ldc, ldct = p.ldct;
   char* stg = lds + wave * Cfg::STG_BYTES;
+  const bool on_diag = p.tri && ti == tj && p.diag != 0.0f;
   if (HAS_CT) __syncthreads();  // every wavefront is done with the operand ring
 
 #pragma unroll
@@ -306,6 +307,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
           d[r] = Dp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldd + j * 32];
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] += beta * bf16_to_f32(d[r]);
+      }
+      if (on_diag) {
+        // element (row, col) of this 32x32 tile sits on the global diagonal
+        const int dcol = col_base + j * 32 + frow - (row_base + i * 32 + 4 * fhalf);
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (dcol == (r >> 2) * 8 + (r & 3)) v[r] += p.diag;
       }
       if (HAS_C) {
 #pragma unroll
@@ -374,6 +382,7 @@ static hipError_t launch_cfg(const GemmParams& p, hipStream_t stream) {
   if (d && c && !ct) return launch_epi<Cfg, true, true, false>(p, stream);   // last X'
   if (d && !c && ct) return launch_epi<Cfg, true, false, true>(p, stream);   // last (X')^T
   if (!d && c && !ct) return launch_epi<Cfg, false, true, false>(p, stream); // plain product
+  if (!d && !c && ct) return launch_epi<Cfg, false, false, true>(p, stream); // transposed product
   return hipErrorInvalidValue;
 }
 
