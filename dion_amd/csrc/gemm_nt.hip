@@ -397,7 +397,14 @@ int gemm_pad_granule(int m, int n, int batch) {
 hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.batch <= 0) return hipSuccess;
   if (variant < 0) {
-    variant = (p.M % 256 == 0 && p.N % 256 == 0) ? 3 : 1;
+    // 256-wide tiles only when there are enough of them to keep 256 CUs busy for a few rounds;
+    // below that the 128-wide tiles (two workgroups per CU) win.
+    static const long thresh = [] {
+      const char* e = getenv("DION_TILE_THRESH");
+      return e ? atol(e) : 512L;
+    }();
+    const long t256 = (long)(p.M / 256) * (p.tri ? (p.M / 256 + 1) / 2 + 0 : p.N / 256) * p.batch;
+    variant = (p.M % 256 == 0 && p.N % 256 == 0 && t256 >= thresh) ? 3 : 1;
     // Tuning knob: DION_GEMM_VARIANT overrides the 256-wide tile configuration.
     static const int forced = [] {
       const char* e = getenv("DION_GEMM_VARIANT");

@@ -248,6 +248,7 @@ class OrthoOptimizer(Optimizer):
             else:
                 raise ValueError(f"Unknown algorithm: {algo}")
 
+        work: List[Tuple[dict, List[Tensor]]] = []
         for group in ortho:
             assert all(p.ndim >= 2 for p in group["params"]), (
                 f"{type(self).__name__} optimizer only supports matrix parameters."
@@ -259,7 +260,8 @@ class OrthoOptimizer(Optimizer):
             for p in with_grad:
                 buckets[(p.shape, p.dtype)].append(p)
             for params in buckets.values():
-                self._update_shape_group(group, params)
+                work.append((group, params))
+        self._run_shape_groups(work)
 
         for group in lion:
             scalar_opts.lion_step(self, group)
@@ -269,6 +271,51 @@ class OrthoOptimizer(Optimizer):
 
     def _update_shape_group(self, group: dict, params: List[Tensor]) -> None:
         raise NotImplementedError
+
+    # Shape groups are independent.  A group whose GEMMs cannot fill the GPU on their own (a few
+    # hundred tiles) is run on one of a handful of side streams so that several such groups
+    # overlap; large groups run one after another on the caller's stream.  The reference reaches
+    # the same goal by interleaving up to three generator tasks (dion/megabatch_base.py:193).
+    _SMALL_GROUP_FLOP = 4e12
+    _N_SIDE_STREAMS = 4
+
+    @staticmethod
+    def _group_flop(params: List[Tensor]) -> float:
+        r, c = params[0].shape[-2], params[0].shape[-1]
+        m, n = min(r, c), max(r, c)
+        mats = len(params) * (params[0].numel() // (r * c))
+        return mats * 5.0 * (4.0 * m * m * n + 2.0 * m ** 3)
+
+    def _run_shape_groups(self, work: List[Tuple[dict, List[Tensor]]]) -> None:
+        if not work:
+            return
+        on_gpu = all(params[0].is_cuda for _g, params in work)
+        small = [w for w in work if self._group_flop(w[1]) < self._SMALL_GROUP_FLOP] if on_gpu else []
+        if len(small) < 2:
+            for group, params in work:
+                self._update_shape_group(group, params)
+            return
+        big = [w for w in work if self._group_flop(w[1]) >= self._SMALL_GROUP_FLOP]
+        for group, params in big:
+            self._update_shape_group(group, params)
+        device = small[0][1][0].device
+        streams = self.__dict__.setdefault("_side_streams", {})
+        pool = streams.get(device)
+        if pool is None:
+            pool = [torch.cuda.Stream(device=device) for _ in range(self._N_SIDE_STREAMS)]
+            streams[device] = pool
+        main = torch.cuda.current_stream(device)
+        fork = main.record_event()
+        used = []
+        for i, (group, params) in enumerate(small):
+            side = pool[i % len(pool)]
+            if side not in used:
+                side.wait_event(fork)
+                used.append(side)
+            with torch.cuda.stream(side):
+                self._update_shape_group(group, params)
+        for side in used:
+            main.wait_stream(side)
 
     # ---------------------------------------------------- orthogonalization
     def _orthogonalize(self, U: Tensor, epsilon: float) -> Tensor:
