@@ -7,6 +7,7 @@ from .newton_schulz import (  # noqa: F401
     ns_line_3,
     polar_express,
     polar_express_triton,
+    zeropower_kj,
     zeropower_via_newtonschulz5,
 )
 
@@ -23,5 +24,6 @@ __all__ = [
     "ns_line_3",
     "polar_express",
     "polar_express_triton",
+    "zeropower_kj",
     "zeropower_via_newtonschulz5",
 ]

@@ -188,8 +188,6 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   if (!in || !out || (n_iters > 0 && !coeffs))
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: null argument");
   if (flags & ~DION_NS_GRAM) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
-  if (flags & DION_NS_GRAM) return fail(DION_E_INVALID, "dion_ns_orthogonalize: Gram recurrence not built");
-  (void)gram_reset;
   const NsPlan pl = make_plan(batch, rows, cols, flags);
   if (!workspace || workspace_bytes < pl.total)
     return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize: workspace %zu < %zu bytes", workspace_bytes,
@@ -205,8 +203,11 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   X[1] = (bf16_t*)w; w += pl.x_bytes;
   Xt[0] = (bf16_t*)w; w += pl.x_bytes;
   Xt[1] = (bf16_t*)w; w += pl.x_bytes;
-  bf16_t* A = (bf16_t*)w; w += pl.a_bytes;
-  bf16_t* Bm = (bf16_t*)w; w += pl.a_bytes;
+  bf16_t* sq[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};  // m x m scratch
+  for (int i = 0; i < ((flags & DION_NS_GRAM) ? 6 : 2); ++i) {
+    sq[i] = (bf16_t*)w;
+    w += pl.a_bytes;
+  }
   float* partial = (float*)w; w += pl.partial_bytes;
   float* inv = (float*)w; w += pl.inv_bytes;
 
@@ -224,14 +225,38 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
             "prepare");
 
   const bool direct = (mp == pl.m && np == pl.n);
-  int cur = 0;
-  for (int it = 0; it < n_iters; ++it) {
-    const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
+
+  // ---- the four GEMM shapes of the iteration, all through launch_gemm_nt
+  // sym(P, Q -> C): C = alpha P Q^T + beta D + diag I for symmetric m x m operands whose product
+  // is symmetric; upper tiles computed, mirrored on store.
+  // With tri == false the whole product is computed: needed when symmetry of the result rests on
+  // the (bf16-rounded, hence only approximate) commutation of P and Q -- mirroring such a product
+  // plants a commutator-sized error.
+  auto sym = [&](const bf16_t* P, const bf16_t* Q, const bf16_t* D, bf16_t* C, float alpha, float beta,
+                 float diag, bool tri = true) -> hipError_t {
     GemmParams p;
-    // A = X X^T
     memset(&p, 0, sizeof(p));
-    p.P = p.Q = X[cur];
-    p.C = p.Ct = A;
+    p.P = P;
+    p.Q = Q;
+    p.D = D;
+    p.C = C;
+    p.Ct = tri ? C : nullptr;
+    p.strideP = p.strideQ = p.strideD = p.strideC = p.strideCt = sA;
+    p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = lda;
+    p.M = p.N = p.K = p.Mst = p.Nst = mp;
+    p.batch = batch;
+    p.tri = tri ? 1 : 0;
+    p.alpha = alpha;
+    p.beta = beta;
+    p.diag = diag;
+    return launch_gemm_nt(p, -1, st);
+  };
+  // gram(Xc -> R): R = Xc Xc^T
+  auto gram = [&](const bf16_t* Xc, bf16_t* R) -> hipError_t {
+    GemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.P = p.Q = Xc;
+    p.C = p.Ct = R;
     p.strideP = p.strideQ = sX;
     p.strideC = p.strideCt = sA;
     p.ldp = p.ldq = ldx;
@@ -241,24 +266,15 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     p.batch = batch;
     p.tri = 1;
     p.alpha = 1.0f;
-    HIP_TRY(launch_gemm_nt(p, -1, st), "A = X X^T");
-    // B = c A A + b A
+    return launch_gemm_nt(p, -1, st);
+  };
+  // apply(S, Xtc -> Xn, Xtn | out): X' = S X given X^T (S symmetric m x m).  `final` writes the
+  // caller's tensor in its own orientation when no padding is in the way.
+  auto apply = [&](const bf16_t* S, const bf16_t* Xtc, bf16_t* Xn, bf16_t* Xtn, bool final_direct) -> hipError_t {
+    GemmParams p;
     memset(&p, 0, sizeof(p));
-    p.P = p.Q = p.D = A;
-    p.C = p.Ct = Bm;
-    p.strideP = p.strideQ = p.strideD = p.strideC = p.strideCt = sA;
-    p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = lda;
-    p.M = p.N = p.K = p.Mst = p.Nst = mp;
-    p.batch = batch;
-    p.tri = 1;
-    p.alpha = c;
-    p.beta = b;
-    p.diag = a;  // a*I folded into B: the next GEMM needs no addend (one fewer pass over X)
-    HIP_TRY(launch_gemm_nt(p, -1, st), "B = c A A + b A + a I");
-    // X' = (c A A + b A + a I) X   (and its transpose)
-    memset(&p, 0, sizeof(p));
-    p.P = Bm;
-    p.Q = Xt[cur];
+    p.P = S;
+    p.Q = Xtc;
     p.strideP = sA;
     p.strideQ = sXt;
     p.ldp = lda;
@@ -268,8 +284,7 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     p.K = mp;
     p.batch = batch;
     p.alpha = 1.0f;
-    const bool last = (it == n_iters - 1);
-    if (last && direct) {
+    if (final_direct) {
       if (pl.tall) {
         p.Ct = (bf16_t*)out;
         p.strideCt = (int64_t)mp * np;
@@ -280,17 +295,83 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
         p.ldc = np;
       }
     } else {
-      p.C = X[cur ^ 1];
-      p.Ct = Xt[cur ^ 1];
+      p.C = Xn;
+      p.Ct = Xtn;
       p.strideC = sX;
       p.strideCt = sXt;
       p.ldc = ldx;
       p.ldct = ldxt;
     }
-    HIP_TRY(launch_gemm_nt(p, -1, st), "X = B X");
-    cur ^= 1;
+    return launch_gemm_nt(p, -1, st);
+  };
+
+  int cur = 0;
+  bool wrote_out = false;
+  if (!(flags & DION_NS_GRAM)) {
+    for (int it = 0; it < n_iters; ++it) {
+      const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
+      HIP_TRY(gram(X[cur], sq[0]), "A = X X^T");
+      // a*I folded into B: the next GEMM needs no addend (one fewer pass over X)
+      HIP_TRY(sym(sq[0], sq[0], sq[0], sq[1], c, b, a), "B = c A A + b A + a I");
+      const bool fin = (it == n_iters - 1) && direct;
+      HIP_TRY(apply(sq[1], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], fin), "X = B X");
+      wrote_out = fin;
+      cur ^= 1;
+    }
+  } else {
+    // Gram recurrence: R = X X^T and Q with X_t = Q X_0 live in m x m; per iteration
+    // Z = a I + b R + c R^2, Q <- Z Q, R <- Z R Z (all symmetric and commuting).  At the restart
+    // iteration X is materialised, R recomputed from it and Q reset, which bounds the bf16 drift
+    // of the R recurrence.  The rectangular work drops from 10 GEMMs to 2 Gram + 2 apply.
+    bool used[6] = {false, false, false, false, false, false};
+    auto take = [&]() -> int {
+      for (int i = 0; i < 6; ++i)
+        if (!used[i]) {
+          used[i] = true;
+          return i;
+        }
+      return -1;
+    };
+    int r = take(), q = -1;
+    HIP_TRY(gram(X[cur], sq[r]), "R = X X^T");
+    for (int it = 0; it < n_iters; ++it) {
+      const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
+      if (it == gram_reset && it > 0 && q >= 0) {
+        HIP_TRY(apply(sq[q], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], false), "X = Q X (restart)");
+        cur ^= 1;
+        used[q] = false;
+        q = -1;
+        HIP_TRY(gram(X[cur], sq[r]), "R = X X^T (restart)");
+      }
+      const int z = take();
+      HIP_TRY(sym(sq[r], sq[r], sq[r], sq[z], c, b, a), "Z = a I + b R + c R R");
+      const bool need_r = !(it == n_iters - 1 || (it + 1 == gram_reset));
+      if (need_r) {
+        const int t = take();
+        HIP_TRY(sym(sq[z], sq[r], nullptr, sq[t], 1.0f, 0.0f, 0.0f, false), "T = Z R");
+        const int rn = take();
+        HIP_TRY(sym(sq[t], sq[z], nullptr, sq[rn], 1.0f, 0.0f, 0.0f), "R = T Z");
+        used[t] = false;
+        used[r] = false;
+        r = rn;
+      }
+      if (q < 0) {
+        q = z;  // Q = Z (Q was the identity)
+      } else {
+        const int qn = take();
+        HIP_TRY(sym(sq[z], sq[q], nullptr, sq[qn], 1.0f, 0.0f, 0.0f, false), "Q = Z Q");
+        used[q] = false;
+        used[z] = false;
+        q = qn;
+      }
+    }
+    if (q >= 0) {
+      HIP_TRY(apply(sq[q], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], direct), "X = Q X");
+      wrote_out = direct;
+      cur ^= 1;
+    }
   }
-  if (!(direct && n_iters > 0)) {
+  if (!wrote_out) {
     if (pl.tall)
       HIP_TRY(launch_unpad(Xt[cur], sXt, ldxt, (bf16_t*)out, batch, rows, cols, st), "unpad");
     else

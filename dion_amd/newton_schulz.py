@@ -29,6 +29,8 @@ POLAR_EXPRESS_COEFFS: Sequence[Tuple[float, float, float]] = (
     (2.3465413258596377, -1.7097828382687081, 0.42323551169305323),
 )
 POLAR_EXPRESS_SAFETY = 1.02  # dion/polar_express.py:35
+# dion/muon_reference.py:16 (Keller Jordan's fixed quintic)
+KJ_COEFFS: Tuple[float, float, float] = (3.4445, -4.7750, 2.0315)
 
 
 def _eps(epsilon: Union[float, Tensor, None], default: float) -> float:
@@ -58,6 +60,14 @@ def gram_newton_schulz(G: Tensor, epsilon: Union[float, Tensor, None] = None) ->
     """Gram-matrix recurrence with the Polar-Express schedule and a restart at iteration 2
     (how dion/megabatch_base.py:77-94 configures the external package; epsilon is ignored there)."""
     return ops.ns_orthogonalize(G, POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 0.0, gram=True, gram_reset=2)
+
+
+@torch.no_grad()
+def zeropower_kj(G: Tensor, steps: int = 5, eps: Union[float, Tensor] = 1e-7) -> Tensor:
+    """Fixed-coefficient Newton-Schulz of the reference's un-batched Muon
+    (``muon_reference.zeropower_via_newtonschulz5``, dion/muon_reference.py:11-27): ``steps``
+    iterations of (3.4445, -4.7750, 2.0315) after ``X / (||X||_F + eps)``."""
+    return ops.ns_orthogonalize(G, [KJ_COEFFS] * int(steps), 1.0, _eps(eps, 1e-7))
 
 
 # The reference exposes Triton-backed twins of the two schedules; here there is one

@@ -224,3 +224,66 @@ def test_int64_batch_offsets():
     ref = ns_line_1(last)
     assert torch.equal(out[-1], ref)
     assert float(out[:-1].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("shape", [(64, 128), (128, 64), (4, 256, 1024), (2, 768, 3072), (2, 3072, 768), (3, 100, 36)])
+def test_gram_newton_schulz(shape):
+    """Gram-matrix recurrence (restart at iteration 2): same odd polynomial as Polar-Express, so
+    it is held to the exact-arithmetic result of the standard iteration.  In bf16 the m x m
+    recurrence is more sensitive to conditioning than the standard form: within 2e-2 for aspect
+    ratios >= 3, and never further from exact than 1.3x the reference's eager bf16 Polar-Express
+    path is (3-6e-2 for aspect <= 2).  Parity against the external gram-newton-schulz package is
+    unpinned (not in the reference tree, not installed)."""
+    from dion_amd import gram_newton_schulz, polar_express
+
+    torch.manual_seed(42)
+    G = torch.randn(shape)
+    out = gram_newton_schulz(G.to(DEV))
+    assert out.dtype == torch.bfloat16 and out.shape == G.shape
+    out_np = out.float().cpu().numpy().astype(np.float64)
+    ref64 = oracle.ns_fp64(G.numpy(), oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 0.0)
+    gram64 = oracle.gram_ns_fp64(G.numpy(), oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 0.0, (2,))
+    assert _np_rel(gram64, ref64) < 1e-9
+    eager = oracle.polar_express_bf16(G, eps=0.0).float().numpy().astype(np.float64)
+    aspect = max(shape[-2:]) / min(shape[-2:])
+    e_gram = _np_rel(out_np, ref64)
+    assert e_gram <= (2e-2 if aspect >= 3 else 1.3 * _np_rel(eager, ref64)), e_gram
+    std = polar_express(G.to(DEV), 0.0).float().cpu().numpy().astype(np.float64)
+    assert _np_rel(out_np, std) <= e_gram + _np_rel(std, ref64) + 1e-6
+    P = out.float() @ out.float().mT if shape[-2] <= shape[-1] else out.float().mT @ out.float()
+    eye = torch.eye(P.shape[-1], device=DEV).expand_as(P)
+    assert float((P - eye).abs().max()) < (0.15 if aspect >= 3 else 0.3)
+
+
+def test_gram_square_matrices_stay_in_band():
+    """Square inputs are the ill-conditioned case of the Gram form; the restart keeps the result
+    within the band the reference's own bf16 paths occupy."""
+    from dion_amd import gram_newton_schulz
+
+    torch.manual_seed(3)
+    G = torch.randn(2, 512, 512)
+    out = gram_newton_schulz(G.to(DEV)).float().cpu().numpy().astype(np.float64)
+    ref64 = oracle.ns_fp64(G.numpy(), oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 0.0)
+    eager = oracle.polar_express_bf16(G, eps=0.0).float().numpy().astype(np.float64)
+    assert _np_rel(out, ref64) <= max(6.5e-2, 1.5 * _np_rel(eager, ref64))
+
+
+@pytest.mark.parametrize("shape", [(768, 3072), (3072, 768), (96, 192)])
+def test_kj_newton_schulz_vs_oracle(shape):
+    """Single-matrix Muon NS with the fixed coefficients (BASELINE config 1:
+    dion/muon_reference.py:11-27)."""
+    from dion_amd import zeropower_kj
+
+    torch.manual_seed(11)
+    G = torch.randn(shape)
+    out = zeropower_kj(G.to(DEV), steps=5, eps=1e-7)
+    ref = oracle.kj_ns_bf16(G, 5, 1e-7).float().numpy().astype(np.float64)
+    ref64 = oracle.ns_fp64(G.numpy(), oracle.KJ_COEFFS, 1.0, 1e-7)
+    out_np = out.float().cpu().numpy().astype(np.float64)
+    # The fixed quintic never settles at 1 (it oscillates in [0.68, 1.16]), so bf16 paths drift
+    # apart like Polar-Express: the reference's eager path is itself 2.3-2.7e-2 from exact here.
+    e_hip, e_ref = _np_rel(out_np, ref64), _np_rel(ref, ref64)
+    assert e_hip <= 2e-2 and e_hip <= e_ref
+    assert _np_rel(out_np, ref) <= 2e-2 + e_ref
+    sv = np.linalg.svd(out.float().cpu().numpy().astype(np.float64), compute_uv=False)
+    assert 0.6 < sv.min() and sv.max() < 1.2  # KJ band [0.68, 1.16] with bf16 slack

@@ -289,3 +289,24 @@ def test_mixed_param_groups():
     opt.step()
     for t, t0 in zip(w + b + e, before):
         assert not torch.equal(t.data, t0) and torch.isfinite(t.data).all()
+
+
+def test_gram_flag_runs_and_tracks_standard():
+    """use_gram_newton_schulz=True selects the Gram recurrence (reference call site
+    dion/megabatch_base.py:77-94); on wide matrices the step stays close to the Polar-Express one."""
+    from dion import Muon
+
+    pa = _make_params([(128, 512)] * 2)
+    pb = _make_params([(128, 512)] * 2)
+    oa = Muon(pa, lr=0.01, use_gram_newton_schulz=True)
+    ob = Muon(pb, lr=0.01, use_polar_express=True)
+    for step in range(2):
+        torch.manual_seed(100 + step)
+        for a, b in zip(pa, pb):
+            g = torch.randn_like(a)
+            a.grad = g.clone()
+            b.grad = g.clone()
+        oa.step()
+        ob.step()
+    for a, b in zip(pa, pb):
+        assert _rel(a.data, b.data) < 1e-3
