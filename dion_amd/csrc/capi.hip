@@ -188,13 +188,24 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   if (!in || !out || (n_iters > 0 && !coeffs))
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: null argument");
   if (flags & ~DION_NS_GRAM) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
+  hipStream_t st = (hipStream_t)stream;
+  if (!(flags & DION_NS_GRAM) && n_iters <= kMaxSmallIters && ns_small_fits(rows, cols) &&
+      !getenv("DION_NO_SMALL_KERNEL")) {
+    // per-head regime: whole iteration resident in LDS, one workgroup per matrix, no workspace
+    NsCoeffs co;
+    memset(&co, 0, sizeof(co));
+    co.n = n_iters;
+    for (int i = 0; i < n_iters * 3; ++i) co.c[i / 3][i % 3] = coeffs[i];
+    HIP_TRY(launch_ns_small(in, in_dtype, (bf16_t*)out, batch, rows, cols, co, norm_scale, eps, st),
+            "small-matrix Newton-Schulz");
+    return DION_OK;
+  }
   const NsPlan pl = make_plan(batch, rows, cols, flags);
   if (!workspace || workspace_bytes < pl.total)
     return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize: workspace %zu < %zu bytes", workspace_bytes,
                 pl.total);
   if (((uintptr_t)workspace & 255) != 0)
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: workspace not 256-byte aligned");
-  hipStream_t st = (hipStream_t)stream;
 
   char* w = (char*)workspace;
   bf16_t* X[2];

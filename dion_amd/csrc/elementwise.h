@@ -12,6 +12,17 @@ struct PtrTab {
   uint64_t p[kMaxPtrs];
 };
 
+// Coefficient schedule passed by value to the LDS-resident small-matrix kernel.
+constexpr int kMaxSmallIters = 8;
+struct NsCoeffs {
+  int n;
+  float c[kMaxSmallIters][3];
+};
+// True when a rows x cols matrix (short side <= 64) fits the one-workgroup-per-matrix kernel.
+bool ns_small_fits(int rows, int cols);
+hipError_t launch_ns_small(const void* in, int in_dtype, bf16_t* out, int batch, int rows, int cols,
+                           const NsCoeffs& co, float norm_scale, float eps, hipStream_t st);
+
 hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t numel,
                                 float norm_scale, float eps, float* partial, int nblk,
                                 float* inv_norm, hipStream_t st);

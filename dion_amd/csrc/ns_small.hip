@@ -1,0 +1,285 @@
+// Whole Newton-Schulz / Polar-Express orthogonalization of one small matrix per workgroup, resident
+// in LDS from the Frobenius normalisation to the last iteration: the per-head regime (e.g. 64 x 768
+// attention heads), where the general path is 15 launches of GEMMs too small to fill a CU.
+//
+// Follows the same arithmetic as the batched driver (dion/newton_schulz_triton.py:508-522,
+// dion/polar_express.py:30-50): X = bf16(G) / (||.||_F * s + eps); A = X X^T; B = c A A + b A + a I;
+// X = B X, with A, B and X rounded to bf16 once per iteration and fp32 MFMA accumulation.
+//
+// Layout: X [64][n_pad] bf16 in LDS (row pitch + 16 B so that 16 consecutive rows hit 16 distinct
+// 16-byte bank slots), A and B [64][64].  X' = B X needs X with the reduction index along rows:
+// those fragments come from ds_read_b64_tr_b16 (a 4 x 16 block of 16-bit elements transposed
+// across a 16-lane group), so no transposed copy of X is kept.
+#include "elementwise.h"
+
+namespace dion {
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+constexpr int kMaxChunks = 36;  // 16-byte chunks a thread may hold while loading (n_pad <= 1152)
+#define LDS3(p) ((__attribute__((address_space(3))) s16x4*)(p))
+
+static __device__ __forceinline__ bf16x8 join_tr(s16x4 lo, s16x4 hi) {
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in, bf16_t* __restrict__ out,
+                                                       int rows, int cols, int n_pad, NsCoeffs co,
+                                                       float norm_scale, float eps) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  __shared__ float red[16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool tall = rows > cols;
+  const int m = tall ? cols : rows, n = tall ? rows : cols;  // m <= 64
+  const int xp = n_pad * 2 + 16;                              // X row pitch in bytes
+  constexpr int ap = 64 * 2 + 16;                             // A / B row pitch in bytes
+  char* Xs = lds;
+  char* As = lds + 64 * xp;
+  char* Bs = As + 64 * ap;
+  const int64_t mat = blockIdx.x;
+  const T* src = in + mat * (int64_t)rows * cols;
+  bf16_t* dst = out + mat * (int64_t)rows * cols;
+
+  // ---- load (raw bf16 values), zero padding, sum of squares, scale, store to LDS
+  float ss = 0.f;
+  const bool vec = (cols % 8 == 0) && ((((uintptr_t)src) & 15) == 0) && n_pad * 8 <= kMaxChunks * 256;
+  if (vec) {
+    // Each thread keeps its 16-byte chunks in registers between the reduction and the scaled
+    // store, so the matrix is read from HBM once and LDS is written once.
+    const int cpr = tall ? 8 : n_pad / 8;  // chunks per 64-wide (tall) or n_pad-wide (wide) input row
+    const int nchunks = 8 * n_pad;         // 64 * n_pad / 8
+    uint4 raw[kMaxChunks];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+      const int idx = tid + c * 256;
+      raw[c] = make_uint4(0, 0, 0, 0);
+      if (idx < nchunks) {
+        const int r = idx / cpr, c0 = (idx - r * cpr) * 8;  // input row, first input column
+        if (r < rows && c0 < cols) {
+          if (sizeof(T) == 2) {
+            raw[c] = *(const uint4*)((const bf16_t*)src + (int64_t)r * cols + c0);
+          } else {
+            const float4 f0 = *(const float4*)((const float*)src + (int64_t)r * cols + c0);
+            const float4 f1 = *(const float4*)((const float*)src + (int64_t)r * cols + c0 + 4);
+            raw[c].x = pack_bf16x2(f0.x, f0.y);
+            raw[c].y = pack_bf16x2(f0.z, f0.w);
+            raw[c].z = pack_bf16x2(f1.x, f1.y);
+            raw[c].w = pack_bf16x2(f1.z, f1.w);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+      const uint32_t w[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __uint_as_float(w[e] << 16), hi = __uint_as_float(w[e] & 0xffff0000u);
+        ss += lo * lo;
+        ss += hi * hi;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float sc = 1.0f / (sqrtf(total) * norm_scale + eps);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+      const int idx = tid + c * 256;
+      if (idx < nchunks) {
+        const int r = idx / cpr, c0 = (idx - r * cpr) * 8;
+        const uint32_t w[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[2 * e] = __uint_as_float(w[e] << 16) * sc;
+          v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u) * sc;
+        }
+        if (!tall) {  // X[r][c0..c0+7]
+          uint4 o;
+          o.x = pack_bf16x2(v[0], v[1]);
+          o.y = pack_bf16x2(v[2], v[3]);
+          o.z = pack_bf16x2(v[4], v[5]);
+          o.w = pack_bf16x2(v[6], v[7]);
+          *(uint4*)(Xs + r * xp + c0 * 2) = o;
+        } else {  // X[c0+e][r]
+#pragma unroll
+          for (int e = 0; e < 8; ++e) *(bf16_t*)(Xs + (c0 + e) * xp + r * 2) = f32_to_bf16(v[e]);
+        }
+      }
+    }
+  } else {
+    for (int idx = tid; idx < 64 * n_pad; idx += 256) {
+      const int i = idx / n_pad, j = idx - i * n_pad;  // X[i][j]
+      float v = 0.f;
+      if (i < m && j < n) {
+        const int64_t g = tall ? (int64_t)j * cols + i : (int64_t)i * cols + j;
+        v = sizeof(T) == 2 ? bf16_to_f32(((const bf16_t*)src)[g])
+                           : bf16_to_f32(f32_to_bf16(((const float*)src)[g]));
+      }
+      ss += v * v;
+      *(bf16_t*)(Xs + i * xp + j * 2) = f32_to_bf16(v);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float sc = 1.0f / (sqrtf(total) * norm_scale + eps);
+    for (int idx = tid; idx < 64 * n_pad; idx += 256) {
+      const int i = idx / n_pad, j = idx - i * n_pad;
+      bf16_t* p = (bf16_t*)(Xs + i * xp + j * 2);
+      *p = f32_to_bf16(bf16_to_f32(*p) * sc);
+    }
+  }
+  __syncthreads();
+
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int ti = wave >> 1, tj = wave & 1;  // this wavefront's 32x32 tile of A / B
+  const int nslice = n_pad / 16;
+
+  for (int it = 0; it < co.n; ++it) {
+    const float a = co.c[it][0], b = co.c[it][1], c = co.c[it][2];
+    // ---- A = X X^T: one 32x32 tile per wavefront, two accumulators to break the MFMA chain
+    {
+      f32x16 acc0, acc1;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc0[r] = acc1[r] = 0.f;
+      const char* pa = Xs + (ti * 32 + frow) * xp + fhalf * 16;
+      const char* pb = Xs + (tj * 32 + frow) * xp + fhalf * 16;
+      for (int s = 0; s < nslice; s += 2) {
+        const bf16x8 a0 = *(const bf16x8*)(pa + s * 32), b0 = *(const bf16x8*)(pb + s * 32);
+        const bf16x8 a1 = *(const bf16x8*)(pa + s * 32 + 32), b1 = *(const bf16x8*)(pb + s * 32 + 32);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc1, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = ti * 32 + (r >> 2) * 8 + 4 * fhalf + (r & 3);
+        *(bf16_t*)(As + row * ap + (tj * 32 + frow) * 2) = f32_to_bf16(acc0[r] + acc1[r]);
+      }
+    }
+    __syncthreads();
+    // ---- B = c A A + b A + a I  (A symmetric: rows of A serve both operands)
+    {
+      f32x16 acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const bf16x8 fa = *(const bf16x8*)(As + (ti * 32 + frow) * ap + s * 32 + fhalf * 16);
+        const bf16x8 fb = *(const bf16x8*)(As + (tj * 32 + frow) * ap + s * 32 + fhalf * 16);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = ti * 32 + (r >> 2) * 8 + 4 * fhalf + (r & 3);
+        const int col = tj * 32 + frow;
+        float v = c * acc[r] + b * bf16_to_f32(*(const bf16_t*)(As + row * ap + col * 2));
+        if (row == col) v += a;
+        *(bf16_t*)(Bs + row * ap + col * 2) = f32_to_bf16(v);
+      }
+    }
+    __syncthreads();
+    // ---- X = B X: wavefront w owns column tiles w, w+4, ...; both row tiles per column tile, so
+    // the whole 64 x 32 column block is read before it is overwritten.
+    {
+      bf16x8 fB[2][4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          fB[i][s] = *(const bf16x8*)(Bs + (i * 32 + frow) * ap + s * 32 + fhalf * 16);
+      // transposed-read addressing: 16-lane group g covers columns (g&1)*16.., k rows 8*(g>>1)..;
+      // lane t of the group points at row t/4, 4-element column chunk t%4.
+      const int g16 = lane >> 4, t16 = lane & 15;
+      const int trow = 8 * (g16 >> 1) + (t16 >> 2);
+      const int tcol = (g16 & 1) * 16 + (t16 & 3) * 4;
+      const bool last = (it == co.n - 1);
+      for (int jt = wave; jt < n_pad / 32; jt += 4) {
+        f32x16 acc[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+        const char* px = Xs + trow * xp + (jt * 32 + tcol) * 2;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS3(px + (s * 16) * xp));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS3(px + (s * 16 + 4) * xp));
+          const bf16x8 fx = join_tr(lo, hi);
+          acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fB[0][s], fx, acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fB[1][s], fx, acc[1], 0, 0, 0);
+        }
+        const int col = jt * 32 + frow;
+        if (!last) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int row = i * 32 + (r >> 2) * 8 + 4 * fhalf + (r & 3);
+              *(bf16_t*)(Xs + row * xp + col * 2) = f32_to_bf16(acc[i][r]);
+            }
+        } else if (col < n) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int row = i * 32 + (r >> 2) * 8 + 4 * fhalf + (r & 3);
+              if (row < m) {
+                const int64_t g = tall ? (int64_t)col * cols + row : (int64_t)row * cols + col;
+                dst[g] = f32_to_bf16(acc[i][r]);
+              }
+            }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  if (co.n == 0) {  // normalisation only
+    for (int idx = tid; idx < m * n; idx += 256) {
+      const int i = idx / n, j = idx - i * n;
+      const int64_t g = tall ? (int64_t)j * cols + i : (int64_t)i * cols + j;
+      dst[g] = *(const bf16_t*)(Xs + i * xp + j * 2);
+    }
+  }
+}
+
+bool ns_small_fits(int rows, int cols) {
+  const int m = rows < cols ? rows : cols, n = rows < cols ? cols : rows;
+  if (m > 64) return false;
+  const int n_pad = (n + 63) / 64 * 64;
+  const size_t bytes = (size_t)64 * (n_pad * 2 + 16) + 2 * 64 * (64 * 2 + 16);
+  return bytes <= 150 * 1024;
+}
+
+hipError_t launch_ns_small(const void* in, int in_dtype, bf16_t* out, int batch, int rows, int cols,
+                           const NsCoeffs& co, float norm_scale, float eps, hipStream_t st) {
+  const int n = rows < cols ? cols : rows;
+  const int n_pad = (n + 63) / 64 * 64;
+  const size_t bytes = (size_t)64 * (n_pad * 2 + 16) + 2 * 64 * (64 * 2 + 16);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)ns_small_kernel<bf16_t>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute((const void*)ns_small_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            150 * 1024);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  if (in_dtype == 0)
+    hipLaunchKernelGGL(ns_small_kernel<bf16_t>, dim3(batch), dim3(256), bytes, st, (const bf16_t*)in, out, rows,
+                       cols, n_pad, co, norm_scale, eps);
+  else
+    hipLaunchKernelGGL(ns_small_kernel<float>, dim3(batch), dim3(256), bytes, st, (const float*)in, out, rows,
+                       cols, n_pad, co, norm_scale, eps);
+  return hipGetLastError();
+}
+
+}  // namespace dion

@@ -88,7 +88,7 @@ def test_ns_line_rank_errors():
 
 
 NS_SHAPES = [(64, 128), (128, 64), (128, 128), (4, 64, 128), (4, 128, 64), (256, 1024), (4, 256, 1024),
-             (2, 768, 3072), (2, 3072, 768), (3, 100, 36), (1, 17, 33)]
+             (2, 768, 3072), (2, 3072, 768), (3, 100, 36), (1, 17, 33), (5, 64, 768), (5, 768, 64), (2, 48, 1000)]
 
 
 def _np_rel(a, b) -> float:
@@ -135,7 +135,8 @@ def test_ns5_vs_oracle(shape):
     ref = oracle.ns_bf16(G, oracle.NS5_COEFFS, 1.0, 1e-7)
     fused = oracle.ns_bf16_fused(G, oracle.NS5_COEFFS, 1.0, 1e-7)
     ref64 = oracle.ns_fp64(G.numpy(), oracle.NS5_COEFFS, 1.0, 1e-7)
-    assert _rel_fro(out, ref) <= 2e-2
+    # below 64 rows the eager path's own noise (1.7-1.8e-2 from exact) leaves no margin: 2.2e-2
+    assert _rel_fro(out, ref) <= (2e-2 if min(shape[-2:]) >= 64 else 2.2e-2)
     assert _rel_fro(out, fused) <= 2e-2
     assert _np_rel(out.float().cpu().numpy().astype(np.float64), ref64) <= 1e-2
     # the reference's own Triton-vs-torch bound (tests/test_newton_shulz.py:145-149)
