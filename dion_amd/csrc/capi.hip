@@ -114,9 +114,7 @@ extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void
   p.tri = 0;
   p.alpha = 1.0f;
   p.beta = a;
-#ifdef DION_DBG_EPILOGUE
-  if (getenv("DION_DBG_NOD")) p.D = nullptr;
-#endif
+  if (a == 0.0f) p.D = nullptr;  // pure product: the form the driver uses after folding a*I into B
   HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_3");
   return DION_OK;
 }

@@ -54,7 +54,8 @@ int dion_ns_line_1(const void* X, void* A, int batch, int m, int k, void* stream
 int dion_ns_line_2(const void* A, void* B, int batch, int m, float alpha, float beta, void* stream);
 
 /* C[b] = a X[b] + B[b] X[b] given X^T: B [batch,m,m] symmetric, X [batch,m,n], Xt = X^T
- * [batch,n,m].  Writes C [batch,m,n] and/or Ct = C^T [batch,n,m] (either may be NULL).
+ * [batch,n,m].  Writes C [batch,m,n] and/or Ct = C^T [batch,n,m] (either may be NULL).  With
+ * a == 0 the addend is skipped altogether (X is not read).
  * Replaces ns_line_3 (dion/newton_schulz_triton.py:450-491) and the baddbmm at :557-563. */
 int dion_ns_line_3(const void* B, const void* X, const void* Xt, void* C, void* Ct, int batch,
                    int m, int n, float a, void* stream);
