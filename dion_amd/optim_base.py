@@ -269,8 +269,14 @@ class OrthoOptimizer(Optimizer):
             scalar_opts.adamw_step(self, group)
         return loss
 
-    def _update_shape_group(self, group: dict, params: List[Tensor]) -> None:
+    def _shape_group_phases(self, group: dict, params: List[Tensor]):
+        """Generator over the three phases of one shape group's update: memory-bound preparation,
+        ``yield``, orthogonalization (GEMM-bound), ``yield``, memory-bound update."""
         raise NotImplementedError
+
+    def _update_shape_group(self, group: dict, params: List[Tensor]) -> None:
+        for _ in self._shape_group_phases(group, params):
+            pass
 
     # Shape groups are independent.  A group whose GEMMs cannot fill the GPU on their own (a few
     # hundred tiles) is run on one of a handful of side streams so that several such groups
@@ -286,24 +292,34 @@ class OrthoOptimizer(Optimizer):
         mats = len(params) * (params[0].numel() // (r * c))
         return mats * 5.0 * (4.0 * m * m * n + 2.0 * m ** 3)
 
-    def _run_shape_groups(self, work: List[Tuple[dict, List[Tensor]]]) -> None:
-        if not work:
-            return
-        on_gpu = all(params[0].is_cuda for _g, params in work)
-        small = [w for w in work if self._group_flop(w[1]) < self._SMALL_GROUP_FLOP] if on_gpu else []
-        if len(small) < 2:
-            for group, params in work:
-                self._update_shape_group(group, params)
-            return
-        big = [w for w in work if self._group_flop(w[1]) >= self._SMALL_GROUP_FLOP]
-        for group, params in big:
-            self._update_shape_group(group, params)
-        device = small[0][1][0].device
+    def _side_pool(self, device) -> List["torch.cuda.Stream"]:
         streams = self.__dict__.setdefault("_side_streams", {})
         pool = streams.get(device)
         if pool is None:
             pool = [torch.cuda.Stream(device=device) for _ in range(self._N_SIDE_STREAMS)]
             streams[device] = pool
+        return pool
+
+    def _run_shape_groups(self, work: List[Tuple[dict, List[Tensor]]]) -> None:
+        if not work:
+            return
+        on_gpu = all(params[0].is_cuda for _g, params in work)
+        if not on_gpu:
+            for group, params in work:
+                self._update_shape_group(group, params)
+            return
+        small = [w for w in work if self._group_flop(w[1]) < self._SMALL_GROUP_FLOP]
+        big = [w for w in work if self._group_flop(w[1]) >= self._SMALL_GROUP_FLOP]
+        # (Running the memory-bound phases of neighbouring large groups under these GEMMs on a
+        # second stream was measured: no gain -- the chip is power-limited, not idle.)
+        for group, params in big:
+            self._update_shape_group(group, params)
+        if len(small) < 2:
+            for group, params in small:
+                self._update_shape_group(group, params)
+            return
+        device = small[0][1][0].device
+        pool = self._side_pool(device)
         main = torch.cuda.current_stream(device)
         fork = main.record_event()
         used = []

@@ -31,6 +31,13 @@ def _check_common(lr, betas, adjust_lr):
         )
 
 
+def _note_stream(t: Tensor) -> None:
+    """A tensor produced on one stream is about to be consumed on the current one: tell the caching
+    allocator so the block is not recycled under the consumer."""
+    if t.is_cuda:
+        t.record_stream(torch.cuda.current_stream(t.device))
+
+
 def _require_fp32(params: List[Tensor], who: str) -> None:
     if params[0].dtype != torch.float32:
         raise NotImplementedError(
@@ -44,7 +51,8 @@ class _MomentumOrtho(OrthoOptimizer):
 
     _normalize = False
 
-    def _update_shape_group(self, group: dict, params: List[Tensor]) -> None:
+    def _shape_group_phases(self, group: dict, params: List[Tensor]):
+        """Generator: [momentum / cast] yield [orthogonalization GEMMs] yield [normalise / update]."""
         num_heads = self._resolve_num_heads(group)
         split_sizes = self._resolve_split_sizes(group)
         shape = params[0].shape
@@ -69,6 +77,8 @@ class _MomentumOrtho(OrthoOptimizer):
         eps = float(group["epsilon"])
 
         U = ops.muon_pre(G, M, group["mu"], group["nesterov"])  # [n, *shape] bf16
+        yield
+        _note_stream(U)
 
         # shape plumbing of muon_update_newton_schulz (dion/megabatch_base.py:884-908)
         if split_sizes is not None:
@@ -77,6 +87,10 @@ class _MomentumOrtho(OrthoOptimizer):
             O = self._orthogonalize(U.view(n, shape[0], -1), eps)
         else:
             O = self._orthogonalize(U.view(n * mats, rows, cols), eps)
+
+        del U
+        yield
+        _note_stream(O)
 
         ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
         row_scale = None
@@ -184,7 +198,8 @@ class Dion2(OrthoOptimizer):
         self.verbose = verbose
         self._triton_post_ortho = bool(triton_post_ortho)
 
-    def _update_shape_group(self, group: dict, params: List[Tensor]) -> None:
+    def _shape_group_phases(self, group: dict, params: List[Tensor]):
+        """Generator: [accumulate / select / gather] yield [orthogonalization] yield [update]."""
         num_heads = self._resolve_num_heads(group)
         if group.get("split_sizes") is not None:
             raise NotImplementedError("split_sizes is currently supported only by Muon and NorMuon.")
@@ -218,6 +233,8 @@ class Dion2(OrthoOptimizer):
 
         U_sel, _idx, imap = ops.dion2_select(G, M, k, select_dim, group["ef_decay"])
         sel_rows, sel_cols = U_sel.shape[-2], U_sel.shape[-1]
+        yield
+        _note_stream(U_sel)
         eps = float(group["epsilon"])
         if flatten and len(shape) >= 3:
             # leading dim stays, the rest of the selected block is one long row
@@ -226,6 +243,9 @@ class Dion2(OrthoOptimizer):
             O = self._orthogonalize(U_sel.view(n, lead, -1), eps)
         else:
             O = self._orthogonalize(U_sel.view(n * mats, sel_rows, sel_cols), eps)
+        del U_sel
+        yield
+        _note_stream(O)
         ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
         ops.dion2_post(X, O.view(n, mats, sel_rows, sel_cols), imap, group["lr"], ratio,
                        group["weight_decay"], select_dim)
