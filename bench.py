@@ -35,7 +35,11 @@ WORKLOADS = {
                  ("proj", 2048, 8192, 24)],
     # the headline shape group on its own
     "ns_4096x14336": [("down", 4096, 14336, 32)],
+    # GPT-small with per-head Newton-Schulz on the fused qkv weight (36 heads of 64x768 per layer)
+    "gpt_small_heads": [("qkv", 2304, 768, 12), ("attn_out", 768, 768, 12), ("fc", 3072, 768, 12),
+                        ("proj", 768, 3072, 12)],
 }
+NUM_HEADS = {"gpt_small_heads": {"qkv": 36}}
 
 
 def ns_flops(rows: int, cols: int, iters: int = 5) -> float:
@@ -95,7 +99,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama3_8b", choices=sorted(WORKLOADS))
-    ap.add_argument("--ns", default="ns5", choices=["ns5", "polar_express"])
+    ap.add_argument("--ns", default="ns5", choices=["ns5", "polar_express", "gram"])
+    ap.add_argument("--optimizer", default="muon", choices=["muon", "normuon", "dion2"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     args = ap.parse_args()
@@ -111,7 +116,7 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
-    from dion import Muon
+    from dion import Dion2, Muon, NorMuon
     from dion_amd import _lib, ops
 
     dev = torch.device("cuda:0")
@@ -120,19 +125,37 @@ def main() -> int:
 
     # ---- synthetic model: X ~ N(0, 0.02) fp32, G ~ N(0, 0.02) bf16, momentum fp32 zeros
     params = []
+    groups = []
     gen = torch.Generator(device=dev).manual_seed(1234)
     total_flops = 0.0
     total_elems = 0
-    for _name, rows, cols, count in spec:
+    fraction = 0.25
+    for name, rows, cols, count in spec:
+        these = []
         for _ in range(count):
             p = torch.nn.Parameter(torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen))
             p.grad_dtype = None
             p.grad = torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen).to(torch.bfloat16)
-            params.append(p)
-        total_flops += count * ns_flops(rows, cols)
+            these.append(p)
+        params += these
+        heads = NUM_HEADS.get(args.workload, {}).get(name)
+        groups.append({"params": these, "num_heads": heads} if heads else {"params": these})
+        r, c = (rows // heads, cols) if heads else (rows, cols)
+        mult = heads or 1
+        if args.optimizer == "dion2":  # NS runs on the selected quarter of the shorter dimension
+            k = -(-min(r, c) * 25 // 100)
+            r, c = (k, c) if r <= c else (r, k)
+        total_flops += count * mult * ns_flops(r, c)
         total_elems += count * rows * cols
-    opt = Muon(params, lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, adjust_lr="spectral_norm",
-               use_polar_express=(args.ns == "polar_express"))
+    ns_kw = dict(use_polar_express=(args.ns == "polar_express"), use_gram_newton_schulz=(args.ns == "gram"))
+    if args.optimizer == "muon":
+        opt = Muon(groups, lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, adjust_lr="spectral_norm", **ns_kw)
+    elif args.optimizer == "normuon":
+        opt = NorMuon(groups, lr=0.02, mu=0.95, muon_beta2=0.95, nesterov=True, weight_decay=0.01,
+                      adjust_lr="spectral_norm", **ns_kw)
+    else:
+        opt = Dion2(groups, lr=0.02, fraction=fraction, ef_decay=0.95, weight_decay=0.01,
+                    adjust_lr="spectral_norm", **ns_kw)
 
     for _ in range(args.warmup):
         opt.step()
@@ -158,7 +181,9 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"{args.workload}: full Muon.step() (nesterov mu=0.95, {args.ns}, wd 0.01, lr 0.02) over "
+            "workload": f"{args.workload}: full {type(opt).__name__}.step() ({args.ns}, wd 0.01, lr 0.02"
+                        + (", fraction 0.25, ef_decay 0.95" if args.optimizer == "dion2" else ", nesterov mu=0.95")
+                        + (", muon_beta2 0.95" if args.optimizer == "normuon" else "") + ") over "
                         + ", ".join(f"{c}x({r}x{k})" for _n, r, k, c in spec),
             "matrices": sum(c for *_x, c in spec),
             "elements": total_elems,
@@ -178,7 +203,7 @@ def main() -> int:
     if not args.no_kernel_timing:
         lib = _lib.load()
         B, m, n = 32, 4096, 14336
-        if args.workload == "gpt_small":
+        if args.workload in ("gpt_small", "gpt_small_heads"):
             B, m, n = 12, 768, 3072
         elif args.workload == "gpt_1p3b":
             B, m, n = 24, 2048, 8192
@@ -222,7 +247,9 @@ def main() -> int:
         # whole NS on the headline group
         from dion_amd import polar_express, zeropower_via_newtonschulz5
 
-        fn = polar_express if args.ns == "polar_express" else zeropower_via_newtonschulz5
+        from dion_amd import gram_newton_schulz
+
+        fn = {"polar_express": polar_express, "gram": gram_newton_schulz}.get(args.ns, zeropower_via_newtonschulz5)
         del C, Ct, Xt, Bm
         ms_ns = time_kernel(lambda: fn(X, 1e-8), iters=3)
         ns_tf = B * ns_flops(m, n) / (ms_ns * 1e-3) * 1e-12
@@ -236,7 +263,7 @@ def main() -> int:
         torch.cuda.empty_cache()
 
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(args.ns)
+        result["cpu_baseline"] = cpu_baseline("polar_express" if args.ns == "gram" else args.ns)
 
     print(json.dumps(result))
     return 0

@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 1; }
+extern "C" int dion_abi_version(void) { return 2; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -476,9 +476,16 @@ static int check_select_dim(const char* who, int select_dim) {
   return DION_OK;
 }
 
+extern "C" size_t dion_dion2_accumulate_scratch_bytes(int n_mat, int rows, int cols, int select_dim) {
+  if (select_dim != -1 || n_mat <= 0 || rows <= 0 || cols <= 0 || cols % 4 != 0) return 0;
+  const int slabs = dion2_acc_slabs(n_mat, rows, cols);
+  return slabs > 1 ? (size_t)slabs * n_mat * cols * sizeof(float) : 0;
+}
+
 extern "C" int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs,
                                      int n, int mats_per_ptr, int rows, int cols, int select_dim,
-                                     float* norms, void* stream) {
+                                     float* norms, void* scratch, size_t scratch_bytes,
+                                     void* stream) {
   if (int rc = check_select_dim("dion_dion2_accumulate", select_dim)) return rc;
   if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0)
     return fail(DION_E_INVALID, "dion_dion2_accumulate: bad size");
@@ -487,13 +494,24 @@ extern "C" int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const 
   if (n == 0 || rows == 0 || cols == 0) return DION_OK;
   if (!G_ptrs || !M_ptrs || !norms) return fail(DION_E_INVALID, "dion_dion2_accumulate: null argument");
   const int dim = select_dim == -2 ? rows : cols;
+  // 16-byte accesses need 4-column alignment of every row of every matrix
+  const bool vec4 = (cols % 4 == 0) && table_aligned(G_ptrs, n) && table_aligned(M_ptrs, n) &&
+                    aligned16((uint64_t)norms);
+  // Row slabs (column sums only): sized for the whole group, used if the scratch holds them.
+  int slabs = 1;
+  if (select_dim == -1 && vec4 && scratch && aligned16((uint64_t)scratch)) {
+    const int64_t n_mat = (int64_t)n * mats_per_ptr;
+    slabs = dion2_acc_slabs((int)n_mat, rows, cols);
+    if ((size_t)slabs * n_mat * cols * sizeof(float) > scratch_bytes) slabs = 1;
+  }
   for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
     const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
     PtrTab g, m;
     fill_tab(g, G_ptrs + i0, c);
     fill_tab(m, M_ptrs + i0, c);
     HIP_TRY(launch_dion2_accumulate(g, g_dtype, m, c * mats_per_ptr, mats_per_ptr, rows, cols,
-                                    select_dim == -2, norms + (int64_t)i0 * mats_per_ptr * dim,
+                                    select_dim == -2, norms + (int64_t)i0 * mats_per_ptr * dim, vec4,
+                                    slabs > 1 ? (float*)scratch : nullptr, slabs,
                                     (hipStream_t)stream),
             "dion_dion2_accumulate");
   }
@@ -520,13 +538,14 @@ extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr
   if (n == 0 || rows == 0 || cols == 0 || k == 0) return DION_OK;
   if (!M_ptrs || !idx || !U_sel) return fail(DION_E_INVALID, "dion_dion2_gather: null argument");
   const int64_t sel_numel = select_dim == -2 ? (int64_t)k * cols : (int64_t)rows * k;
+  const bool vec4 = (cols % 4 == 0) && table_aligned(M_ptrs, n) && aligned16((uint64_t)U_sel);
   for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
     const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
     PtrTab m;
     fill_tab(m, M_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
     HIP_TRY(launch_dion2_gather(m, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
-                                idx + mat0 * k, k, ef_decay, (bf16_t*)U_sel + mat0 * sel_numel,
+                                idx + mat0 * k, k, ef_decay, (bf16_t*)U_sel + mat0 * sel_numel, vec4,
                                 (hipStream_t)stream),
             "dion_dion2_gather");
   }
@@ -545,6 +564,8 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
     return fail(DION_E_INVALID, "dion_dion2_post: null argument");
   const int dim = select_dim == -2 ? rows : cols;
   const int64_t sel_numel = select_dim == -2 ? (int64_t)k * cols : (int64_t)rows * k;
+  const bool vec4 = (cols % 4 == 0) && table_aligned(X_ptrs, n) && aligned16((uint64_t)U_sel) &&
+                    aligned16((uint64_t)map);
   for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
     const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
     PtrTab x;
@@ -552,7 +573,7 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
     HIP_TRY(launch_dion2_post(x, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
                               (const bf16_t*)U_sel + mat0 * sel_numel, k, map + mat0 * dim, lr_dev,
-                              adj_ratio, wd_dev, wd_host, (hipStream_t)stream),
+                              adj_ratio, wd_dev, wd_host, vec4, (hipStream_t)stream),
             "dion_dion2_post");
   }
   return DION_OK;

@@ -43,15 +43,18 @@ hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int n_mat, int
                                 hipStream_t st);
 hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int n_mat,
                                    int mats_per_ptr, int rows, int cols, int select_rows,
-                                   float* norms, hipStream_t st);
+                                   float* norms, bool vec4, float* slab_scratch, int slabs,
+                                   hipStream_t st);
+// Row slabs the column-sum path of launch_dion2_accumulate wants for this shape (1 = no scratch).
+int dion2_acc_slabs(int n_mat, int rows, int cols);
 hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
                              int32_t* map, hipStream_t st);
 hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int rows, int cols,
                                int select_rows, const int32_t* idx, int k, float ef_decay, bf16_t* U,
-                               hipStream_t st);
+                               bool vec4, hipStream_t st);
 hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
                              int select_rows, const bf16_t* U, int k, const int32_t* map,
                              const float* lr_dev, float adj_ratio, const float* wd_dev,
-                             float wd_host, hipStream_t st);
+                             float wd_host, bool vec4, hipStream_t st);
 
 }  // namespace dion

@@ -575,9 +575,86 @@ __global__ __launch_bounds__(256) void dion2_acc_cols_kernel(PtrTab G, PtrTab M,
                                      (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
+// 4 columns per thread (16-byte accesses): each block owns 256 columns, four row lanes.
+// With gridDim.z row slabs the block writes its slab's partial sums to out[(slab*n_mat + mat)*cols]
+// (n_mat = gridDim.y); dion2_sum_slabs_kernel adds the slabs in a fixed order.
+template <typename GT>
+__global__ __launch_bounds__(256) void dion2_acc_cols_vec_kernel(PtrTab G, PtrTab M, int mats_per_ptr,
+                                                                 int rows, int cols, int slab_rows,
+                                                                 float* __restrict__ norms) {
+  __shared__ float4 red[4][64];
+  const int mat = blockIdx.y;
+  const int r0 = blockIdx.z * slab_rows;
+  const int r1 = (r0 + slab_rows) < rows ? (r0 + slab_rows) : rows;
+  norms += (int64_t)blockIdx.z * gridDim.y * cols;
+  const int c = (blockIdx.x * 64 + (threadIdx.x & 63)) * 4;
+  const int ry = threadIdx.x >> 6;
+  const int64_t base = (int64_t)(mat % mats_per_ptr) * rows * cols;
+  const GT* g = (const GT*)G.p[mat / mats_per_ptr] + base;
+  float* m = (float*)M.p[mat / mats_per_ptr] + base;
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (c < cols) {
+#pragma unroll 4
+    for (int r = r0 + ry; r < r1; r += 4) {
+      const int64_t i = (int64_t)r * cols + c;
+      float4 gv;
+      if (sizeof(GT) == 2) {
+        const uint2 raw = *(const uint2*)((const bf16_t*)g + i);
+        gv.x = __uint_as_float(raw.x << 16);
+        gv.y = __uint_as_float(raw.x & 0xffff0000u);
+        gv.z = __uint_as_float(raw.y << 16);
+        gv.w = __uint_as_float(raw.y & 0xffff0000u);
+      } else {
+        gv = *(const float4*)((const float*)g + i);
+      }
+      float4 mv = *(const float4*)(m + i);
+      mv.x = __fadd_rn(mv.x, gv.x);
+      mv.y = __fadd_rn(mv.y, gv.y);
+      mv.z = __fadd_rn(mv.z, gv.z);
+      mv.w = __fadd_rn(mv.w, gv.w);
+      *(float4*)(m + i) = mv;
+      s.x += fabsf(mv.x);
+      s.y += fabsf(mv.y);
+      s.z += fabsf(mv.z);
+      s.w += fabsf(mv.w);
+    }
+  }
+  red[ry][threadIdx.x & 63] = s;
+  __syncthreads();
+  if (ry == 0 && c < cols) {
+    const int t = threadIdx.x;
+    float4 o;
+    o.x = (red[0][t].x + red[1][t].x) + (red[2][t].x + red[3][t].x);
+    o.y = (red[0][t].y + red[1][t].y) + (red[2][t].y + red[3][t].y);
+    o.z = (red[0][t].z + red[1][t].z) + (red[2][t].z + red[3][t].z);
+    o.w = (red[0][t].w + red[1][t].w) + (red[2][t].w + red[3][t].w);
+    *(float4*)(norms + (int64_t)mat * cols + c) = o;
+  }
+}
+
+__global__ __launch_bounds__(256) void dion2_sum_slabs_kernel(const float* __restrict__ part,
+                                                             int64_t n, int slabs,
+                                                             float* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float s = part[i];
+  for (int z = 1; z < slabs; ++z) s += part[(int64_t)z * n + i];
+  out[i] = s;
+}
+
+int dion2_acc_slabs(int n_mat, int rows, int cols) {
+  const int64_t blocks = (int64_t)((cols / 4 + 63) / 64) * n_mat;
+  int64_t s = (2048 + blocks - 1) / blocks;
+  const int64_t s_max = rows / 64 > 0 ? rows / 64 : 1;
+  if (s > s_max) s = s_max;
+  if (s > 32) s = 32;
+  return s < 1 ? 1 : (int)s;
+}
+
 hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int n_mat,
                                    int mats_per_ptr, int rows, int cols, int select_rows,
-                                   float* norms, hipStream_t st) {
+                                   float* norms, bool vec4, float* slab_scratch, int slabs,
+                                   hipStream_t st) {
   if (select_rows) {
     dim3 grid((rows + 3) / 4, n_mat);
     if (g_dtype == 0)
@@ -586,6 +663,23 @@ hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M
     else
       hipLaunchKernelGGL(dion2_acc_rows_kernel<float>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
                          rows, cols, norms);
+  } else if (vec4) {
+    if (!slab_scratch) slabs = 1;
+    const int slab_rows = ((rows + slabs - 1) / slabs + 3) / 4 * 4;
+    slabs = (rows + slab_rows - 1) / slab_rows;
+    float* dst = slabs > 1 ? slab_scratch : norms;
+    dim3 grid((cols / 4 + 63) / 64, n_mat, slabs);
+    if (g_dtype == 0)
+      hipLaunchKernelGGL(dion2_acc_cols_vec_kernel<bf16_t>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
+                         rows, cols, slab_rows, dst);
+    else
+      hipLaunchKernelGGL(dion2_acc_cols_vec_kernel<float>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
+                         rows, cols, slab_rows, dst);
+    if (slabs > 1) {
+      const int64_t n = (int64_t)n_mat * cols;
+      hipLaunchKernelGGL(dion2_sum_slabs_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                         slab_scratch, n, slabs, norms);
+    }
   } else {
     dim3 grid((cols + 63) / 64, n_mat);
     if (g_dtype == 0)
@@ -598,37 +692,56 @@ hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M
   return hipGetLastError();
 }
 
-// Exact top-k by rank counting (rank = number of entries that beat this one; ties go to the lower
-// index), one block per matrix.  Selected indices come out ascending, which keeps the gather and
-// the scatter walking memory forwards.  NaNs order as +inf like torch.topk.
-__global__ __launch_bounds__(1024) void dion2_topk_kernel(const float* __restrict__ norms, int dim,
-                                                          int k, int32_t* __restrict__ idx,
-                                                          int32_t* __restrict__ map) {
-  extern __shared__ float vals[];  // dim floats + 17 ints
-  int* wave_tot = (int*)(vals + dim);
-  const int mat = blockIdx.x;
+// Top-k by rank counting.  Stage 1 (block = 256 candidates of one matrix): the rank of a candidate is
+// the number of entries that beat it (larger value, or equal value at a lower index); it is selected
+// iff rank < k, and the flag goes to map (0 / -1).  NaN counts as +inf.  The whole row sits in LDS and
+// is compared four entries per LDS read; entries before / after the block's own range need one
+// comparison each (>= / >).  Stage 2 (one block per matrix) turns the flags into ascending positions.
+__global__ __launch_bounds__(256) void dion2_rank_kernel(const float* __restrict__ norms, int dim,
+                                                         int k, int32_t* __restrict__ map) {
+  extern __shared__ float4 vals4[];  // dim rounded up to 4 floats; padding -1 (never beats anything)
+  float* vals = (float*)vals4;
+  const int mat = blockIdx.y;
   const float* v = norms + (int64_t)mat * dim;
-  for (int i = threadIdx.x; i < dim; i += 1024) {
-    float x = v[i];
+  const int dim4 = (dim + 3) / 4;
+  for (int i = threadIdx.x; i < dim4 * 4; i += 256) {
+    float x = i < dim ? v[i] : -1.0f;
     if (x != x) x = INFINITY;
     vals[i] = x;
   }
   __syncthreads();
+  const int b0 = blockIdx.x * 256;  // multiple of 4
+  const int b1 = (b0 + 256) < dim4 * 4 ? (b0 + 256) : dim4 * 4;
+  const int i = b0 + threadIdx.x;
+  if (i >= dim) return;
+  const float x = vals[i];
+  int rank = 0;
+  for (int j4 = 0; j4 < b0 / 4; ++j4) {
+    const float4 y = vals4[j4];
+    rank += (y.x >= x) + (y.y >= x) + (y.z >= x) + (y.w >= x);
+  }
+  for (int j4 = b0 / 4; j4 < b1 / 4; ++j4) {
+    const float4 y = vals4[j4];
+    const int j = j4 * 4;
+    rank += ((y.x > x) || (y.x == x && j < i)) + ((y.y > x) || (y.y == x && j + 1 < i)) +
+            ((y.z > x) || (y.z == x && j + 2 < i)) + ((y.w > x) || (y.w == x && j + 3 < i));
+  }
+  for (int j4 = b1 / 4; j4 < dim4; ++j4) {
+    const float4 y = vals4[j4];
+    rank += (y.x > x) + (y.y > x) + (y.z > x) + (y.w > x);
+  }
+  map[(int64_t)mat * dim + i] = rank < k ? 0 : -1;
+}
+
+__global__ __launch_bounds__(1024) void dion2_compact_kernel(int dim, int k, int32_t* __restrict__ idx,
+                                                             int32_t* __restrict__ map) {
+  __shared__ int wave_tot[16];
+  const int mat = blockIdx.x;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   int running = 0;  // selected entries before the current chunk (same in every thread)
   for (int base = 0; base < dim; base += 1024) {
     const int i = base + threadIdx.x;
-    int sel = 0;
-    if (i < dim) {
-      const float x = vals[i];
-      int rank = 0;
-      for (int j = 0; j < dim; ++j) {
-        const float y = vals[j];
-        rank += (y > x) || (y == x && j < i);
-      }
-      sel = rank < k;
-    }
-    // block-wide exclusive scan of sel
+    const int sel = (i < dim) ? (map[(int64_t)mat * dim + i] == 0) : 0;
     const unsigned long long ball = __ballot(sel);
     const int in_wave = __popcll(ball & ((1ull << lane) - 1ull));
     __syncthreads();
@@ -640,10 +753,10 @@ __global__ __launch_bounds__(1024) void dion2_topk_kernel(const float* __restric
       if (q < w) before += tq;
       total += tq;
     }
-    if (i < dim) {
+    if (sel) {
       const int pos = running + before + in_wave;
-      if (sel) idx[(int64_t)mat * k + pos] = i;
-      map[(int64_t)mat * dim + i] = sel ? pos : -1;
+      idx[(int64_t)mat * k + pos] = i;
+      map[(int64_t)mat * dim + i] = pos;
     }
     running += total;
   }
@@ -651,19 +764,24 @@ __global__ __launch_bounds__(1024) void dion2_topk_kernel(const float* __restric
 
 hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
                              int32_t* map, hipStream_t st) {
-  const size_t shmem = (size_t)dim * sizeof(float) + 17 * sizeof(int);
+  const size_t shmem = (size_t)((dim + 3) / 4) * 16;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)dion2_topk_kernel,
+    hipError_t e = hipFuncSetAttribute((const void*)dion2_rank_kernel,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(dion2_topk_kernel, dim3(n_mat), dim3(1024), shmem, st, norms, dim, k, idx, map);
+  hipLaunchKernelGGL(dion2_rank_kernel, dim3((dim + 255) / 256, n_mat), dim3(256), shmem, st, norms,
+                     dim, k, map);
+  hipLaunchKernelGGL(dion2_compact_kernel, dim3(n_mat), dim3(1024), 0, st, dim, k, idx, map);
   return hipGetLastError();
 }
 
 // U_sel = bf16(M[sel]); M[sel] *= ef_decay.
+// rows selected: block (j, mat) copies row idx[j]; columns selected: block (row, mat) gathers the k
+// selected columns (ascending, so the reads walk the row forwards).
+template <bool VEC>
 __global__ __launch_bounds__(256) void dion2_gather_kernel(PtrTab M, int mats_per_ptr, int rows,
                                                            int cols, int select_rows,
                                                            const int32_t* __restrict__ idx, int k,
@@ -671,40 +789,59 @@ __global__ __launch_bounds__(256) void dion2_gather_kernel(PtrTab M, int mats_pe
   const int mat = blockIdx.y;
   float* m = (float*)M.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
   const int32_t* id = idx + (int64_t)mat * k;
-  const int64_t stride = (int64_t)gridDim.x * 256;
   if (select_rows) {
-    bf16_t* u = U + (int64_t)mat * k * cols;
-    const int64_t n = (int64_t)k * cols;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-      const int j = (int)(i / cols), c = (int)(i - (int64_t)j * cols);
-      const int64_t src = (int64_t)id[j] * cols + c;
-      const float v = m[src];
-      u[i] = f32_to_bf16(v);
-      m[src] = __fmul_rn(v, ef_decay);
+    const int j = blockIdx.x;
+    float* src = m + (int64_t)id[j] * cols;
+    bf16_t* u = U + ((int64_t)mat * k + j) * cols;
+    if (VEC) {
+      for (int c = threadIdx.x * 4; c < cols; c += 1024) {
+        float4 v = *(const float4*)(src + c);
+        uint2 o;
+        o.x = pack_bf16x2(v.x, v.y);
+        o.y = pack_bf16x2(v.z, v.w);
+        *(uint2*)(u + c) = o;
+        v.x = __fmul_rn(v.x, ef_decay);
+        v.y = __fmul_rn(v.y, ef_decay);
+        v.z = __fmul_rn(v.z, ef_decay);
+        v.w = __fmul_rn(v.w, ef_decay);
+        *(float4*)(src + c) = v;
+      }
+    } else {
+      for (int c = threadIdx.x; c < cols; c += 256) {
+        const float v = src[c];
+        u[c] = f32_to_bf16(v);
+        src[c] = __fmul_rn(v, ef_decay);
+      }
     }
   } else {
-    bf16_t* u = U + (int64_t)mat * rows * k;
-    const int64_t n = (int64_t)rows * k;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-      const int r = (int)(i / k), j = (int)(i - (int64_t)r * k);
-      const int64_t src = (int64_t)r * cols + id[j];
-      const float v = m[src];
-      u[i] = f32_to_bf16(v);
-      m[src] = __fmul_rn(v, ef_decay);
+    const int r = blockIdx.x;
+    float* src = m + (int64_t)r * cols;
+    bf16_t* u = U + ((int64_t)mat * rows + r) * k;
+    for (int j = threadIdx.x; j < k; j += 256) {
+      const int c = id[j];
+      const float v = src[c];
+      u[j] = f32_to_bf16(v);
+      src[c] = __fmul_rn(v, ef_decay);
     }
   }
 }
 
 hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int rows, int cols,
                                int select_rows, const int32_t* idx, int k, float ef_decay, bf16_t* U,
-                               hipStream_t st) {
-  const int64_t n = select_rows ? (int64_t)k * cols : (int64_t)rows * k;
-  hipLaunchKernelGGL(dion2_gather_kernel, dim3(ew_blocks(n), n_mat), dim3(256), 0, st, M,
-                     mats_per_ptr, rows, cols, select_rows, idx, k, ef_decay, U);
+                               bool vec4, hipStream_t st) {
+  dim3 grid(select_rows ? k : rows, n_mat);
+  if (vec4)
+    hipLaunchKernelGGL(dion2_gather_kernel<true>, grid, dim3(256), 0, st, M, mats_per_ptr, rows, cols,
+                       select_rows, idx, k, ef_decay, U);
+  else
+    hipLaunchKernelGGL(dion2_gather_kernel<false>, grid, dim3(256), 0, st, M, mats_per_ptr, rows, cols,
+                       select_rows, idx, k, ef_decay, U);
   return hipGetLastError();
 }
 
 // x = a*x - b*u[map] on selected slices, x = a*x elsewhere; one rounding of the sum.
+// Block (row group of 8, mat); 4 columns per thread on the vector path.
+template <bool VEC>
 __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_ptr, int rows,
                                                          int cols, int select_rows,
                                                          const bf16_t* __restrict__ U, int k,
@@ -722,24 +859,73 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
   const int dim = select_rows ? rows : cols;
   const int32_t* mp = map + (int64_t)mat * dim;
   const bf16_t* u = U + (int64_t)mat * (select_rows ? (int64_t)k * cols : (int64_t)rows * k);
-  const int64_t n = (int64_t)rows * cols;
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-    const int r = (int)(i / cols), c = (int)(i - (int64_t)r * cols);
-    const int j = mp[select_rows ? r : c];
-    float uv = 0.f;
-    if (j >= 0) uv = bf16_to_f32(select_rows ? u[(int64_t)j * cols + c] : u[(int64_t)r * k + j]);
-    x[i] = fmaf(a, x[i], -(b * uv));
+  const int r_end = (blockIdx.x * 8 + 8) < rows ? (blockIdx.x * 8 + 8) : rows;
+  for (int r = blockIdx.x * 8; r < r_end; ++r) {
+    float* xr = x + (int64_t)r * cols;
+    if (select_rows) {
+      const int j = mp[r];
+      const bf16_t* ur = u + (int64_t)(j < 0 ? 0 : j) * cols;
+      if (VEC) {
+        for (int c = threadIdx.x * 4; c < cols; c += 1024) {
+          float4 v = *(const float4*)(xr + c);
+          float4 uv = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (j >= 0) {
+            const uint2 raw = *(const uint2*)(ur + c);
+            uv.x = __uint_as_float(raw.x << 16);
+            uv.y = __uint_as_float(raw.x & 0xffff0000u);
+            uv.z = __uint_as_float(raw.y << 16);
+            uv.w = __uint_as_float(raw.y & 0xffff0000u);
+          }
+          v.x = fmaf(a, v.x, -(b * uv.x));
+          v.y = fmaf(a, v.y, -(b * uv.y));
+          v.z = fmaf(a, v.z, -(b * uv.z));
+          v.w = fmaf(a, v.w, -(b * uv.w));
+          *(float4*)(xr + c) = v;
+        }
+      } else {
+        for (int c = threadIdx.x; c < cols; c += 256) {
+          const float uv = j >= 0 ? bf16_to_f32(ur[c]) : 0.f;
+          xr[c] = fmaf(a, xr[c], -(b * uv));
+        }
+      }
+    } else {
+      const bf16_t* ur = u + (int64_t)r * k;
+      if (VEC) {
+        for (int c = threadIdx.x * 4; c < cols; c += 1024) {
+          float4 v = *(const float4*)(xr + c);
+          const int4 j4 = *(const int4*)(mp + c);
+          const float u0 = j4.x >= 0 ? bf16_to_f32(ur[j4.x]) : 0.f;
+          const float u1 = j4.y >= 0 ? bf16_to_f32(ur[j4.y]) : 0.f;
+          const float u2 = j4.z >= 0 ? bf16_to_f32(ur[j4.z]) : 0.f;
+          const float u3 = j4.w >= 0 ? bf16_to_f32(ur[j4.w]) : 0.f;
+          v.x = fmaf(a, v.x, -(b * u0));
+          v.y = fmaf(a, v.y, -(b * u1));
+          v.z = fmaf(a, v.z, -(b * u2));
+          v.w = fmaf(a, v.w, -(b * u3));
+          *(float4*)(xr + c) = v;
+        }
+      } else {
+        for (int c = threadIdx.x; c < cols; c += 256) {
+          const int j = mp[c];
+          const float uv = j >= 0 ? bf16_to_f32(ur[j]) : 0.f;
+          xr[c] = fmaf(a, xr[c], -(b * uv));
+        }
+      }
+    }
   }
 }
 
 hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
                              int select_rows, const bf16_t* U, int k, const int32_t* map,
                              const float* lr_dev, float adj_ratio, const float* wd_dev,
-                             float wd_host, hipStream_t st) {
-  hipLaunchKernelGGL(dion2_post_kernel, dim3(ew_blocks((int64_t)rows * cols), n_mat), dim3(256), 0,
-                     st, X, mats_per_ptr, rows, cols, select_rows, U, k, map, lr_dev, adj_ratio,
-                     wd_dev, wd_host);
+                             float wd_host, bool vec4, hipStream_t st) {
+  dim3 grid((rows + 7) / 8, n_mat);
+  if (vec4)
+    hipLaunchKernelGGL(dion2_post_kernel<true>, grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols,
+                       select_rows, U, k, map, lr_dev, adj_ratio, wd_dev, wd_host);
+  else
+    hipLaunchKernelGGL(dion2_post_kernel<false>, grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols,
+                       select_rows, U, k, map, lr_dev, adj_ratio, wd_dev, wd_host);
   return hipGetLastError();
 }
 

@@ -301,8 +301,11 @@ def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_d
     U = torch.empty(sel_shape, dtype=torch.bfloat16, device=dev)
     lib = _lib.load()
     st = _stream_handle(dev)
+    sbytes = lib.dion_dion2_accumulate_scratch_bytes(n_mat, rows, cols, select_dim)
+    scratch = torch.empty(sbytes, dtype=torch.uint8, device=dev) if sbytes else None
     check(lib.dion_dion2_accumulate(gp, _dtype_code(G[0], "G"), mp, n, mats_per_ptr, rows, cols, select_dim,
-                                    norms.data_ptr(), st), "dion2_accumulate")
+                                    norms.data_ptr(), scratch.data_ptr() if sbytes else None, sbytes, st),
+          "dion2_accumulate")
     check(lib.dion_dion2_topk(norms.data_ptr(), n_mat, dim, k, idx.data_ptr(), imap.data_ptr(), st),
           "dion2_topk")
     check(lib.dion_dion2_gather(mp, n, mats_per_ptr, rows, cols, select_dim, idx.data_ptr(), k,

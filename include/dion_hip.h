@@ -120,10 +120,15 @@ int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_pe
  *   M_i += G_i;  norms[i][s] = sum |M_i| over the other dim, for each slice s along select_dim
  * select_dim: -2 (rows) or -1 (columns).  norms out [n_mat, dim] fp32 (dim = rows or cols).
  * M_ptrs entries each cover mats_per_ptr consecutive matrices.
+ * scratch (nullable): device memory of dion_dion2_accumulate_scratch_bytes() bytes, 16-byte
+ * aligned; with it the column sums (select_dim -1) of tall matrices are split over row slabs so
+ * that the launch fills the chip, and added in a fixed order.  Without it one workgroup walks
+ * all rows of its columns.
  * Replaces the first half of dion2_pre_orthogonalize (dion/dion2.py:487-509). */
+size_t dion_dion2_accumulate_scratch_bytes(int n_mat, int rows, int cols, int select_dim);
 int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int n,
                           int mats_per_ptr, int rows, int cols, int select_dim, float* norms,
-                          void* stream);
+                          void* scratch, size_t scratch_bytes, void* stream);
 
 /* Dion2 top-k selection: for each of n_mat rows of norms [n_mat, dim] pick the k largest
  * (ties: lower index first), write their indices ascending to idx [n_mat, k] (int32) and the
