@@ -115,6 +115,15 @@ extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void
   p.alpha = 1.0f;
   p.beta = a;
   if (a == 0.0f) p.D = nullptr;  // pure product: the form the driver uses after folding a*I into B
+  if (!Ct && X) {
+    // X' alone: read X with the reduction index along rows; X^T is not needed
+    p.Q = (const bf16_t*)X;
+    p.ldq = n;
+    p.q_kmajor = 1;
+  } else if (!Xt) {
+    return fail(DION_E_INVALID, "dion_ns_line_3: Xt is required when Ct is requested");
+  }
+  if (p.D == nullptr && a != 0.0f) return fail(DION_E_INVALID, "dion_ns_line_3: X is required when a != 0");
   HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_3");
   return DION_OK;
 }
@@ -162,9 +171,11 @@ NsPlan make_plan(int batch, int rows, int cols, int flags) {
   pl.a_bytes = align256((size_t)batch * pl.mp * pl.lda * 2);
   pl.partial_bytes = align256((size_t)batch * pl.nblk * 4);
   pl.inv_bytes = align256((size_t)batch * 4);
-  // X, Xt ping-pong pairs; A, B (+ Q, Z, T for the Gram recurrence)
+  // X, Xt ping-pong pairs (X-only form: the X pair and one X^T for a padded tall result);
+  // A, B (+ Q, Z, T for the Gram recurrence)
   const int n_sq = (flags & DION_NS_GRAM) ? 6 : 2;
-  pl.total = 4 * pl.x_bytes + n_sq * pl.a_bytes + pl.partial_bytes + pl.inv_bytes;
+  const int n_x = (flags & DION_NS_XONLY) ? 3 : 4;
+  pl.total = n_x * pl.x_bytes + n_sq * pl.a_bytes + pl.partial_bytes + pl.inv_bytes;
   return pl;
 }
 }  // namespace
@@ -185,7 +196,7 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   if (batch == 0 || rows == 0 || cols == 0) return DION_OK;
   if (!in || !out || (n_iters > 0 && !coeffs))
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: null argument");
-  if (flags & ~DION_NS_GRAM) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
+  if (flags & ~(DION_NS_GRAM | DION_NS_XONLY)) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
   hipStream_t st = (hipStream_t)stream;
   if (!(flags & DION_NS_GRAM) && n_iters <= kMaxSmallIters && ns_small_fits(rows, cols) &&
       !getenv("DION_NO_SMALL_KERNEL")) {
@@ -211,7 +222,11 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   X[0] = (bf16_t*)w; w += pl.x_bytes;
   X[1] = (bf16_t*)w; w += pl.x_bytes;
   Xt[0] = (bf16_t*)w; w += pl.x_bytes;
-  Xt[1] = (bf16_t*)w; w += pl.x_bytes;
+  if (flags & DION_NS_XONLY) {
+    Xt[1] = Xt[0];  // only ever written by the last product
+  } else {
+    Xt[1] = (bf16_t*)w; w += pl.x_bytes;
+  }
   bf16_t* sq[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};  // m x m scratch
   for (int i = 0; i < ((flags & DION_NS_GRAM) ? 6 : 2); ++i) {
     sq[i] = (bf16_t*)w;
@@ -226,11 +241,17 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   HIP_TRY(launch_frobenius_inv(in, in_dtype, batch, (int64_t)rows * cols, norm_scale, eps, partial,
                                pl.nblk, inv, st),
           "frobenius norm");
+  // DION_NS_XONLY: X' = B X reads X itself (reduction index along rows) and no X^T is carried.
+  // The default form (X and X^T side by side) is the faster one: its operand tiles are contiguous
+  // along the reduction index in memory.
+  const bool nn = (flags & DION_NS_XONLY) != 0;
   if (pl.tall)
-    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, Xt[0], np, mp, ldxt, sXt, X[0], ldx, sX, st),
+    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, nn ? nullptr : Xt[0], np, mp, ldxt, sXt,
+                              X[0], ldx, sX, st),
             "prepare");
   else
-    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, X[0], mp, np, ldx, sX, Xt[0], ldxt, sXt, st),
+    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, X[0], mp, np, ldx, sX,
+                              nn ? nullptr : Xt[0], ldxt, sXt, st),
             "prepare");
 
   const bool direct = (mp == pl.m && np == pl.n);
@@ -279,15 +300,25 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   };
   // apply(S, Xtc -> Xn, Xtn | out): X' = S X given X^T (S symmetric m x m).  `final` writes the
   // caller's tensor in its own orientation when no padding is in the way.
-  auto apply = [&](const bf16_t* S, const bf16_t* Xtc, bf16_t* Xn, bf16_t* Xtn, bool final_direct) -> hipError_t {
+  // In the X-only form (nn) the last product of a tall input is written transposed (the caller's
+  // orientation), every other one as X' alone.
+  auto apply = [&](const bf16_t* S, const bf16_t* Xc, const bf16_t* Xtc, bf16_t* Xn, bf16_t* Xtn,
+                   bool last, bool final_direct) -> hipError_t {
     GemmParams p;
     memset(&p, 0, sizeof(p));
     p.P = S;
-    p.Q = Xtc;
     p.strideP = sA;
-    p.strideQ = sXt;
     p.ldp = lda;
-    p.ldq = ldxt;
+    if (nn) {
+      p.Q = Xc;
+      p.strideQ = sX;
+      p.ldq = ldx;
+      p.q_kmajor = 1;
+    } else {
+      p.Q = Xtc;
+      p.strideQ = sXt;
+      p.ldq = ldxt;
+    }
     p.M = p.Mst = mp;
     p.N = p.Nst = np;
     p.K = mp;
@@ -304,8 +335,8 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
         p.ldc = np;
       }
     } else {
-      p.C = Xn;
-      p.Ct = Xtn;
+      p.C = (nn && last && pl.tall) ? nullptr : Xn;
+      p.Ct = (nn && !(last && pl.tall)) ? nullptr : Xtn;
       p.strideC = sX;
       p.strideCt = sXt;
       p.ldc = ldx;
@@ -323,7 +354,7 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
       // a*I folded into B: the next GEMM needs no addend (one fewer pass over X)
       HIP_TRY(sym(sq[0], sq[0], sq[0], sq[1], c, b, a), "B = c A A + b A + a I");
       const bool fin = (it == n_iters - 1) && direct;
-      HIP_TRY(apply(sq[1], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], fin), "X = B X");
+      HIP_TRY(apply(sq[1], X[cur], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], it == n_iters - 1, fin), "X = B X");
       wrote_out = fin;
       cur ^= 1;
     }
@@ -346,7 +377,7 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     for (int it = 0; it < n_iters; ++it) {
       const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
       if (it == gram_reset && it > 0 && q >= 0) {
-        HIP_TRY(apply(sq[q], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], false), "X = Q X (restart)");
+        HIP_TRY(apply(sq[q], X[cur], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], false, false), "X = Q X (restart)");
         cur ^= 1;
         used[q] = false;
         q = -1;
@@ -375,7 +406,7 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
       }
     }
     if (q >= 0) {
-      HIP_TRY(apply(sq[q], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], direct), "X = Q X");
+      HIP_TRY(apply(sq[q], X[cur], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], true, direct), "X = Q X");
       wrote_out = direct;
       cur ^= 1;
     }

@@ -36,7 +36,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // GEMM of a chain can write into an unpadded destination.
 struct GemmParams {
   const bf16_t* P;   // [batch][M][K], leading dimension ldp
-  const bf16_t* Q;   // [batch][N][K], leading dimension ldq (== P when tri)
+  const bf16_t* Q;   // [batch][N][K], leading dimension ldq (== P when tri); [batch][K][N] if q_kmajor
   const bf16_t* D;   // optional [batch][M][N] addend, leading dimension ldd
   bf16_t* C;         // optional [batch][Mst][Nst]
   bf16_t* Ct;        // optional [batch][Nst][Mst] (transposed copy; == C when tri -> mirror)
@@ -46,6 +46,7 @@ struct GemmParams {
   int Mst, Nst;
   int batch;
   int tri;           // 1: Q == P, only tiles with tile_row <= tile_col are computed, Ct mirrors
+  int q_kmajor;      // 1: Q is stored [K][N] (reduction index along rows); not with tri
   float alpha, beta;
   float diag;        // added to C[i][i] (global diagonal); used with tri to fold a*I into B
 };

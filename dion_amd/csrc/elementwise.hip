@@ -123,9 +123,10 @@ __global__ __launch_bounds__(256) void ns_prepare_kernel(const T* __restrict__ i
     bf16_t v = 0;
     if (r < R && c < C) v = f32_to_bf16(load_as_bf16_f32<T>(src, (int64_t)r * C + c) * sc);
     tile[i][tx] = v;
-    ds[(int64_t)r * ld_same + c] = v;
+    if (same) ds[(int64_t)r * ld_same + c] = v;
   }
   __syncthreads();
+  if (!trans) return;
 #pragma unroll 4
   for (int i = ty; i < 64; i += 4) {
     // trans row (c0 + i), column (r0 + tx)
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(256) void ns_prepare_kernel(const T* __restrict__ i
   }
 }
 
-// Same operation, 16-byte accesses: needs C % 8 == 0, 16-byte aligned input and row pitches.
+// Same operation (either output may be null), 16-byte accesses: needs C % 8 == 0, 16-byte aligned input and row pitches.
 template <typename T>
 __global__ __launch_bounds__(256) void ns_prepare_vec_kernel(const T* __restrict__ in, int R, int C,
                                                              const float* __restrict__ inv_norm,
@@ -163,9 +164,10 @@ __global__ __launch_bounds__(256) void ns_prepare_vec_kernel(const T* __restrict
       o.w = pack_bf16x2(v[6] * sc, v[7] * sc);
     }
     *(uint4*)&tile[i][chunk * 8] = o;
-    *(uint4*)(ds + (int64_t)r * ld_same + c) = o;
+    if (same) *(uint4*)(ds + (int64_t)r * ld_same + c) = o;
   }
   __syncthreads();
+  if (!trans) return;
   // transposed: thread -> (trans row = column rr + 32*pass of the tile, 8 consecutive source rows)
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {

@@ -5,6 +5,9 @@
 //   A  = X X^T                     P = Q = X            (tri: upper tiles + mirrored store)
 //   B  = c A A + b A + a I         P = Q = A (A = A^T)  (tri, D = A, a on the diagonal)
 //   X' = B X  (= a X + (B - aI) X)  P = B, Q = X^T, stores X' and (X')^T
+// A second operand form (QK) takes Q stored with the reduction index along rows, [K][N]: X' = B X
+// then reads X itself, its MFMA fragments come from ds_read_b64_tr_b16 (transposing LDS read), and
+// no X^T has to be kept or written.
 // This replaces the reference's ns_line_1 / ns_line_2 / ns_line_3
 // (dion/newton_schulz_triton.py:88-157, :206-287, :384-447) and the baddbmm of
 // dion/newton_schulz_triton.py:557-563.
@@ -116,7 +119,9 @@ __device__ __forceinline__ void pipeline_barrier() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT>
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false>
 __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, KK = Cfg::KK, NSTAGE = Cfg::NSTAGE;
@@ -126,6 +131,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
   static_assert(KK % 2 == 0, "fragment double buffer needs an even slice count per stage");
   constexpr int RPM = (NR + NM - 1) / NM;    // fragment reads slotted behind each MFMA
   constexpr int LPM = (LPS + NM - 1) / NM;   // refill loads slotted behind each MFMA
+  // With three or more ring slots the refill of a slot need not be issued in one burst: it is
+  // spread over the KK slices that follow the barrier which frees the slot (the last slice of its
+  // slab and the first KK-1 slices of the next), LPW loads per slice at even MFMA spacing, so the
+  // loads reach the vector memory pipeline at the rate it drains them.
+  constexpr bool SPREAD = NSTAGE >= 3 && LPS % KK == 0 && NM % (LPS / KK) == 0;
+  constexpr int LPW = SPREAD ? LPS / KK : LPS;
+  constexpr int QPL = SPREAD ? NM / LPW : 1;  // MFMAs per load slot
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int tid = threadIdx.x;
@@ -167,11 +179,22 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
   const int ld_phys = tid % Cfg::CPR;
   const int ld_chunk = ld_phys ^ ((ld_row / Cfg::SWZ_DIV) % Cfg::CPR);
   const char* gP = (const char*)(p.P + (int64_t)b * p.strideP + (int64_t)(ti * BM) * p.ldp);
-  const char* gQ = (const char*)(p.Q + (int64_t)b * p.strideQ + (int64_t)(tj * BN) * p.ldq);
+  // QK: the Q tile is BK rows (reduction index) of BN bf16; chunk q lands at LDS byte q*16 and holds
+  // logical chunk ((c >> 2) ^ (row & 3)) << 2 | (c & 3), c = q % QCPR, of tile row q / QCPR: the four
+  // rows one transposing read gathers land in four distinct 64-byte bank groups.
+  constexpr int QCPR = BN / 8;               // 16-byte chunks per K-major tile row
+  constexpr int QROWS_PER_LOAD = Cfg::NT / QCPR;
+  static_assert(!QK || (BK % QROWS_PER_LOAD == 0 && QROWS_PER_LOAD % 4 == 0), "K-major tile/threads");
+  const int qk_row = tid / QCPR;
+  const int qk_chunk = ((((tid % QCPR) >> 2) ^ (qk_row & 3)) << 2) | (tid & 3);
+  const char* gQ = QK ? (const char*)(p.Q + (int64_t)b * p.strideQ + tj * BN)
+                      : (const char*)(p.Q + (int64_t)b * p.strideQ + (int64_t)(tj * BN) * p.ldq);
   const uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
-  const uint32_t offQ = (uint32_t)(ld_row * p.ldq + ld_chunk * 8) * 2u;
+  const uint32_t offQ = QK ? (uint32_t)(qk_row * p.ldq + qk_chunk * 8) * 2u
+                           : (uint32_t)(ld_row * p.ldq + ld_chunk * 8) * 2u;
   const uint32_t stepP = (uint32_t)(Cfg::ROWS_PER_LOAD * p.ldp) * 2u;
-  const uint32_t stepQ = (uint32_t)(Cfg::ROWS_PER_LOAD * p.ldq) * 2u;
+  const uint32_t stepQ = (uint32_t)((QK ? QROWS_PER_LOAD : Cfg::ROWS_PER_LOAD) * p.ldq) * 2u;
+  const int64_t slabQ = QK ? (int64_t)BK * p.ldq * 2 : (int64_t)BK * 2;  // bytes between k-slabs of Q
   const int KT = p.K / BK;
 
   // One direct-to-LDS load (index j of the LPS that make up a stage) of k-slab kt into ring
@@ -188,7 +211,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
       __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
     } else {
       const int jq = j - Cfg::P_LOADS;
-      const char* src = gQ + (int64_t)k * (BK * 2) + (offQ + jq * stepQ);
+      const char* src = gQ + k * slabQ + (offQ + jq * stepQ);
       __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + Cfg::P_BYTES + jq * (Cfg::NT * 16)),
                                        16, 0, 0);
     }
@@ -206,12 +229,41 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
     boff[kk] = (uint32_t)(Cfg::P_BYTES + (wn * Cfg::WTN + frow) * (BK * 2) + chunk);
   }
 
+  // QK fragments: within a 16-lane group, lane 4r+q addresses row r / 4-element piece q of a 4x16
+  // block; the transposing read hands lane i column i.  Lanes 0-31 take k 0..7 of the slice (two
+  // reads of 4 rows), lanes 32-63 k 8..15; column = lane % 32.
+  uint32_t qoff[TN];
+  if (QK) {
+    const int g16 = lane >> 4, t16 = lane & 15;
+#pragma unroll
+    for (int r = 0; r < TN; ++r)
+      qoff[r] = (uint32_t)(Cfg::P_BYTES + (8 * (g16 >> 1) + (t16 >> 2)) * (BN * 2) +
+                           ((((wn * Cfg::WTN + r * 32) >> 5) ^ (t16 >> 2)) << 6) + (g16 & 1) * 32 +
+                           (t16 & 3) * 8);
+  }
+
   bf16x8 fa[2][TM], fb[2][TN];
-  // Fragment read r (0..NR-1) of slice kk of ring slot buf into fragment set f.
+  // Fragment read r (0..NR-1) of slice kk of ring slot buf into fragment set f, in the order the
+  // MFMAs (row-major over the TM x TN accumulators) first need them: A0, B0..B(TN-1), A1..A(TM-1).
   auto read_frag = [&](int buf, int kk, int f, int r) {
     const char* st = lds + buf * Cfg::STAGE_BYTES;
-    if (r < TM) fa[f][r] = *(const bf16x8*)(st + aoff[kk] + r * (32 * BK * 2));
-    else fb[f][r - TM] = *(const bf16x8*)(st + boff[kk] + (r - TM) * (32 * BK * 2));
+    if (r == 0 || r > TN) {
+      const int i = r == 0 ? 0 : r - TN;
+      fa[f][i] = *(const bf16x8*)(st + aoff[kk] + i * (32 * BK * 2));
+    } else if (QK) {
+      const int j = r - 1;
+      const char* q = st + qoff[j] + kk * (16 * BN * 2);
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4*)(q));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4*)(q + 4 * BN * 2));
+      typedef __attribute__((ext_vector_type(8))) short s16x8;
+      const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      fb[f][j] = __builtin_bit_cast(bf16x8, v);
+    } else {
+      const int j = r - 1;
+      fb[f][j] = *(const bf16x8*)(st + boff[kk] + j * (32 * BK * 2));
+    }
   };
 
   f32x16 acc[TM][TN];
@@ -232,7 +284,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
 #pragma unroll
   for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
 #pragma unroll
-  for (int j = 0; j < LPS; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
+  for (int j = 0; j < LPW; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- main loop.  Slices run back to back across slab boundaries: while the MFMAs of one slice
@@ -260,7 +312,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
             if (last) read_frag((s + 1) % NSTAGE, 0, nxt, r);
             else read_frag(s, kk + 1, nxt, r);
           }
-          if (last) {
+          if (SPREAD) {
+            if (q % QPL == QPL / 2) {
+              const int jw = q / QPL;
+              if (last) issue_load(kt0 + s + NSTAGE, s, jw);
+              else issue_load(kt0 + s - 1 + NSTAGE, (s + NSTAGE - 1) % NSTAGE, (kk + 1) * LPW + jw);
+            }
+          } else if (last) {
 #pragma unroll
             for (int j = q * LPM; j < (q + 1) * LPM && j < LPS; ++j)
               issue_load(kt0 + s + NSTAGE, s, j);
@@ -353,11 +411,12 @@ typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg128;
 typedef TileCfg<256, 256, 32, 2, 2, 4> Cfg256k32;
 typedef TileCfg<256, 256, 64, 2, 4, 2> Cfg256w8;   // 8 wavefronts, 128x64 each: two per SIMD
 typedef TileCfg<256, 256, 64, 4, 2, 2> Cfg256w8b;  // 8 wavefronts, 64x128 each
+typedef TileCfg<256, 256, 32, 2, 4, 4> Cfg256w8k32;  // 8 wavefronts, 4 x 32-deep slabs, spread refill
 
-template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT>
+template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false>
 static hipError_t launch_epi(const GemmParams& p, hipStream_t stream) {
   static bool attr_set = false;
-  auto kern = gemm_nt_kernel<Cfg, HAS_D, HAS_C, HAS_CT>;
+  auto kern = gemm_nt_kernel<Cfg, HAS_D, HAS_C, HAS_CT, QK>;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        Cfg::LDS_BYTES);
@@ -377,6 +436,13 @@ template <class Cfg>
 static hipError_t launch_cfg(const GemmParams& p, hipStream_t stream) {
   if (p.M % Cfg::BM || p.N % Cfg::BN || p.K % (Cfg::BK * Cfg::NSTAGE)) return hipErrorInvalidValue;
   const bool d = p.D != nullptr, c = p.C != nullptr, ct = p.Ct != nullptr;
+  if (p.q_kmajor) {
+    if (p.tri) return hipErrorInvalidValue;
+    if (!d && c && !ct) return launch_epi<Cfg, false, true, false, true>(p, stream);  // X' = B X
+    if (!d && !c && ct) return launch_epi<Cfg, false, false, true, true>(p, stream);  // (B X)^T only
+    if (d && c && !ct) return launch_epi<Cfg, true, true, false, true>(p, stream);    // a X + B X
+    return hipErrorInvalidValue;
+  }
   if (!d && c && ct) return launch_epi<Cfg, false, true, true>(p, stream);   // A = X X^T
   if (d && c && ct) return launch_epi<Cfg, true, true, true>(p, stream);     // B, X' (both layouts)
   if (d && c && !ct) return launch_epi<Cfg, true, true, false>(p, stream);   // last X'
@@ -419,6 +485,7 @@ hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) 
     case 2: return launch_cfg<Cfg256k32>(p, stream);
     case 3: return launch_cfg<Cfg256w8>(p, stream);
     case 4: return launch_cfg<Cfg256w8b>(p, stream);
+    case 5: return launch_cfg<Cfg256w8k32>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -11,7 +11,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from ._lib import DION_BF16, DION_F32, DION_NS_GRAM, check, ptr_table
+from ._lib import DION_BF16, DION_F32, DION_NS_GRAM, DION_NS_XONLY, check, ptr_table
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -130,9 +130,9 @@ def ns_line_2(A: Tensor, alpha: float, beta: float, *, out: Optional[Tensor] = N
 def ns_line_3(B: Tensor, X: Tensor, a: float, *, out: Optional[Tensor] = None) -> Tensor:
     """``a * X + B @ X`` for symmetric ``B``.
 
-    Mirrors ``ns_line_3`` of the reference (dion/newton_schulz_triton.py:450-491).  The kernel
-    wants X with the reduction dimension contiguous, so X^T is materialised here; the whole-NS
-    driver keeps both layouts alive instead.
+    Mirrors ``ns_line_3`` of the reference (dion/newton_schulz_triton.py:450-491).  X is read as it
+    lies (reduction index along rows, transposing LDS reads in the kernel); the whole-NS driver
+    carries X^T alongside instead, which loads faster.
     """
     _check_bf16(B, "B")
     _check_bf16(X, "X")
@@ -143,11 +143,10 @@ def ns_line_3(B: Tensor, X: Tensor, a: float, *, out: Optional[Tensor] = None) -
     b, m, n = X3.shape
     Bp = _pad128(B3)
     Xp = _pad128(X3)
-    Xtp = Xp.transpose(-2, -1).contiguous()
     mp, np_ = Xp.shape[-2:]
     res = torch.empty(b, mp, np_, dtype=torch.bfloat16, device=X.device)
     lib = _lib.load()
-    check(lib.dion_ns_line_3(Bp.data_ptr(), Xp.data_ptr(), Xtp.data_ptr(), res.data_ptr(), None, b, mp,
+    check(lib.dion_ns_line_3(Bp.data_ptr(), Xp.data_ptr(), None, res.data_ptr(), None, b, mp,
                              np_, float(a), _stream_handle(X.device)), "ns_line_3")
     res = res[:, :m, :n]
     if squeeze:
@@ -159,11 +158,12 @@ def ns_line_3(B: Tensor, X: Tensor, a: float, *, out: Optional[Tensor] = None) -
 
 
 def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: float, epsilon: float,
-                     gram: bool = False, gram_reset: int = 0) -> Tensor:
+                     gram: bool = False, gram_reset: int = 0, x_only: bool = False) -> Tensor:
     """Batched Newton-Schulz / Polar-Express orthogonalization of ``G[..., rows, cols]``.
 
     X0 = bf16(G) / (||bf16(G)||_F * norm_scale + epsilon), then ``len(coeffs)`` quintic
     iterations on the orientation with rows <= cols; result is bf16 with the shape of ``G``.
+    ``x_only`` keeps a single copy of X between iterations (smaller workspace, slower GEMM loads).
     """
     _require_gpu(G, "G")
     if G.ndim < 2:
@@ -182,7 +182,7 @@ def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: f
         raise ValueError("coeffs must be (a, b, c) triples")
     n_iters = len(flat) // 3
     carr = (_lib.ctypes.c_float * max(1, len(flat)))(*flat)
-    flags = DION_NS_GRAM if gram else 0
+    flags = (DION_NS_GRAM if gram else 0) | (DION_NS_XONLY if x_only else 0)
     lib = _lib.load()
     nbytes = lib.dion_ns_workspace_bytes(batch, rows, cols, flags)
     ws = _workspace(G.device, nbytes)

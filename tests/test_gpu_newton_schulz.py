@@ -143,6 +143,23 @@ def test_ns5_vs_oracle(shape):
     assert float((out.float().cpu() - ref.float()).abs().max()) < 0.02
 
 
+@pytest.mark.parametrize("shape", [(256, 1024), (2, 768, 3072), (2, 3072, 768), (3, 100, 300), (2, 1000, 130)])
+@pytest.mark.parametrize("gram", [False, True])
+def test_x_only_form_is_bit_identical(shape, gram):
+    """DION_NS_XONLY changes which copy of X the X' = B X kernel reads (transposing LDS reads of X
+    instead of plain reads of X^T), not the arithmetic: same MFMA operands, same accumulation
+    order, so the results must agree bit for bit."""
+    from dion_amd import ops
+    from dion_amd.newton_schulz import POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY
+
+    torch.manual_seed(11)
+    G = torch.randn(shape, device=DEV).to(torch.bfloat16)
+    kw = dict(gram=gram, gram_reset=2 if gram else 0)
+    a = ops.ns_orthogonalize(G, POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 1e-7, **kw)
+    b = ops.ns_orthogonalize(G, POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 1e-7, x_only=True, **kw)
+    assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("shape", [(64, 128), (128, 64), (128, 128), (4, 64, 128), (4, 128, 64)])
 def test_orthogonality_bound(shape):
     """max|X X^T - I| < 0.15 on the reference's shapes and seed (tests/test_polar_express.py:10-42)."""
