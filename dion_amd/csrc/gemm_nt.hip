@@ -26,9 +26,14 @@ namespace dion {
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int NSTAGE_>
+// VG_: operand slabs travel global -> VGPR -> LDS (plain 16-byte loads, ds_write_b128 one slab
+// later) instead of the direct-to-LDS DMA: every load gets a full slab of latency slack and the
+// kernel places the LDS writes itself, between MFMAs.
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int NSTAGE_, bool VG_ = false>
 struct TileCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, NSTAGE = NSTAGE_;
+  static constexpr bool VG = VG_;
+  static_assert(!VG_ || NSTAGE_ == 2, "register staging is written for a two-slot ring");
   static constexpr int NT = WM * WN * 64;
   static constexpr int CPR = BK / 8;            // 16-byte chunks per tile row
   static constexpr int ROWS_PER_LOAD = NT / CPR; // tile rows covered by one load instruction
@@ -217,6 +222,19 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
     }
   };
 
+  // Register-staged transport (Cfg::VG): stage_reg[j] holds load j of the slab after next.
+  typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+  u32x4 stage_reg[Cfg::VG ? LPS : 1];
+  auto stage_fetch = [&](int kt, int j) {
+    const int k = kt < KT ? kt : KT - 1;
+    const char* src = j < Cfg::P_LOADS ? gP + (int64_t)k * (BK * 2) + (offP + j * stepP)
+                                       : gQ + k * slabQ + (offQ + (j - Cfg::P_LOADS) * stepQ);
+    stage_reg[j] = *(const u32x4*)src;
+  };
+  auto stage_store = [&](int buf, int j) {
+    *(u32x4*)(lds + buf * Cfg::STAGE_BYTES + j * (Cfg::NT * 16) + tid * 16) = stage_reg[j];
+  };
+
   // ---- LDS -> register fragment addressing (per lane, per 16-wide k slice).
   const int frow = lane & 31;
   const int fhalf = lane >> 5;
@@ -276,15 +294,28 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
 
   // ---- prologue: fill NSTAGE-1 ring slots, wait for slab 0, read its first fragments, start the
   // last free slot.
+  if (Cfg::VG) {
 #pragma unroll
-  for (int s = 0; s < NSTAGE - 1; ++s)
+    for (int j = 0; j < LPS; ++j) stage_fetch(0, j);
 #pragma unroll
-    for (int j = 0; j < LPS; ++j) issue_load(s, s, j);
-  pipeline_barrier<(NSTAGE - 2) * LPS>();
+    for (int j = 0; j < LPS; ++j) {
+      stage_store(0, j);
+      stage_fetch(1, j);
+    }
+    pipeline_barrier<63>();
 #pragma unroll
-  for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
+    for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
+  } else {
 #pragma unroll
-  for (int j = 0; j < LPW; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
+    for (int s = 0; s < NSTAGE - 1; ++s)
+#pragma unroll
+      for (int j = 0; j < LPS; ++j) issue_load(s, s, j);
+    pipeline_barrier<(NSTAGE - 2) * LPS>();
+#pragma unroll
+    for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
+  }
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- main loop.  Slices run back to back across slab boundaries: while the MFMAs of one slice
@@ -298,7 +329,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
       for (int kk = 0; kk < KK; ++kk) {
         const int cur = kk & 1, nxt = cur ^ 1;
         const bool last = (kk == KK - 1);
-        if (last) pipeline_barrier<(NSTAGE - 2) * LPS>();  // slab kt+1 landed, slab kt fully read
+        // slab kt+1 landed (DMA) / written by every wavefront (VG), slab kt fully read
+        if (last) pipeline_barrier<Cfg::VG ? 63 : (NSTAGE - 2) * LPS>();
 #pragma unroll
         for (int q = 0; q < NM; ++q) {
 #ifdef DION_DBG_NO_MFMA
@@ -312,7 +344,18 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
             if (last) read_frag((s + 1) % NSTAGE, 0, nxt, r);
             else read_frag(s, kk + 1, nxt, r);
           }
-          if (SPREAD) {
+          if (Cfg::VG) {
+            // slices 0..KK-2 of slab kt: write slab kt+1 (fetched during slab kt-1) into the other
+            // slot, then fetch slab kt+2 into the freed registers, at even MFMA spacing
+            constexpr int SLOTS = (KK - 1) * NM;
+            constexpr int STRIDE = SLOTS / LPS > 0 ? SLOTS / LPS : 1;
+            static_assert(!Cfg::VG || SLOTS >= LPS, "not enough MFMA slots for the staged stores");
+            const int t = kk * NM + q;
+            if (!last && t % STRIDE == 0 && t / STRIDE < LPS) {
+              stage_store((s + 1) % NSTAGE, t / STRIDE);
+              stage_fetch(kt0 + s + 2, t / STRIDE);
+            }
+          } else if (SPREAD) {
             if (q % QPL == QPL / 2) {
               const int jw = q / QPL;
               if (last) issue_load(kt0 + s + NSTAGE, s, jw);
@@ -328,7 +371,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
       }
     }
   }
-  wait_vmcnt<0>();  // drain the redundant tail refills before LDS is reused / the wave exits
+  if (!Cfg::VG) wait_vmcnt<0>();  // drain the redundant tail refills before LDS is reused / the wave exits
 
   // ---- epilogue.  Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4,
   // column l%32 of its 32x32 tile.  Whole tiles are stored: destinations are padded to the tile.
@@ -412,6 +455,8 @@ typedef TileCfg<256, 256, 32, 2, 2, 4> Cfg256k32;
 typedef TileCfg<256, 256, 64, 2, 4, 2> Cfg256w8;   // 8 wavefronts, 128x64 each: two per SIMD
 typedef TileCfg<256, 256, 64, 4, 2, 2> Cfg256w8b;  // 8 wavefronts, 64x128 each
 typedef TileCfg<256, 256, 32, 2, 4, 4> Cfg256w8k32;  // 8 wavefronts, 4 x 32-deep slabs, spread refill
+typedef TileCfg<256, 256, 64, 2, 4, 2, true> Cfg256w8vg;  // 8 wavefronts, register-staged operands
+typedef TileCfg<128, 128, 64, 2, 2, 2, true> Cfg128vg;
 
 template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false>
 static hipError_t launch_epi(const GemmParams& p, hipStream_t stream) {
@@ -477,6 +522,17 @@ hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) 
       return e ? atoi(e) : -1;
     }();
     if (forced >= 0 && variant == 3) variant = forced;
+    static const int forced128 = [] {
+      const char* e = getenv("DION_GEMM_VARIANT128");
+      return e ? atoi(e) : -1;
+    }();
+    if (forced128 >= 0 && variant == 1) variant = forced128;
+    // The K-major second operand loads better through registers than through the DMA.
+    static const bool qk_vg = [] {
+      const char* e = getenv("DION_QK_VG");
+      return !(e && atoi(e) == 0);
+    }();
+    if (p.q_kmajor && qk_vg) variant = variant == 3 ? 6 : (variant == 1 ? 8 : variant);
   }
   if (p.tri && (p.M != p.N)) return hipErrorInvalidValue;
   switch (variant) {
@@ -486,6 +542,8 @@ hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) 
     case 3: return launch_cfg<Cfg256w8>(p, stream);
     case 4: return launch_cfg<Cfg256w8b>(p, stream);
     case 5: return launch_cfg<Cfg256w8k32>(p, stream);
+    case 6: return launch_cfg<Cfg256w8vg>(p, stream);
+    case 8: return launch_cfg<Cfg128vg>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }
