@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libdion_hip.so")
 DION_BF16 = 0
 DION_F32 = 1
 DION_NS_GRAM = 1
-DION_NS_XONLY = 2
+DION_NS_CARRY_XT = 2
 
 _u64p = ctypes.POINTER(ctypes.c_uint64)
 _f32p = ctypes.POINTER(c_float)

@@ -171,10 +171,10 @@ NsPlan make_plan(int batch, int rows, int cols, int flags) {
   pl.a_bytes = align256((size_t)batch * pl.mp * pl.lda * 2);
   pl.partial_bytes = align256((size_t)batch * pl.nblk * 4);
   pl.inv_bytes = align256((size_t)batch * 4);
-  // X, Xt ping-pong pairs (X-only form: the X pair and one X^T for a padded tall result);
+  // X, Xt ping-pong pairs (default X-only form: the X pair and one X^T for a padded tall result);
   // A, B (+ Q, Z, T for the Gram recurrence)
   const int n_sq = (flags & DION_NS_GRAM) ? 6 : 2;
-  const int n_x = (flags & DION_NS_XONLY) ? 3 : 4;
+  const int n_x = (flags & DION_NS_CARRY_XT) ? 4 : 3;
   pl.total = n_x * pl.x_bytes + n_sq * pl.a_bytes + pl.partial_bytes + pl.inv_bytes;
   return pl;
 }
@@ -196,7 +196,7 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   if (batch == 0 || rows == 0 || cols == 0) return DION_OK;
   if (!in || !out || (n_iters > 0 && !coeffs))
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: null argument");
-  if (flags & ~(DION_NS_GRAM | DION_NS_XONLY)) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
+  if (flags & ~(DION_NS_GRAM | DION_NS_CARRY_XT)) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
   hipStream_t st = (hipStream_t)stream;
   if (!(flags & DION_NS_GRAM) && n_iters <= kMaxSmallIters && ns_small_fits(rows, cols) &&
       !getenv("DION_NO_SMALL_KERNEL")) {
@@ -222,10 +222,10 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   X[0] = (bf16_t*)w; w += pl.x_bytes;
   X[1] = (bf16_t*)w; w += pl.x_bytes;
   Xt[0] = (bf16_t*)w; w += pl.x_bytes;
-  if (flags & DION_NS_XONLY) {
-    Xt[1] = Xt[0];  // only ever written by the last product
-  } else {
+  if (flags & DION_NS_CARRY_XT) {
     Xt[1] = (bf16_t*)w; w += pl.x_bytes;
+  } else {
+    Xt[1] = Xt[0];  // only ever written by the last product
   }
   bf16_t* sq[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};  // m x m scratch
   for (int i = 0; i < ((flags & DION_NS_GRAM) ? 6 : 2); ++i) {
@@ -241,10 +241,9 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
   HIP_TRY(launch_frobenius_inv(in, in_dtype, batch, (int64_t)rows * cols, norm_scale, eps, partial,
                                pl.nblk, inv, st),
           "frobenius norm");
-  // DION_NS_XONLY: X' = B X reads X itself (reduction index along rows) and no X^T is carried.
-  // The default form (X and X^T side by side) is the faster one: its operand tiles are contiguous
-  // along the reduction index in memory.
-  const bool nn = (flags & DION_NS_XONLY) != 0;
+  // Default: X' = B X reads X itself (reduction index along rows) and no X^T is carried.
+  // DION_NS_CARRY_XT keeps X and X^T side by side instead.
+  const bool nn = (flags & DION_NS_CARRY_XT) == 0;
   if (pl.tall)
     HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, nn ? nullptr : Xt[0], np, mp, ldxt, sXt,
                               X[0], ldx, sX, st),

@@ -11,7 +11,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from ._lib import DION_BF16, DION_F32, DION_NS_GRAM, DION_NS_XONLY, check, ptr_table
+from ._lib import DION_BF16, DION_F32, DION_NS_GRAM, DION_NS_CARRY_XT, check, ptr_table
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -131,8 +131,8 @@ def ns_line_3(B: Tensor, X: Tensor, a: float, *, out: Optional[Tensor] = None) -
     """``a * X + B @ X`` for symmetric ``B``.
 
     Mirrors ``ns_line_3`` of the reference (dion/newton_schulz_triton.py:450-491).  X is read as it
-    lies (reduction index along rows, transposing LDS reads in the kernel); the whole-NS driver
-    carries X^T alongside instead, which loads faster.
+    lies (reduction index along rows, transposing LDS reads in the kernel), as in the whole-NS
+    driver.
     """
     _check_bf16(B, "B")
     _check_bf16(X, "X")
@@ -158,12 +158,12 @@ def ns_line_3(B: Tensor, X: Tensor, a: float, *, out: Optional[Tensor] = None) -
 
 
 def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: float, epsilon: float,
-                     gram: bool = False, gram_reset: int = 0, x_only: bool = False) -> Tensor:
+                     gram: bool = False, gram_reset: int = 0, carry_xt: bool = False) -> Tensor:
     """Batched Newton-Schulz / Polar-Express orthogonalization of ``G[..., rows, cols]``.
 
     X0 = bf16(G) / (||bf16(G)||_F * norm_scale + epsilon), then ``len(coeffs)`` quintic
     iterations on the orientation with rows <= cols; result is bf16 with the shape of ``G``.
-    ``x_only`` keeps a single copy of X between iterations (smaller workspace, slower GEMM loads).
+    ``carry_xt`` keeps X and X^T side by side between iterations instead of X alone (same result).
     """
     _require_gpu(G, "G")
     if G.ndim < 2:
@@ -182,7 +182,7 @@ def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: f
         raise ValueError("coeffs must be (a, b, c) triples")
     n_iters = len(flat) // 3
     carr = (_lib.ctypes.c_float * max(1, len(flat)))(*flat)
-    flags = (DION_NS_GRAM if gram else 0) | (DION_NS_XONLY if x_only else 0)
+    flags = (DION_NS_GRAM if gram else 0) | (DION_NS_CARRY_XT if carry_xt else 0)
     lib = _lib.load()
     nbytes = lib.dion_ns_workspace_bytes(batch, rows, cols, flags)
     ws = _workspace(G.device, nbytes)

@@ -75,10 +75,12 @@ int dion_ns_line_3(const void* B, const void* X, const void* Xt, void* C, void* 
  * workspace: device scratch of at least dion_ns_workspace_bytes() bytes, 256-byte aligned.
  * ------------------------------------------------------------------------------------------ */
 #define DION_NS_GRAM 1
-/* DION_NS_XONLY: keep only X between iterations (X' = B X reads X with the reduction index along
- * rows through transposing LDS reads) instead of X and X^T side by side.  Same arithmetic, same
- * result; slower GEMM operand loads, one fewer store per iteration. */
-#define DION_NS_XONLY 2
+/* By default only X is kept between iterations: X' = B X reads X with the reduction index along
+ * rows (register-staged loads, transposing LDS reads).  DION_NS_CARRY_XT selects the other form,
+ * X and X^T carried side by side with both GEMM operands contiguous along the reduction index
+ * (one more store per iteration, a workspace one X larger).  Same arithmetic, bit-identical
+ * result. */
+#define DION_NS_CARRY_XT 2
 size_t dion_ns_workspace_bytes(int batch, int rows, int cols, int flags);
 int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, int rows, int cols,
                           const float* coeffs, int n_iters, float norm_scale, float eps, int flags,

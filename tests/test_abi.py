@@ -35,8 +35,9 @@ def test_library_exports_every_declared_symbol():
     # pure host entry points
     assert lib.dion_ns_workspace_bytes(0, 128, 128, 0) == 0
     n = lib.dion_ns_workspace_bytes(2, 768, 3072, 0)
-    assert n >= 2 * 768 * 3072 * 2 * 4
+    assert n >= 2 * 768 * 3072 * 2 * 3  # X ping-pong pair + one X^T
     assert lib.dion_ns_workspace_bytes(2, 3072, 768, 0) == n
+    assert lib.dion_ns_workspace_bytes(2, 768, 3072, _lib.DION_NS_CARRY_XT) >= n + 2 * 768 * 3072 * 2
 
 
 def test_missing_library_is_a_hard_error(monkeypatch, tmp_path):

@@ -145,9 +145,9 @@ def test_ns5_vs_oracle(shape):
 
 @pytest.mark.parametrize("shape", [(256, 1024), (2, 768, 3072), (2, 3072, 768), (3, 100, 300), (2, 1000, 130)])
 @pytest.mark.parametrize("gram", [False, True])
-def test_x_only_form_is_bit_identical(shape, gram):
-    """DION_NS_XONLY changes which copy of X the X' = B X kernel reads (transposing LDS reads of X
-    instead of plain reads of X^T), not the arithmetic: same MFMA operands, same accumulation
+def test_carry_xt_form_is_bit_identical(shape, gram):
+    """DION_NS_CARRY_XT changes which copy of X the X' = B X kernel reads (plain reads of X^T
+    instead of transposing LDS reads of X), not the arithmetic: same MFMA operands, same accumulation
     order, so the results must agree bit for bit."""
     from dion_amd import ops
     from dion_amd.newton_schulz import POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY
@@ -156,7 +156,7 @@ def test_x_only_form_is_bit_identical(shape, gram):
     G = torch.randn(shape, device=DEV).to(torch.bfloat16)
     kw = dict(gram=gram, gram_reset=2 if gram else 0)
     a = ops.ns_orthogonalize(G, POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 1e-7, **kw)
-    b = ops.ns_orthogonalize(G, POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 1e-7, x_only=True, **kw)
+    b = ops.ns_orthogonalize(G, POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 1e-7, carry_xt=True, **kw)
     assert torch.equal(a, b)
 
 
