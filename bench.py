@@ -100,7 +100,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama3_8b", choices=sorted(WORKLOADS))
     ap.add_argument("--ns", default="ns5", choices=["ns5", "polar_express", "gram"])
-    ap.add_argument("--optimizer", default="muon", choices=["muon", "normuon", "dion2"])
+    ap.add_argument("--optimizer", default="muon", choices=["muon", "normuon", "dion2", "nordion2"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     args = ap.parse_args()
@@ -116,7 +116,7 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
-    from dion import Dion2, Muon, NorMuon
+    from dion import Dion2, Muon, NorDion2, NorMuon
     from dion_amd import _lib, ops
 
     dev = torch.device("cuda:0")
@@ -145,6 +145,8 @@ def main() -> int:
         if args.optimizer == "dion2":  # NS runs on the selected quarter of the shorter dimension
             k = -(-min(r, c) * 25 // 100)
             r, c = (k, c) if r <= c else (r, k)
+        elif args.optimizer == "nordion2":  # always the selected quarter of the rows
+            r = -(-r * 25 // 100)
         total_flops += count * mult * ns_flops(r, c)
         total_elems += count * rows * cols
     ns_kw = dict(use_polar_express=(args.ns == "polar_express"), use_gram_newton_schulz=(args.ns == "gram"))
@@ -153,6 +155,9 @@ def main() -> int:
     elif args.optimizer == "normuon":
         opt = NorMuon(groups, lr=0.02, mu=0.95, muon_beta2=0.95, nesterov=True, weight_decay=0.01,
                       adjust_lr="spectral_norm", **ns_kw)
+    elif args.optimizer == "nordion2":
+        opt = NorDion2(groups, lr=0.02, fraction=fraction, mu=0.95, muon_beta2=0.95, weight_decay=0.01,
+                       adjust_lr="spectral_norm", **ns_kw)
     else:
         opt = Dion2(groups, lr=0.02, fraction=fraction, ef_decay=0.95, weight_decay=0.01,
                     adjust_lr="spectral_norm", **ns_kw)
@@ -182,8 +187,9 @@ def main() -> int:
         "data": "synthetic",
         "config": {
             "workload": f"{args.workload}: full {type(opt).__name__}.step() ({args.ns}, wd 0.01, lr 0.02"
-                        + (", fraction 0.25, ef_decay 0.95" if args.optimizer == "dion2" else ", nesterov mu=0.95")
-                        + (", muon_beta2 0.95" if args.optimizer == "normuon" else "") + ") over "
+                        + ({"dion2": ", fraction 0.25, ef_decay 0.95", "nordion2": ", fraction 0.25, mu 0.95"}
+                           .get(args.optimizer, ", nesterov mu=0.95"))
+                        + (", muon_beta2 0.95" if args.optimizer in ("normuon", "nordion2") else "") + ") over "
                         + ", ".join(f"{c}x({r}x{k})" for _n, r, k, c in spec),
             "matrices": sum(c for *_x, c in spec),
             "elements": total_elems,

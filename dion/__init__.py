@@ -5,5 +5,7 @@ import dion_amd as _impl
 Muon = _impl.Muon
 NorMuon = _impl.NorMuon
 Dion2 = _impl.Dion2
+NorDion2 = _impl.NorDion2
+Dion3 = _impl.Dion3  # alias of NorDion2 (dion/__init__.py:10)
 
-__all__ = ["Muon", "NorMuon", "Dion2"]
+__all__ = ["Muon", "NorMuon", "Dion2", "NorDion2", "Dion3"]

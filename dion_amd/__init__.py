@@ -1,4 +1,4 @@
-"""MI355X-native Muon / NorMuon / Dion2 optimizer-step kernels behind the microsoft/dion API."""
+"""MI355X-native Muon / NorMuon / Dion2 / NorDion2 optimizer-step kernels behind the microsoft/dion API."""
 from .newton_schulz import (  # noqa: F401
     gram_newton_schulz,
     newton_schulz_triton,
@@ -11,12 +11,14 @@ from .newton_schulz import (  # noqa: F401
     zeropower_via_newtonschulz5,
 )
 
-from .optimizers import Dion2, Muon, NorMuon  # noqa: E402,F401
+from .optimizers import Dion2, Dion3, Muon, NorDion2, NorMuon  # noqa: E402,F401
 
 __all__ = [
     "Muon",
     "NorMuon",
     "Dion2",
+    "NorDion2",
+    "Dion3",
     "gram_newton_schulz",
     "newton_schulz_triton",
     "ns_line_1",

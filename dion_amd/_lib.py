@@ -35,6 +35,8 @@ SIGNATURES = {
                                c_float, c_void_p, c_float, c_int, c_void_p]),
     "dion_normuon_stats": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_float, c_void_p,
                                    c_void_p, c_void_p]),
+    "dion_normuon_stats_selected": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_void_p, c_int,
+                                            c_float, c_void_p, c_void_p]),
     "dion_dion2_accumulate_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "dion_dion2_accumulate": (c_int, [_u64p, c_int, _u64p, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -42,7 +44,7 @@ SIGNATURES = {
     "dion_dion2_gather": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
                                   c_void_p, c_void_p]),
     "dion_dion2_post": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
-                                c_void_p, c_float, c_void_p, c_float, c_void_p]),
+                                c_void_p, c_void_p, c_float, c_void_p, c_float, c_void_p]),
 }
 
 _lib = None

@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 2; }
+extern "C" int dion_abi_version(void) { return 3; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -478,14 +478,13 @@ extern "C" int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype
   return DION_OK;
 }
 
-extern "C" int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr,
-                                  int rows, int cols, float beta2, float* row_scale, float* scratch,
-                                  void* stream) {
-  (void)scratch;
-  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0)
-    return fail(DION_E_INVALID, "dion_normuon_stats: bad size");
+static int normuon_stats_impl(const char* who, const void* U, const uint64_t* V_ptrs, int n,
+                              int mats_per_ptr, int rows, int cols, const int32_t* row_idx, int v_rows,
+                              float beta2, float* row_scale, void* stream) {
+  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || v_rows < rows)
+    return fail(DION_E_INVALID, "%s: bad size", who);
   if (n == 0 || rows == 0 || cols == 0) return DION_OK;
-  if (!U || !V_ptrs || !row_scale) return fail(DION_E_INVALID, "dion_normuon_stats: null argument");
+  if (!U || !V_ptrs || !row_scale) return fail(DION_E_INVALID, "%s: null argument", who);
   const float w = 1.0f - beta2;
   for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
     const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
@@ -493,11 +492,27 @@ extern "C" int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, 
     fill_tab(v, V_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
     HIP_TRY(launch_normuon_stats((const bf16_t*)U + mat0 * rows * cols, v, c * mats_per_ptr, 0,
-                                 mats_per_ptr, rows, cols, w, row_scale + mat0 * rows,
-                                 (hipStream_t)stream),
-            "dion_normuon_stats");
+                                 mats_per_ptr, rows, cols, row_idx ? row_idx + mat0 * rows : nullptr,
+                                 v_rows, w, row_scale + mat0 * rows, (hipStream_t)stream),
+            who);
   }
   return DION_OK;
+}
+
+extern "C" int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr,
+                                  int rows, int cols, float beta2, float* row_scale, float* scratch,
+                                  void* stream) {
+  (void)scratch;
+  return normuon_stats_impl("dion_normuon_stats", U, V_ptrs, n, mats_per_ptr, rows, cols, nullptr, rows,
+                            beta2, row_scale, stream);
+}
+
+extern "C" int dion_normuon_stats_selected(const void* U, const uint64_t* V_ptrs, int n,
+                                           int mats_per_ptr, int k, int cols, const int32_t* row_idx,
+                                           int v_rows, float beta2, float* row_scale, void* stream) {
+  if (!row_idx) return fail(DION_E_INVALID, "dion_normuon_stats_selected: null row_idx");
+  return normuon_stats_impl("dion_normuon_stats_selected", U, V_ptrs, n, mats_per_ptr, k, cols, row_idx,
+                            v_rows, beta2, row_scale, stream);
 }
 
 static int check_select_dim(const char* who, int select_dim) {
@@ -584,9 +599,11 @@ extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr
 
 extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, int cols,
                                int select_dim, const void* U_sel, int k, const int32_t* map,
-                               const float* lr_dev, float adj_ratio, const float* wd_dev,
-                               float wd_host, void* stream) {
+                               const float* row_scale, const float* lr_dev, float adj_ratio,
+                               const float* wd_dev, float wd_host, void* stream) {
   if (int rc = check_select_dim("dion_dion2_post", select_dim)) return rc;
+  if (row_scale && select_dim != -2)
+    return fail(DION_E_INVALID, "dion_dion2_post: row_scale needs select_dim == -2");
   if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || k < 0)
     return fail(DION_E_INVALID, "dion_dion2_post: bad size");
   if (n == 0 || rows == 0 || cols == 0) return DION_OK;
@@ -602,8 +619,9 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
     fill_tab(x, X_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
     HIP_TRY(launch_dion2_post(x, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
-                              (const bf16_t*)U_sel + mat0 * sel_numel, k, map + mat0 * dim, lr_dev,
-                              adj_ratio, wd_dev, wd_host, vec4, (hipStream_t)stream),
+                              (const bf16_t*)U_sel + mat0 * sel_numel, k, map + mat0 * dim,
+                              row_scale ? row_scale + mat0 * k : nullptr, lr_dev, adj_ratio, wd_dev,
+                              wd_host, vec4, (hipStream_t)stream),
             "dion_dion2_post");
   }
   return DION_OK;

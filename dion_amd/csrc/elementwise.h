@@ -39,8 +39,8 @@ hipError_t launch_muon_post(const PtrTab& X, const void* U, int u_dtype, int n, 
                             const float* wd_dev, float wd_host, int cautious, bool vec,
                             hipStream_t st);
 hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int n_mat, int mat0,
-                                int mats_per_ptr, int rows, int cols, float w, float* row_scale,
-                                hipStream_t st);
+                                int mats_per_ptr, int rows, int cols, const int32_t* row_idx,
+                                int v_rows, float w, float* row_scale, hipStream_t st);
 hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int n_mat,
                                    int mats_per_ptr, int rows, int cols, int select_rows,
                                    float* norms, bool vec4, float* slab_scratch, int slabs,
@@ -54,7 +54,7 @@ hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int
                                bool vec4, hipStream_t st);
 hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
                              int select_rows, const bf16_t* U, int k, const int32_t* map,
-                             const float* lr_dev, float adj_ratio, const float* wd_dev,
-                             float wd_host, bool vec4, hipStream_t st);
+                             const float* row_scale, const float* lr_dev, float adj_ratio,
+                             const float* wd_dev, float wd_host, bool vec4, hipStream_t st);
 
 }  // namespace dion

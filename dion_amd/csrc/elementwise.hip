@@ -445,10 +445,15 @@ hipError_t launch_muon_post(const PtrTab& X, const void* U, int u_dtype, int n, 
 // ------------------------------------------------------------------------------------------
 // NorMuon: per-row second moment EMA and the Frobenius-preserving row scales.
 // ------------------------------------------------------------------------------------------
+// Row r of matrix mat keeps its second moment at V[mat][row_idx ? row_idx[mat][r] : r]; V holds
+// v_rows entries per matrix (v_rows == rows without row_idx).  The indirection serves updates made
+// of selected rows only (NorDion2, dion/nordion2.py:430-447).
 // Pass 1: one wavefront per row.  V <- lerp(V, mean(u^2), w);  tmp[row] = sum(u^2).
 __global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restrict__ U, PtrTab V,
                                                            int mats_per_ptr, int rows, int cols,
-                                                           float w, float* __restrict__ rowsq) {
+                                                           const int32_t* __restrict__ row_idx,
+                                                           int v_rows, float w,
+                                                           float* __restrict__ rowsq) {
   const int mat = blockIdx.y;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -474,7 +479,8 @@ __global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restr
   }
   s = wave_sum(s);
   if (lane == 0) {
-    float* v = (float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows + row;
+    const int vr = row_idx ? row_idx[(int64_t)mat * rows + row] : row;
+    float* v = (float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * v_rows + vr;
     const float mean = s / (float)cols;
     const float vo = *v;
     *v = vo + w * (mean - vo);  // torch.lerp for weight < 0.5
@@ -485,15 +491,17 @@ __global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restr
 // Pass 2: one block per matrix.  scale[row] = (1/d) * sqrt(S1) / max(sqrt(S2), 1e-8) with
 // d = sqrt(V)+1e-8, S1 = sum rowsq, S2 = sum rowsq/d^2.  In place over rowsq.
 __global__ __launch_bounds__(1024) void normuon_scale_kernel(PtrTab V, int mats_per_ptr, int rows,
-                                                             float* __restrict__ scale) {
+                                                             const int32_t* __restrict__ row_idx,
+                                                             int v_rows, float* __restrict__ scale) {
   __shared__ float red[16];
   const int mat = blockIdx.x;
-  const float* v = (const float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows;
+  const float* v = (const float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * v_rows;
+  const int32_t* ri = row_idx ? row_idx + (int64_t)mat * rows : nullptr;
   float* sc = scale + (int64_t)mat * rows;
   float s1 = 0.f, s2 = 0.f;
   for (int r = threadIdx.x; r < rows; r += 1024) {
     const float q = sc[r];
-    const float inv = 1.0f / (sqrtf(v[r]) + 1e-8f);
+    const float inv = 1.0f / (sqrtf(v[ri ? ri[r] : r]) + 1e-8f);
     s1 += q;
     s2 += q * inv * inv;
   }
@@ -502,20 +510,21 @@ __global__ __launch_bounds__(1024) void normuon_scale_kernel(PtrTab V, int mats_
   const float ratio = sqrtf(s1) / fmaxf(sqrtf(s2), 1e-8f);
   __syncthreads();
   for (int r = threadIdx.x; r < rows; r += 1024) {
-    const float inv = 1.0f / (sqrtf(v[r]) + 1e-8f);
+    const float inv = 1.0f / (sqrtf(v[ri ? ri[r] : r]) + 1e-8f);
     sc[r] = inv * ratio;
   }
 }
 
 hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int n_mat, int mat0,
-                                int mats_per_ptr, int rows, int cols, float w, float* row_scale,
-                                hipStream_t st) {
-  // U / row_scale are offset to matrix mat0 by the caller; V is the table chunk covering them.
+                                int mats_per_ptr, int rows, int cols, const int32_t* row_idx,
+                                int v_rows, float w, float* row_scale, hipStream_t st) {
+  // U / row_scale / row_idx are offset to matrix mat0 by the caller; V is the table chunk covering
+  // them.
   (void)mat0;
   hipLaunchKernelGGL(normuon_rows_kernel, dim3((rows + 3) / 4, n_mat), dim3(256), 0, st, U, V,
-                     mats_per_ptr, rows, cols, w, row_scale);
+                     mats_per_ptr, rows, cols, row_idx, v_rows, w, row_scale);
   hipLaunchKernelGGL(normuon_scale_kernel, dim3(n_mat), dim3(1024), 0, st, V, mats_per_ptr, rows,
-                     row_scale);
+                     row_idx, v_rows, row_scale);
   return hipGetLastError();
 }
 
@@ -848,6 +857,7 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
                                                          int cols, int select_rows,
                                                          const bf16_t* __restrict__ U, int k,
                                                          const int32_t* __restrict__ map,
+                                                         const float* __restrict__ row_scale,
                                                          const float* __restrict__ lr_dev,
                                                          float adj_ratio,
                                                          const float* __restrict__ wd_dev,
@@ -857,7 +867,8 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
   const float lr = *lr_dev;
   const float wd = wd_dev ? *wd_dev : wd_host;
   const float a = __fsub_rn(1.0f, __fmul_rn(lr, wd));
-  const float b = __fmul_rn(lr, adj_ratio);
+  const float b0 = __fmul_rn(lr, adj_ratio);
+  float b = b0;
   const int dim = select_rows ? rows : cols;
   const int32_t* mp = map + (int64_t)mat * dim;
   const bf16_t* u = U + (int64_t)mat * (select_rows ? (int64_t)k * cols : (int64_t)rows * k);
@@ -867,6 +878,8 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
     if (select_rows) {
       const int j = mp[r];
       const bf16_t* ur = u + (int64_t)(j < 0 ? 0 : j) * cols;
+      // per-row scale of the selected slice (rows selected only): u is multiplied by it first
+      if (row_scale && j >= 0) b = __fmul_rn(b0, row_scale[(int64_t)mat * k + j]);
       if (VEC) {
         for (int c = threadIdx.x * 4; c < cols; c += 1024) {
           float4 v = *(const float4*)(xr + c);
@@ -919,15 +932,15 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
 
 hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
                              int select_rows, const bf16_t* U, int k, const int32_t* map,
-                             const float* lr_dev, float adj_ratio, const float* wd_dev,
-                             float wd_host, bool vec4, hipStream_t st) {
+                             const float* row_scale, const float* lr_dev, float adj_ratio,
+                             const float* wd_dev, float wd_host, bool vec4, hipStream_t st) {
   dim3 grid((rows + 7) / 8, n_mat);
   if (vec4)
     hipLaunchKernelGGL(dion2_post_kernel<true>, grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols,
-                       select_rows, U, k, map, lr_dev, adj_ratio, wd_dev, wd_host);
+                       select_rows, U, k, map, row_scale, lr_dev, adj_ratio, wd_dev, wd_host);
   else
     hipLaunchKernelGGL(dion2_post_kernel<false>, grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols,
-                       select_rows, U, k, map, lr_dev, adj_ratio, wd_dev, wd_host);
+                       select_rows, U, k, map, row_scale, lr_dev, adj_ratio, wd_dev, wd_host);
   return hipGetLastError();
 }
 

@@ -277,6 +277,29 @@ def normuon_stats(U: Tensor, V: List[Tensor], beta2: float) -> Tensor:
     return scale
 
 
+def normuon_stats_selected(U: Tensor, V: List[Tensor], idx: Tensor, beta2: float) -> Tensor:
+    """NorMuon statistics for an update made of ``k`` selected rows per matrix: ``U [N, ..., k, cols]``
+    bf16, ``idx [n_mat, k]`` int32 (rows of the parameter), ``V[i]`` the full ``[..., rows, 1]`` fp32
+    buffers, of which only the selected entries are read and updated.  Returns the per-row scales
+    ``[n_mat, k]``.  Mirrors ``nordion2_normalize_selected_stacked`` (dion/nordion2.py:430-447)."""
+    n = len(V)
+    assert n > 0 and U.shape[0] == n
+    _check_bf16(U, "U")
+    k, cols = U.shape[-2], U.shape[-1]
+    n_mat = U.numel() // (k * cols)
+    mats_per_ptr = n_mat // n
+    v_rows = V[0].numel() // mats_per_ptr
+    vp = _list_ptrs(V, "V", torch.float32, mats_per_ptr * v_rows)
+    if idx.dtype != torch.int32 or not idx.is_contiguous() or idx.numel() != n_mat * k:
+        raise ValueError("idx must be a contiguous int32 tensor of n_mat * k entries")
+    scale = torch.empty(n_mat, k, dtype=torch.float32, device=U.device)
+    lib = _lib.load()
+    check(lib.dion_normuon_stats_selected(U.data_ptr(), vp, n, mats_per_ptr, k, cols, idx.data_ptr(), v_rows,
+                                          float(beta2), scale.data_ptr(), _stream_handle(U.device)),
+          "normuon_stats_selected")
+    return scale
+
+
 def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_decay: float):
     """``M += G``; pick the ``k`` slices of largest L1 norm along ``select_dim`` of every matrix; return
     (U_sel bf16 arena, idx int32 [n_mat, k] ascending, map int32 [n_mat, dim]) and decay the selected
@@ -314,9 +337,10 @@ def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_d
 
 
 def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: float, weight_decay,
-               select_dim: int) -> None:
+               select_dim: int, row_scale: Optional[Tensor] = None) -> None:
     """Fused ``x = (1 - lr*wd)*x - lr*adj_ratio*u[map]`` over every ``X[i]``.  Mirrors
-    ``dion2_post_orthogonalize_triton`` (dion/dion2_triton.py:147-242)."""
+    ``dion2_post_orthogonalize_triton`` (dion/dion2_triton.py:147-242).  ``row_scale [n_mat, k]``
+    (rows selected only) multiplies each selected row of ``U`` first."""
     if select_dim not in (-2, -1):
         raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
     n = len(X)
@@ -330,5 +354,11 @@ def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: 
     k = U.shape[-2] if select_dim == -2 else U.shape[-1]
     lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, U.device)
     lib = _lib.load()
+    rs = None
+    if row_scale is not None:
+        if row_scale.dtype != torch.float32 or not row_scale.is_contiguous() or \
+                row_scale.numel() != n * mats_per_ptr * k:
+            raise ValueError("row_scale must be a contiguous float32 tensor of n_mat * k entries")
+        rs = row_scale.data_ptr()
     check(lib.dion_dion2_post(xp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(), k, imap.data_ptr(),
-                              lr_p, float(adj_ratio), wd_p, wd_h, _stream_handle(U.device)), "dion2_post")
+                              rs, lr_p, float(adj_ratio), wd_p, wd_h, _stream_handle(U.device)), "dion2_post")

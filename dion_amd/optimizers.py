@@ -1,11 +1,12 @@
-"""Muon, NorMuon and Dion2 with the constructor / param-group / step() / state_dict() contract of
-microsoft/dion (dion/muon.py:20-110, dion/normuon.py:20-133, dion/dion2.py:19-127), executing on
-the hand-written gfx950 kernels.
+"""Muon, NorMuon, Dion2 and NorDion2 with the constructor / param-group / step() / state_dict()
+contract of microsoft/dion (dion/muon.py:20-110, dion/normuon.py:20-133, dion/dion2.py:19-127,
+dion/nordion2.py:26-136), executing on the hand-written gfx950 kernels.
 
 Per shape group (all parameters of one shape and dtype) a step is:
   Muon     muon_pre -> orthogonalize -> muon_post
   NorMuon  muon_pre -> orthogonalize -> normuon_stats -> muon_post(row_scale)
   Dion2    dion2_select -> orthogonalize(selected slices) -> dion2_post
+  NorDion2 dion2_select(rows) -> orthogonalize -> normuon_stats_selected -> dion2_post(row_scale)
 where the orthogonalization input/output is one dense bf16 arena ``[N, *shape]`` written and read
 directly by the fused kernels (the reference stacks and unbinds lists of tensors around it,
 dion/megabatch_base.py:870-881).
@@ -249,3 +250,88 @@ class Dion2(OrthoOptimizer):
         ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
         ops.dion2_post(X, O.view(n, mats, sel_rows, sel_cols), imap, group["lr"], ratio,
                        group["weight_decay"], select_dim)
+
+
+class NorDion2(OrthoOptimizer):
+    """NorDion2 ("Dion2 update applied to NorMuon") on one MI355X.  Same arguments as the reference
+    ``NorDion2`` (dion/nordion2.py:67-86).  Per shape group (dion/nordion2.py:233-428, unsharded
+    branch): ``M += G``; the ``ceil(fraction * rows)`` rows of largest L1 norm are selected (always
+    rows, so that a selected slice is a whole neuron); those rows of ``M`` decay by ``mu``; the
+    selected block is orthogonalized; NorMuon's per-row second-moment normalisation runs on it
+    against the selected entries of ``variance_neuron``; the scaled rows update ``X``."""
+
+    def __init__(self, params, distributed_mesh=None, lr: float = 0.01, fraction: float = 0.25,
+                 mu: float = 0.95, muon_beta2: float = 0.95, betas: Tuple[float, float] = (0.9, 0.95),
+                 weight_decay: Union[float, Tensor] = 0.01, epsilon: float = 1e-8,
+                 adjust_lr: Optional[str] = "spectral_norm", flatten: bool = False,
+                 use_triton: bool = False, use_polar_express: bool = True,
+                 use_gram_newton_schulz: bool = False, newton_schulz_func: Optional[Callable] = None,
+                 triton_post_ortho: bool = False, selection_scope: str = "local"):
+        if lr < 0.0:
+            raise ValueError(f"Invalid learning rate: {lr}")
+        if not (0.0 < fraction <= 1.0):
+            raise ValueError(f"fraction must be in (0, 1], got {fraction}")
+        if selection_scope not in ("local", "global"):
+            raise ValueError(f"selection_scope must be 'local' or 'global', got {selection_scope!r}")
+        if mu < 0.0:
+            raise ValueError(f"Invalid momentum factor (mu): {mu}")
+        if muon_beta2 < 0.0:
+            raise ValueError(f"Invalid muon_beta2: {muon_beta2}")
+        _check_common(lr, betas, adjust_lr)
+        defaults = dict(lr=lr, fraction=float(fraction), mu=mu, muon_beta2=muon_beta2, beta1=betas[0],
+                        beta2=betas[1], weight_decay=weight_decay, epsilon=epsilon, flatten=flatten,
+                        adjust_lr=adjust_lr, algorithm="nordion2", step=0, selection_scope=selection_scope)
+        super().__init__(params, distributed_mesh, "nordion2", defaults,
+                         use_gram_newton_schulz=use_gram_newton_schulz, use_triton=use_triton,
+                         use_polar_express=use_polar_express, newton_schulz_func=newton_schulz_func)
+        self._triton_post_ortho = bool(triton_post_ortho)
+
+    def _get_or_initialize_state(self, param: Tensor, algo: str) -> dict:
+        state = super()._get_or_initialize_state(param, algo)
+        if algo == self._algo_name and "variance_neuron" not in state:
+            state["variance_neuron"] = torch.zeros_like(param[..., 0:1])
+        return state
+
+    def _shape_group_phases(self, group: dict, params: List[Tensor]):
+        """Generator: [accumulate / select rows / gather] yield [orthogonalization] yield
+        [normalise selected rows / update]."""
+        num_heads = self._resolve_num_heads(group)
+        if group.get("split_sizes") is not None:
+            raise NotImplementedError("split_sizes is currently supported only by Muon and NorMuon.")
+        shape = params[0].shape
+        flatten = group["flatten"]
+        if flatten and len(shape) >= 3:
+            raise NotImplementedError("NorDion2: flatten=True is built for 2D parameters only.")
+        if num_heads is not None:
+            mats, rows, cols = self._head_geometry(num_heads, shape)
+            ratio_shape = (mats, rows, cols)
+        else:
+            rows, cols = shape[-2], shape[-1]
+            mats = params[0].numel() // (rows * cols)
+            ratio_shape = shape
+        _require_fp32(params, "NorDion2")
+        n = len(params)
+        select_dim = -2  # whole rows, so the per-neuron normalisation sees complete neurons
+        k = min(max(1, int(math.ceil(group["fraction"] * rows))), rows)
+        X = [p.data.view(mats, rows, cols) for p in params]
+        G = [p.grad.contiguous().view(mats, rows, cols) for p in params]
+        states = [self._get_or_initialize_state(p, self._algo_name) for p in params]
+        M = [s["momentum"].view(mats, rows, cols) for s in states]
+        V = [s["variance_neuron"].view(mats, rows, 1) for s in states]
+
+        # error-feedback decay of the selected rows is the momentum factor (dion/nordion2.py:352-359)
+        U_sel, idx, imap = ops.dion2_select(G, M, k, select_dim, group["mu"])
+        yield
+        _note_stream(U_sel)
+        O = self._orthogonalize(U_sel.view(n * mats, k, cols), float(group["epsilon"]))
+        del U_sel
+        yield
+        _note_stream(O)
+        O4 = O.view(n, mats, k, cols)
+        row_scale = ops.normuon_stats_selected(O4, V, idx, group["muon_beta2"])
+        ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
+        ops.dion2_post(X, O4, imap, group["lr"], ratio, group["weight_decay"], select_dim,
+                       row_scale=row_scale)
+
+
+Dion3 = NorDion2  # the reference exports the same class under both names (dion/__init__.py:9-10)

@@ -122,6 +122,15 @@ int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype, int n, in
 int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr, int rows,
                        int cols, float beta2, float* row_scale, float* scratch, void* stream);
 
+/* NorMuon statistics for an update made of k selected rows per matrix (NorDion2): U [n_mat, k,
+ * cols] bf16, row_idx [n_mat, k] int32 gives the row of the parameter each update row belongs to;
+ * V_ptrs entries each point to mats_per_ptr * v_rows fp32 (the full per-row buffers); only the
+ * selected entries of V are read and written.  row_scale out [n_mat, k].
+ * Replaces nordion2_normalize_selected_stacked (dion/nordion2.py:430-447). */
+int dion_normuon_stats_selected(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr, int k,
+                                int cols, const int32_t* row_idx, int v_rows, float beta2,
+                                float* row_scale, void* stream);
+
 /* Dion2 momentum accumulate + slice L1 norms for one shape group.
  *   M_i += G_i;  norms[i][s] = sum |M_i| over the other dim, for each slice s along select_dim
  * select_dim: -2 (rows) or -1 (columns).  norms out [n_mat, dim] fp32 (dim = rows or cols).
@@ -154,12 +163,14 @@ int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr, int rows,
 
 /* Dion2 fused weight decay + selective update, single rounding:
  *   x = (1 - lr wd) x - lr adj_ratio u[map]   on selected slices,  x = (1 - lr wd) x elsewhere
- * Replaces dion2_post_orthogonalize_triton (dion/dion2_triton.py:147-242, kernel :57-144) and
- * dion2_post_orthogonalize (dion/dion2.py:666-697). */
+ * row_scale (nullable, select_dim -2 only): device [n_mat, k] fp32; selected row j of U_sel is
+ * multiplied by row_scale[i][j] first (NorDion2's normalised update).
+ * Replaces dion2_post_orthogonalize_triton (dion/dion2_triton.py:147-242, kernel :57-144),
+ * dion2_post_orthogonalize (dion/dion2.py:666-697) and its use at dion/nordion2.py:403-425. */
 int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, int cols,
                     int select_dim, const void* U_sel, int k, const int32_t* map,
-                    const float* lr_dev, float adj_ratio, const float* wd_dev, float wd_host,
-                    void* stream);
+                    const float* row_scale, const float* lr_dev, float adj_ratio, const float* wd_dev,
+                    float wd_host, void* stream);
 
 #ifdef __cplusplus
 }

@@ -298,6 +298,30 @@ def dion2_post(X: torch.Tensor, U: torch.Tensor, idx: torch.Tensor, lr: float, a
     return out.to(torch.float32)
 
 
+def nordion2_normalize_selected(U: torch.Tensor, V_full: torch.Tensor, idx: torch.Tensor, beta2: float):
+    """dion/nordion2.py:430-447 for one matrix: gather the selected rows of the full per-neuron
+    variance buffer, run the NorMuon normalisation on them, scatter the new values back.
+    U [k, cols], V_full [rows, 1], idx [k] (long).  Returns (normalized U, new V_full)."""
+    V_sel = V_full[idx]
+    nU, V_sel_new = normuon_normalize(U, V_sel, beta2)
+    V_new = V_full.clone()
+    V_new[idx] = V_sel_new.to(V_full.dtype)
+    return nU, V_new
+
+
+def nordion2_step(x: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor, lr: float,
+                  fraction: float, mu: float, beta2: float, wd: float, adjust_lr: Optional[str],
+                  ns=None):
+    """One NorDion2 step on one 2D parameter (dion/nordion2.py:233-428, unsharded branch): rows are
+    always the selected dimension and the error-feedback decay is the momentum factor.
+    ``ns`` maps the bf16 selected block to its orthogonalization (default: fused-rounding NS5)."""
+    m2, u, idx = dion2_pre(g, m, fraction, mu, -2)
+    o = ns(u) if ns is not None else ns_bf16_fused(u, NS5_COEFFS, 1.0, 1e-8)
+    nU, v2 = nordion2_normalize_selected(o, v, idx, beta2)
+    x2 = dion2_post(x, nU, idx, lr, adjust_lr_ratio(x.shape, adjust_lr), wd, -2)
+    return x2, m2, v2, idx
+
+
 def muon_step(X: List[torch.Tensor], G: List[torch.Tensor], M: List[torch.Tensor], lr: float, mu: float,
               wd: float, nesterov: bool, adjust_lr: Optional[str], ns: str = "polar_express",
               epsilon: float = 1e-8, cautious: bool = False, adj_ratio: Optional[float] = None):

@@ -310,3 +310,78 @@ def test_gram_flag_runs_and_tracks_standard():
         ob.step()
     for a, b in zip(pa, pb):
         assert _rel(a.data, b.data) < 1e-3
+
+
+@pytest.mark.parametrize("shape", [(128, 512), (512, 128), (256, 256)])
+def test_nordion2_step_vs_oracle(shape):
+    """Two NorDion2 steps against the CPU restatement of dion/nordion2.py:233-428: momentum and the
+    selected set exact, variance_neuron and X to the accuracy the bf16 orthogonalization leaves."""
+    from dion import NorDion2
+
+    torch.manual_seed(12)
+    x = torch.randn(shape) * 0.02
+    p = torch.nn.Parameter(x.clone().to(DEV))
+    p.grad_dtype = None
+    opt = NorDion2([p], lr=0.02, fraction=0.25, mu=0.95, muon_beta2=0.95, weight_decay=0.01,
+                   use_polar_express=False)
+    M = torch.zeros(shape)
+    V = torch.zeros(shape[0], 1)
+    for step in range(2):
+        g = (torch.randn(shape) * 0.02).to(torch.bfloat16)
+        p.grad = g.to(DEV)
+        opt.step()
+        x, M, V_ref, idx = oracle.nordion2_step(x, g, M, V, 0.02, 0.25, 0.95, 0.95, 0.01, "spectral_norm")
+        assert _rel(opt.state[p]["momentum"], M) <= 1e-6
+        v_gpu = opt.state[p]["variance_neuron"].cpu()
+        mask = torch.ones(shape[0], dtype=torch.bool)
+        mask[idx] = False
+        assert torch.equal(v_gpu[mask], V[mask])  # unselected neurons keep their second moment
+        assert _rel(v_gpu, V_ref) <= 3e-2
+        assert _rel(p.data, x) <= 1e-3
+        x = p.data.cpu().clone()
+        V = v_gpu.clone()
+
+
+def test_nordion2_fraction_one_is_normuon_without_momentum_decay():
+    """fraction = 1: every row selected, so the update is NorMuon's normalised orthogonalization of
+    M + G and the whole momentum decays by mu."""
+    from dion import NorDion2
+    from dion_amd import ops, zeropower_via_newtonschulz5
+
+    torch.manual_seed(13)
+    shape = (64, 256)
+    p = torch.nn.Parameter(torch.randn(shape, device=DEV) * 0.02)
+    x0 = p.data.clone()
+    g = torch.randn(shape, device=DEV) * 0.02
+    p.grad = g.clone()
+    opt = NorDion2([p], lr=0.02, fraction=1.0, mu=0.9, muon_beta2=0.95, weight_decay=0.0,
+                   use_polar_express=False, adjust_lr=None)
+    opt.step()
+    assert torch.equal(opt.state[p]["momentum"], g * 0.9)
+    O = zeropower_via_newtonschulz5(g.to(torch.bfloat16), 1e-8).unsqueeze(0)
+    V = [torch.zeros(shape[0], 1, device=DEV)]
+    scale = ops.normuon_stats(O, V, 0.95)
+    ref = x0 - 0.02 * (O[0].float() * scale.view(-1, 1))
+    assert _rel(p.data, ref) <= 1e-6
+    assert _rel(opt.state[p]["variance_neuron"], V[0]) <= 1e-6
+
+
+def test_nordion2_num_heads_matches_3d_param_and_alias():
+    from dion import Dion3, NorDion2
+
+    assert Dion3 is NorDion2
+    torch.manual_seed(14)
+    H, d, n_in = 4, 32, 96
+    init = torch.randn(H * d, n_in, device=DEV) * 0.02
+    grads = [torch.randn(H * d, n_in, device=DEV) * 0.02 for _ in range(2)]
+    p2 = torch.nn.Parameter(init.clone())
+    p3 = torch.nn.Parameter(init.clone().view(H, d, n_in))
+    o2 = NorDion2([dict(params=[p2], num_heads=H)], lr=0.02, fraction=0.5)
+    o3 = NorDion2([p3], lr=0.02, fraction=0.5)
+    for g in grads:
+        p2.grad = g.clone()
+        p3.grad = g.clone().view(H, d, n_in)
+        o2.step()
+        o3.step()
+    assert torch.equal(p2.data.view(H, d, n_in), p3.data)
+    assert torch.equal(o2.state[p2]["variance_neuron"].view(-1), o3.state[p3]["variance_neuron"].view(-1))

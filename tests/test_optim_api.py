@@ -4,7 +4,7 @@ of tests/test_optimizers.py."""
 import pytest
 import torch
 
-from dion import Dion2, Muon, NorMuon
+from dion import Dion2, Dion3, Muon, NorDion2, NorMuon
 
 
 def _params(shapes):
@@ -14,12 +14,13 @@ def _params(shapes):
 
 def test_state_exists_at_construction():
     p = _params([(16, 32), (32, 16)])
-    for cls, keys in [(Muon, {"momentum"}), (Dion2, {"momentum"}), (NorMuon, {"momentum", "variance_neuron"})]:
+    for cls, keys in [(Muon, {"momentum"}), (Dion2, {"momentum"}), (NorMuon, {"momentum", "variance_neuron"}),
+                      (NorDion2, {"momentum", "variance_neuron"})]:
         opt = cls(p, lr=0.01)
         for q in p:
             assert set(opt.state[q].keys()) == keys
             assert torch.equal(opt.state[q]["momentum"], torch.zeros_like(q))
-        if cls is NorMuon:
+        if cls in (NorMuon, NorDion2):
             assert opt.state[p[0]]["variance_neuron"].shape == (16, 1)
 
 
@@ -34,6 +35,23 @@ def test_param_group_keys_and_defaults():
     g = Dion2(p, fraction=1).param_groups[0]
     assert g["algorithm"] == "dion2" and g["fraction"] == 1.0 and isinstance(g["fraction"], float)
     assert g["ef_decay"] == 0.95 and g["selection_scope"] == "local"
+    # dion/nordion2.py:108-122
+    g = NorDion2(p, fraction=1).param_groups[0]
+    assert g["algorithm"] == "nordion2" and g["fraction"] == 1.0 and isinstance(g["fraction"], float)
+    assert g["mu"] == 0.95 and g["muon_beta2"] == 0.95 and g["selection_scope"] == "local" and "ef_decay" not in g
+    assert Dion3 is NorDion2
+
+
+def test_nordion2_constructor_validation():
+    p = _params([(16, 32)])
+    for kw in [dict(lr=-1.0), dict(fraction=0.0), dict(fraction=1.5), dict(selection_scope="everywhere"),
+               dict(mu=-0.1), dict(muon_beta2=-0.1), dict(betas=(0.9,)), dict(adjust_lr="bogus")]:
+        with pytest.raises(ValueError):
+            NorDion2(p, **kw)
+    with pytest.raises(NotImplementedError):
+        opt = NorDion2([dict(params=p, split_sizes=(8, 8))])
+        p[0].grad = torch.zeros_like(p[0])
+        opt.step()
 
 
 def test_lr_is_a_persistent_tensor_and_state_dict_is_portable():

@@ -207,3 +207,47 @@ def test_dion2_post_unselected_is_exactly_a_times_x():
     out = o.dion2_post(X, Uc, torch.tensor([0, 13]), 0.02, 1.5, 0.1, -1)
     assert torch.allclose(out[:, [0, 13]], a * X[:, [0, 13]] - b * Uc.float(), rtol=1e-6)
     assert torch.allclose(out[:, 1:13], a * X[:, 1:13])
+
+
+def test_nordion2_selected_normalisation_reduces_to_normuon():
+    """With every row selected, in order, the selected-row normalisation IS NorMuon's; with a subset,
+    unselected entries of V are untouched and the update keeps the Frobenius norm of its input."""
+    torch.manual_seed(9)
+    U = torch.randn(6, 10).to(torch.bfloat16)
+    V = torch.rand(6, 1) * 1e-2
+    nU_all, V_all = o.nordion2_normalize_selected(U, V, torch.arange(6), 0.9)
+    nU_ref, V_ref = o.normuon_normalize(U, V, 0.9)
+    assert torch.equal(nU_all, nU_ref) and torch.equal(V_all, V_ref)
+    idx = torch.tensor([1, 4, 5])
+    nU, V2 = o.nordion2_normalize_selected(U[idx], V, idx, 0.9)
+    keep = torch.tensor([0, 2, 3])
+    assert torch.equal(V2[keep], V[keep])
+    assert not torch.equal(V2[idx], V[idx])
+    assert abs(float(nU.norm() / U[idx].float().norm()) - 1.0) < 1e-5
+
+
+def test_nordion2_step_closed_cases():
+    """fraction = 1 selects every row: M_after = mu * (M + G) everywhere, and the update equals a
+    NorMuon-normalised orthogonalization of M + G.  First step from zero state: V = (1 - beta2) *
+    mean(O^2) on selected rows and 0 elsewhere."""
+    torch.manual_seed(10)
+    x = torch.randn(8, 16) * 0.02
+    g = (torch.randn(8, 16) * 0.02).to(torch.bfloat16)
+    m = torch.randn(8, 16) * 0.02
+    v = torch.zeros(8, 1)
+    ident = lambda u: u  # keeps the case checkable by hand
+    x2, m2, v2, idx = o.nordion2_step(x, g, m, v, 0.02, 1.0, 0.95, 0.9, 0.01, None, ns=ident)
+    acc = m + g.float()
+    assert torch.equal(idx, torch.arange(8))
+    assert torch.allclose(m2, acc * 0.95, rtol=0, atol=0)
+    u = acc.to(torch.bfloat16)
+    nU, v_ref = o.normuon_normalize(u, v, 0.9)
+    assert torch.equal(v2, v_ref)
+    assert torch.allclose(x2, x * (1 - 0.02 * 0.01) - 0.02 * nU, rtol=1e-6, atol=1e-9)
+    # a quarter of the rows: V stays zero off the selection
+    x3, m3, v3, idx3 = o.nordion2_step(x, g, m, v, 0.02, 0.25, 0.95, 0.9, 0.01, None, ns=ident)
+    assert idx3.numel() == 2
+    mask = torch.ones(8, dtype=torch.bool)
+    mask[idx3] = False
+    assert float(v3[mask].abs().max()) == 0.0 and float(v3[idx3].min()) > 0.0
+    assert torch.equal(m3[mask], acc[mask]) and torch.equal(x3[mask], (x * torch.tensor(1 - 0.02 * 0.01))[mask])
