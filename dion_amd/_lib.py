@@ -17,6 +17,7 @@ DION_NS_GRAM = 1
 DION_NS_CARRY_XT = 2
 
 _u64p = ctypes.POINTER(ctypes.c_uint64)
+_i64p = ctypes.POINTER(ctypes.c_int64)
 _f32p = ctypes.POINTER(c_float)
 
 # name -> (restype, argtypes); mirrors include/dion_hip.h one to one.
@@ -45,6 +46,10 @@ SIGNATURES = {
                                   c_void_p, c_void_p]),
     "dion_dion2_post": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
                                 c_void_p, c_void_p, c_float, c_void_p, c_float, c_void_p]),
+    "dion_adamw_step": (c_int, [_u64p, _u64p, c_int, _u64p, _u64p, _u64p, _i64p, c_int, c_void_p, c_float,
+                                c_float, c_float, c_void_p, c_float, c_int, c_void_p]),
+    "dion_lion_step": (c_int, [_u64p, _u64p, c_int, _u64p, _i64p, c_int, c_void_p, c_float, c_float,
+                               c_void_p, c_float, c_int, c_void_p]),
 }
 
 _lib = None

@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 3; }
+extern "C" int dion_abi_version(void) { return 4; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -623,6 +623,65 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
                               row_scale ? row_scale + mat0 * k : nullptr, lr_dev, adj_ratio, wd_dev,
                               wd_host, vec4, (hipStream_t)stream),
             "dion_dion2_post");
+  }
+  return DION_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Multi-tensor AdamW / Lion for the non-matrix parameter groups
+// ---------------------------------------------------------------------------------------------
+static int check_mta(const char* who, const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M,
+                     const int64_t* numels, int n, const float* lr_dev) {
+  if (n < 0) return fail(DION_E_INVALID, "%s: negative count", who);
+  if (g_dtype != DION_BF16 && g_dtype != DION_F32) return fail(DION_E_INVALID, "%s: g_dtype", who);
+  if (n == 0) return DION_OK;
+  if (!X || !G || !M || !numels || !lr_dev) return fail(DION_E_INVALID, "%s: null argument", who);
+  for (int i = 0; i < n; ++i)
+    if (numels[i] < 0 || (numels[i] > 0 && (!X[i] || !G[i] || !M[i])))
+      return fail(DION_E_INVALID, "%s: tensor %d has a null pointer or a negative size", who, i);
+  return DION_OK;
+}
+
+extern "C" int dion_adamw_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype,
+                               const uint64_t* M_ptrs, const uint64_t* V_ptrs,
+                               const uint64_t* step_ptrs, const int64_t* numels, int n,
+                               const float* lr_dev, float beta1, float beta2, float eps,
+                               const float* wd_dev, float wd_host, int cautious, void* stream) {
+  if (int rc = check_mta("dion_adamw_step", X_ptrs, G_ptrs, g_dtype, M_ptrs, numels, n, lr_dev)) return rc;
+  if (n == 0) return DION_OK;
+  if (!V_ptrs || !step_ptrs) return fail(DION_E_INVALID, "dion_adamw_step: null argument");
+  for (int i = 0; i < n; ++i)
+    if (!step_ptrs[i] || (numels[i] > 0 && !V_ptrs[i]))
+      return fail(DION_E_INVALID, "dion_adamw_step: tensor %d has a null state pointer", i);
+  // One step counter may serve several tensors; a counter shared ACROSS launch chunks would be
+  // advanced once per chunk, so every chunk must own its counters.
+  for (int i0 = 0; i0 < n; i0 += kMtaTensors) {
+    const int c = (n - i0) < kMtaTensors ? (n - i0) : kMtaTensors;
+    for (int i = i0; i < i0 + c; ++i)
+      for (int j = 0; j < i0; ++j)
+        if (step_ptrs[i] == step_ptrs[j])
+          return fail(DION_E_INVALID,
+                      "dion_adamw_step: step counter of tensor %d is shared with tensor %d of an earlier "
+                      "chunk of %d tensors",
+                      i, j, kMtaTensors);
+    HIP_TRY(launch_adamw_mt(X_ptrs + i0, G_ptrs + i0, g_dtype, M_ptrs + i0, V_ptrs + i0, step_ptrs + i0,
+                            numels + i0, c, lr_dev, beta1, beta2, eps, wd_dev, wd_host, cautious,
+                            (hipStream_t)stream),
+            "dion_adamw_step");
+  }
+  return DION_OK;
+}
+
+extern "C" int dion_lion_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype,
+                              const uint64_t* M_ptrs, const int64_t* numels, int n, const float* lr_dev,
+                              float beta1, float beta2, const float* wd_dev, float wd_host, int cautious,
+                              void* stream) {
+  if (int rc = check_mta("dion_lion_step", X_ptrs, G_ptrs, g_dtype, M_ptrs, numels, n, lr_dev)) return rc;
+  for (int i0 = 0; i0 < n; i0 += kMtaTensors) {
+    const int c = (n - i0) < kMtaTensors ? (n - i0) : kMtaTensors;
+    HIP_TRY(launch_lion_mt(X_ptrs + i0, G_ptrs + i0, g_dtype, M_ptrs + i0, numels + i0, c, lr_dev, beta1,
+                           beta2, wd_dev, wd_host, cautious, (hipStream_t)stream),
+            "dion_lion_step");
   }
   return DION_OK;
 }

@@ -57,4 +57,16 @@ hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int r
                              const float* row_scale, const float* lr_dev, float adj_ratio,
                              const float* wd_dev, float wd_host, bool vec4, hipStream_t st);
 
+
+// Multi-tensor AdamW / Lion (scalar_opts.hip): n <= kMtaTensors tensors per launch, host arrays of
+// device pointers and element counts.
+constexpr int kMtaTensors = 48;
+hipError_t launch_adamw_mt(const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M,
+                           const uint64_t* V, const uint64_t* steps, const int64_t* numel, int n,
+                           const float* lr_dev, float beta1, float beta2, float eps, const float* wd_dev,
+                           float wd_host, int cautious, hipStream_t st);
+hipError_t launch_lion_mt(const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M,
+                          const int64_t* numel, int n, const float* lr_dev, float beta1, float beta2,
+                          const float* wd_dev, float wd_host, int cautious, hipStream_t st);
+
 }  // namespace dion

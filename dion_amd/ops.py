@@ -362,3 +362,55 @@ def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: 
         rs = row_scale.data_ptr()
     check(lib.dion_dion2_post(xp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(), k, imap.data_ptr(),
                               rs, lr_p, float(adj_ratio), wd_p, wd_h, _stream_handle(U.device)), "dion2_post")
+
+
+# ---------------------------------------------------------------------------------------------
+# multi-tensor AdamW / Lion for the non-matrix parameter groups
+# ---------------------------------------------------------------------------------------------
+def _mta_tables(X: List[Tensor], G: List[Tensor], states: List[List[Tensor]]):
+    n = len(X)
+    assert n > 0 and len(G) == n and all(len(s) == n for s in states)
+    gdt = G[0].dtype
+    for x, g in zip(X, G):
+        _require_gpu(x, "X")
+        _require_gpu(g, "G")
+        if x.dtype != torch.float32:
+            raise NotImplementedError(f"X: the gfx950 step kernels keep parameters in float32, got {x.dtype}")
+        if g.dtype != gdt:
+            raise TypeError("G: one gradient dtype per call")
+        if not x.is_contiguous() or not g.is_contiguous() or g.numel() != x.numel():
+            raise ValueError("X / G must be contiguous and of equal size")
+    for name, st in zip("MV", states):
+        for x, s in zip(X, st):
+            if s.dtype != torch.float32 or not s.is_contiguous() or s.numel() != x.numel() or not s.is_cuda:
+                raise ValueError(f"{name}: optimizer state must be contiguous float32 GPU tensors shaped like X")
+    numels = (_lib.ctypes.c_int64 * n)(*[x.numel() for x in X])
+    tabs = [ptr_table([t.data_ptr() for t in ts]) for ts in (X, G, *states)]
+    return tabs, numels, _dtype_code(G[0], "G")
+
+
+def adamw_step(X: List[Tensor], G: List[Tensor], M: List[Tensor], V: List[Tensor], steps: List[Tensor],
+               lr: Tensor, beta1: float, beta2: float, weight_decay, epsilon: float,
+               cautious_wd: bool = False) -> None:
+    """One fused AdamW step over tensors of any sizes (dion/scalar_opts.py:7-65, :121-268).  ``steps``
+    are 0-d float32 device counters (one per tensor; tensors may share one), advanced on the device."""
+    (xp, gp, mp, vp), numels, gcode = _mta_tables(X, G, [M, V])
+    for s in steps:
+        if not (s.is_cuda and s.dtype == torch.float32 and s.numel() == 1):
+            raise TypeError("steps must be 0-d float32 GPU tensors")
+    sp = ptr_table([s.data_ptr() for s in steps])
+    lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, X[0].device)
+    lib = _lib.load()
+    check(lib.dion_adamw_step(xp, gp, gcode, mp, vp, sp, numels, len(X), lr_p, float(beta1), float(beta2),
+                              float(epsilon), wd_p, wd_h, int(bool(cautious_wd)), _stream_handle(X[0].device)),
+          "adamw_step")
+
+
+def lion_step(X: List[Tensor], G: List[Tensor], M: List[Tensor], lr: Tensor, beta1: float, beta2: float,
+              weight_decay, cautious_wd: bool = False) -> None:
+    """One fused Lion step over tensors of any sizes (dion/scalar_opts.py:68-118, :271-325)."""
+    (xp, gp, mp), numels, gcode = _mta_tables(X, G, [M])
+    lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, X[0].device)
+    lib = _lib.load()
+    check(lib.dion_lion_step(xp, gp, gcode, mp, numels, len(X), lr_p, float(beta1), float(beta2), wd_p, wd_h,
+                             int(bool(cautious_wd)), _stream_handle(X[0].device)), "lion_step")

@@ -172,6 +172,32 @@ int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, i
                     const float* row_scale, const float* lr_dev, float adj_ratio, const float* wd_dev,
                     float wd_host, void* stream);
 
+/* --------------------------------------------------------------------------------------------
+ * Multi-tensor AdamW / Lion for the non-matrix parameter groups (algorithm "adamw" / "lion").
+ * X_ptrs, G_ptrs, M_ptrs, V_ptrs: host ptr tables of n device pointers; tensor i has numels[i]
+ * elements (host array); X, M, V fp32, G bf16 or fp32 per g_dtype (one dtype per call).
+ * lr_dev / wd_dev as in dion_muon_post.  Any number of tensors per call, any sizes.
+ * ------------------------------------------------------------------------------------------ */
+
+/* AdamW with bias correction and decoupled (optionally cautious) weight decay:
+ *   step_i += 1 (device float counters, step_ptrs; a counter may be shared by tensors of one call
+ *   if they lie within the same run of 48 consecutive tensors)
+ *   M = lerp(M, G, 1-beta1); V = beta2 V + (1-beta2) G^2; d = sqrt(V)/sqrt(1-beta2^step) + eps
+ *   X = X (1 - lr wd)   [cautious: X -= X [M/d * X >= 0] lr wd];   X -= lr/(1-beta1^step) M/d
+ * Replaces adamw_update / adamw_update_foreach (dion/scalar_opts.py:7-65, :121-268; capturable
+ * form: counters advance on the device, lr is read on the device). */
+int dion_adamw_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs,
+                    const uint64_t* V_ptrs, const uint64_t* step_ptrs, const int64_t* numels, int n,
+                    const float* lr_dev, float beta1, float beta2, float eps, const float* wd_dev,
+                    float wd_host, int cautious, void* stream);
+
+/* Lion:  U = sign(lerp(M, G, 1-beta1)); M = lerp(M, G, 1-beta2);
+ *   X = X (1 - lr wd)   [cautious: X -= X [U X >= 0] lr wd];   X -= lr U
+ * Replaces lion_update / lion_update_foreach (dion/scalar_opts.py:68-118, :271-325). */
+int dion_lion_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs,
+                   const int64_t* numels, int n, const float* lr_dev, float beta1, float beta2,
+                   const float* wd_dev, float wd_host, int cautious, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

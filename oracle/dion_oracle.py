@@ -322,6 +322,40 @@ def nordion2_step(x: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Te
     return x2, m2, v2, idx
 
 
+def adamw_update(X: torch.Tensor, G: torch.Tensor, M: torch.Tensor, V: torch.Tensor, lr: float, beta1: float,
+                 beta2: float, wd: float, step: int, eps: float, cautious: bool = False):
+    """dion/scalar_opts.py:7-65 in float64.  Returns (X_new, M_new, V_new)."""
+    X, G, M, V = (t.to(torch.float64) for t in (X, G, M, V))
+    M = M + (1 - beta1) * (G - M)
+    V = V * beta2 + (1 - beta2) * G * G
+    bc1 = 1 - beta1 ** step
+    bc2 = 1 - beta2 ** step
+    denom = V.sqrt() / math.sqrt(bc2) + eps
+    upd = M / denom
+    if cautious:
+        mask = (upd * X >= 0).to(X.dtype)
+        X = X - (X * mask) * (lr * wd)
+    else:
+        X = X * (1 - lr * wd)
+    X = X - (lr / bc1) * upd
+    return X, M, V
+
+
+def lion_update(X: torch.Tensor, G: torch.Tensor, M: torch.Tensor, lr: float, beta1: float, beta2: float,
+                wd: float, cautious: bool = False):
+    """dion/scalar_opts.py:68-118 in float64.  Returns (X_new, M_new)."""
+    X, G, M = (t.to(torch.float64) for t in (X, G, M))
+    U = torch.sign(M + (1 - beta1) * (G - M))
+    M = M + (1 - beta2) * (G - M)
+    if cautious:
+        mask = (U * X >= 0).to(X.dtype)
+        X = X - (X * mask) * (lr * wd)
+    else:
+        X = X * (1 - lr * wd)
+    X = X - lr * U
+    return X, M
+
+
 def muon_step(X: List[torch.Tensor], G: List[torch.Tensor], M: List[torch.Tensor], lr: float, mu: float,
               wd: float, nesterov: bool, adjust_lr: Optional[str], ns: str = "polar_express",
               epsilon: float = 1e-8, cautious: bool = False, adj_ratio: Optional[float] = None):

@@ -178,3 +178,116 @@ def test_select_dim_validation():
     with pytest.raises(ValueError, match="select_dim"):
         ops.dion2_post(t, torch.zeros(1, 1, 2, 8, device=DEV, dtype=torch.bfloat16),
                        torch.zeros(1, 8, dtype=torch.int32, device=DEV), torch.tensor(0.1, device=DEV), 1.0, 0.0, 1)
+
+
+@pytest.mark.parametrize("cautious", [False, True])
+@pytest.mark.parametrize("gdtype", [torch.bfloat16, torch.float32])
+def test_adamw_multi_tensor_vs_oracle(cautious, gdtype):
+    """Ragged list (empty, scalar-sized, odd, unaligned view, > 48 tensors, one large) over three
+    steps against the float64 restatement of dion/scalar_opts.py:7-65."""
+    from dion_amd import ops
+
+    torch.manual_seed(31)
+    sizes = [0, 1, 3, 7, 64, 129, 1000, 4096 * 33 + 5] + [17 + i for i in range(50)]
+    base = [torch.randn(n + 1) for n in sizes]
+    X = [b[1:].clone() if i % 3 else b[:-1].clone() for i, b in enumerate(base)]
+    Xd = [x.to(DEV) for x in X]
+    # every third tensor is an offset view: 4-byte aligned only
+    for i in range(0, len(Xd), 3):
+        buf = torch.zeros(sizes[i] + 1, device=DEV)
+        buf[1:].copy_(Xd[i])
+        Xd[i] = buf[1:]
+    M = [torch.zeros_like(x) for x in X]
+    V = [torch.zeros_like(x) for x in X]
+    Md = [torch.zeros_like(x) for x in Xd]
+    Vd = [torch.zeros_like(x) for x in Xd]
+    steps = [torch.zeros((), device=DEV) for _ in Xd]
+    lr = torch.tensor(0.01, device=DEV)
+    for step in range(1, 4):
+        G = [torch.randn(n).to(gdtype) for n in sizes]
+        ops.adamw_step(Xd, [g.to(DEV) for g in G], Md, Vd, steps, lr, 0.9, 0.95, 0.1, 1e-8, cautious)
+        for i in range(len(X)):
+            X[i], M[i], V[i] = oracle.adamw_update(X[i], G[i].float(), M[i], V[i], 0.01, 0.9, 0.95, 0.1, step,
+                                                   1e-8, cautious)
+            if sizes[i] == 0:
+                continue
+            assert _rel(Md[i], M[i]) <= 1e-6 and _rel(Vd[i], V[i]) <= 1e-6
+            # bf16 gradients cancel the momentum exactly now and then (g2 == -0.9 g1): its sign, and
+            # with it the cautious mask, is then decided by rounding -- leave those entries out
+            clear = M[i].abs() > 1e-6 * G[i].double().abs()
+            assert float(((Xd[i].double().cpu() - X[i]).abs() * clear).max()) <= 2e-6
+            assert int((~clear).sum()) <= 1 + sizes[i] // 1000
+            # keep fp32 rounding from accumulating into a sign flip of the cautious mask
+            X[i], M[i], V[i] = Xd[i].double().cpu(), Md[i].double().cpu(), Vd[i].double().cpu()
+        assert all(float(s) == float(step) for s in steps)
+
+
+def test_adamw_known_answer_and_shared_step_counter():
+    """The reference's hand-computed cautious case (tests/test_adamw_foreach.py:80-112) and a step
+    counter shared by the tensors of one call (advanced once per call)."""
+    from dion_amd import ops
+
+    X = [torch.tensor([1.0, 1.0, -1.0, -1.0], device=DEV), torch.tensor([1.0, 1.0, -1.0, -1.0], device=DEV)]
+    G = [torch.tensor([2.0, -2.0, 2.0, -2.0], device=DEV) for _ in range(2)]
+    M = [torch.zeros(4, device=DEV) for _ in range(2)]
+    V = [torch.zeros(4, device=DEV) for _ in range(2)]
+    step = torch.zeros((), device=DEV)
+    ops.adamw_step(X, G, M, V, [step, step], torch.tensor(0.1, device=DEV), 0.9, 0.999, 0.5, 1e-8, True)
+    assert float(step) == 1.0
+    g = torch.tensor([2.0, -2.0, 2.0, -2.0])
+    x0 = torch.tensor([1.0, 1.0, -1.0, -1.0])
+    m_new, v_new = 0.1 * g, 0.001 * g * g
+    update = (0.1 / 0.1) * m_new / (v_new.sqrt() / (1 - 0.999) ** 0.5 + 1e-8)
+    expected = x0 - 0.1 * 0.5 * x0 * torch.tensor([1.0, 0.0, 0.0, 1.0]) - update
+    for x in X:
+        assert torch.allclose(x.cpu(), expected, atol=1e-6, rtol=0)
+
+
+@pytest.mark.parametrize("cautious", [False, True])
+@pytest.mark.parametrize("gdtype", [torch.bfloat16, torch.float32])
+def test_lion_multi_tensor_vs_oracle(cautious, gdtype):
+    from dion_amd import ops
+
+    torch.manual_seed(32)
+    sizes = [0, 1, 5, 64, 1001, 4096 * 17 + 3] + [9 + i for i in range(50)]
+    X = [torch.randn(n) for n in sizes]
+    M = [torch.randn(n) * 0.1 for n in sizes]
+    Xd, Md = [x.to(DEV) for x in X], [m.to(DEV) for m in M]
+    lr = torch.tensor(0.01, device=DEV)
+    for _ in range(2):
+        G = [torch.randn(n).to(gdtype) for n in sizes]
+        ops.lion_step(Xd, [g.to(DEV) for g in G], Md, lr, 0.9, 0.99, 0.1, cautious)
+        for i in range(len(X)):
+            x_ref, m_ref = oracle.lion_update(X[i], G[i].float(), M[i], 0.01, 0.9, 0.99, 0.1, cautious)
+            if sizes[i]:
+                assert _rel(Md[i], m_ref) <= 1e-6
+                # a blend within rounding of zero may take the other sign: allow a handful of 2*lr moves
+                d = (Xd[i].double().cpu() - x_ref).abs()
+                assert int((d > 2e-6).sum()) <= max(1, sizes[i] // 100000)
+            X[i], M[i] = Xd[i].cpu(), Md[i].cpu()
+
+
+def test_scalar_groups_inside_an_optimizer():
+    """Mixed param groups through Muon.step(): AdamW and Lion groups follow the restatement while
+    the matrix group is orthogonalized; step_dev advances on the device."""
+    from dion import Muon
+
+    torch.manual_seed(33)
+    w = torch.nn.Parameter(torch.randn(64, 128, device=DEV) * 0.02)
+    b = torch.nn.Parameter(torch.randn(300, device=DEV))
+    e = torch.nn.Parameter(torch.randn(50, 16, device=DEV))
+    opt = Muon([{"params": [w]}, {"params": [b], "algorithm": "adamw", "lr": 0.003},
+                {"params": [e], "algorithm": "lion", "lr": 0.001, "cautious_wd": True}], lr=0.02)
+    xb, mb, vb = b.data.cpu().clone(), torch.zeros(300), torch.zeros(300)
+    xe, me = e.data.cpu().clone(), torch.zeros(50, 16)
+    for step in range(1, 4):
+        for p in (w, b, e):
+            p.grad = torch.randn_like(p)
+        opt.step()
+        xb, mb, vb = oracle.adamw_update(xb, b.grad.cpu(), mb, vb, 0.003, 0.9, 0.95, 0.01, step, 1e-8)
+        xe, me = oracle.lion_update(xe, e.grad.cpu(), me, 0.001, 0.9, 0.95, 0.01, True)
+        assert float((b.data.double().cpu() - xb).abs().max()) <= 2e-6
+        assert float((e.data.double().cpu() - xe).abs().max()) <= 2e-6
+        xb, mb, vb = b.data.double().cpu(), opt.state[b]["momentum"].double().cpu(), opt.state[b]["variance"].double().cpu()
+        xe, me = e.data.double().cpu(), opt.state[e]["momentum"].double().cpu()
+    assert float(opt.state[b]["step_dev"]) == 3.0

@@ -251,3 +251,50 @@ def test_nordion2_step_closed_cases():
     mask[idx3] = False
     assert float(v3[mask].abs().max()) == 0.0 and float(v3[idx3].min()) > 0.0
     assert torch.equal(m3[mask], acc[mask]) and torch.equal(x3[mask], (x * torch.tensor(1 - 0.02 * 0.01))[mask])
+
+
+def test_adamw_restatement_known_answers():
+    """The reference's hand-computed cautious-weight-decay vector (tests/test_adamw_foreach.py:80-112):
+    mask [1, 0, 0, 1], two positions decayed, two not.  Plus torch.optim.AdamW as an independent
+    implementation of the non-cautious rule over several steps."""
+    X = torch.tensor([1.0, 1.0, -1.0, -1.0])
+    G = torch.tensor([2.0, -2.0, 2.0, -2.0])
+    lr, b1, b2, wd, eps = 0.1, 0.9, 0.999, 0.5, 1e-8
+    x2, m2, v2 = o.adamw_update(X, G, torch.zeros(4), torch.zeros(4), lr, b1, b2, wd, 1, eps, cautious=True)
+    m_new = (1 - b1) * G.double()
+    v_new = (1 - b2) * G.double() ** 2
+    update = (lr / (1 - b1)) * m_new / (v_new.sqrt() / math.sqrt(1 - b2) + eps)
+    expected = X.double() - lr * wd * X.double() * torch.tensor([1.0, 0.0, 0.0, 1.0]).double() - update
+    assert torch.allclose(x2, expected, atol=1e-12, rtol=0)
+    assert torch.allclose(m2, m_new) and torch.allclose(v2, v_new)
+
+    torch.manual_seed(21)
+    p = torch.nn.Parameter(torch.randn(50, dtype=torch.float64))
+    x, m, v = p.data.clone(), torch.zeros(50, dtype=torch.float64), torch.zeros(50, dtype=torch.float64)
+    ref = torch.optim.AdamW([p], lr=0.01, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    for step in range(1, 5):
+        g = torch.randn(50, dtype=torch.float64)
+        p.grad = g.clone()
+        ref.step()
+        x, m, v = o.adamw_update(x, g, m, v, 0.01, 0.9, 0.95, 0.1, step, 1e-8)
+        assert torch.allclose(x, p.data, rtol=1e-10, atol=1e-12)
+
+
+def test_lion_restatement_closed_cases():
+    """First step from zero momentum: U = sign(G), so X moves by exactly lr against the gradient sign
+    after the decay; M = (1-beta2) G.  Cautious decay touches only entries where sign(U) == sign(X)."""
+    X = torch.tensor([1.0, 1.0, -1.0, -1.0, 0.5])
+    G = torch.tensor([2.0, -2.0, 2.0, -2.0, 0.0])
+    x2, m2 = o.lion_update(X, G, torch.zeros(5), 0.1, 0.9, 0.99, 0.5)
+    assert torch.allclose(x2, X.double() * 0.95 - 0.1 * torch.sign(G).double(), atol=1e-15)
+    assert torch.allclose(m2, 0.01 * G.double(), atol=1e-15)
+    x3, _ = o.lion_update(X, G, torch.zeros(5), 0.1, 0.9, 0.99, 0.5, cautious=True)
+    mask = torch.tensor([1.0, 0.0, 0.0, 1.0, 1.0]).double()  # U*X >= 0 (U = 0 counts)
+    assert torch.allclose(x3, X.double() - 0.05 * X.double() * mask - 0.1 * torch.sign(G).double(), atol=1e-15)
+    # second step blends momentum and gradient with beta1 before the sign
+    M = torch.tensor([1.0, -1.0, 1.0, -1.0, 0.0])
+    G2 = torch.tensor([-5.0, 5.0, -20.0, 20.0, 1.0])
+    x4, m4 = o.lion_update(X, G2, M, 0.1, 0.9, 0.99, 0.0)
+    blend = 0.9 * M.double() + 0.1 * G2.double()  # [0.4, -0.4, -1.1, 1.1, 0.1]
+    assert torch.allclose(x4, X.double() - 0.1 * torch.sign(blend), atol=1e-15)
+    assert torch.allclose(m4, 0.99 * M.double() + 0.01 * G2.double(), atol=1e-15)
