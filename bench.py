@@ -101,6 +101,8 @@ def main() -> int:
     ap.add_argument("--workload", default="llama3_8b", choices=sorted(WORKLOADS))
     ap.add_argument("--ns", default="ns5", choices=["ns5", "polar_express", "gram"])
     ap.add_argument("--optimizer", default="muon", choices=["muon", "normuon", "dion2", "nordion2"])
+    ap.add_argument("--graph", action="store_true",
+                    help="capture the step into a hipGraph during warm-up and time replays (needs --warmup >= 2)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     args = ap.parse_args()
@@ -162,6 +164,13 @@ def main() -> int:
         opt = Dion2(groups, lr=0.02, fraction=fraction, ef_decay=0.95, weight_decay=0.01,
                     adjust_lr="spectral_norm", **ns_kw)
 
+    if args.graph:
+        if args.warmup < 2:
+            print("bench.py: --graph needs --warmup >= 2 (one eager step, one capture step)", file=sys.stderr)
+            return 2
+        from dion.cuda_graph import CudaGraphOptimizer
+
+        opt = CudaGraphOptimizer(opt, warmup_steps=args.warmup - 1)
     for _ in range(args.warmup):
         opt.step()
     torch.cuda.synchronize()
@@ -186,7 +195,8 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"{args.workload}: full {type(opt).__name__}.step() ({args.ns}, wd 0.01, lr 0.02"
+            "workload": f"{args.workload}: full {type(getattr(opt, 'optimizer', opt)).__name__}.step() ("
+                        + ("hipGraph replay, " if args.graph else "") + f"{args.ns}, wd 0.01, lr 0.02"
                         + ({"dion2": ", fraction 0.25, ef_decay 0.95", "nordion2": ", fraction 0.25, mu 0.95"}
                            .get(args.optimizer, ", nesterov mu=0.95"))
                         + (", muon_beta2 0.95" if args.optimizer in ("normuon", "nordion2") else "") + ") over "

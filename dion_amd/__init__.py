@@ -11,6 +11,7 @@ from .newton_schulz import (  # noqa: F401
     zeropower_via_newtonschulz5,
 )
 
+from .hip_graph import CudaGraphOptimizer, HipGraphOptimizer  # noqa: E402,F401
 from .optimizers import Dion2, Dion3, Muon, NorDion2, NorMuon  # noqa: E402,F401
 
 __all__ = [
@@ -19,6 +20,8 @@ __all__ = [
     "Dion2",
     "NorDion2",
     "Dion3",
+    "HipGraphOptimizer",
+    "CudaGraphOptimizer",
     "gram_newton_schulz",
     "newton_schulz_triton",
     "ns_line_1",

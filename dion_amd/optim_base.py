@@ -139,6 +139,18 @@ class OrthoOptimizer(Optimizer):
         group[name] = tensor
         return tensor
 
+    @property
+    def _hyperparam_tensors(self) -> Dict[Tuple[int, str], Tensor]:
+        """The persistent device tensors behind ``lr`` (and an opted-in ``weight_decay``); a graph
+        wrapper compares their count before and after capture (dion/cuda_graph.py:212-229)."""
+        return self._hyper_tensors
+
+    def _advance_host_step_counters(self) -> None:
+        """Host-side bookkeeping of one step that a graph replay does not execute
+        (dion/cuda_graph.py:307-311)."""
+        for group in self.param_groups:
+            group["step"] += 1
+
     def _sync_hyperparam_tensors(self) -> None:
         for index in range(len(self.param_groups)):
             for name in self._live_hyperparams(index):

@@ -1,0 +1,108 @@
+"""hipGraph capture of the optimizer step (the contract of the reference's tests/test_cuda_graph.py):
+a wrapped optimizer must follow the eager one bit for bit on every step -- warm-up, the capture step
+and every replay -- with eager work and synchronisations of the test itself between the replays, under
+a constant and a scheduled learning rate, for every optimizer of the package and mixed param groups."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+# GPT-small-like shape groups (several small groups -> the side-stream fork/join is captured too),
+# a per-head group, an AdamW and a Lion group
+SHAPES = [(256, 128), (256, 128), (128, 128), (128, 128), (128, 512), (512, 128), (384, 128)]
+
+
+def _build(cls_name, kwargs, seed):
+    import dion
+
+    torch.manual_seed(seed)
+    mats = [torch.nn.Parameter(torch.randn(s, device=DEV) * 0.02) for s in SHAPES]
+    heads = [torch.nn.Parameter(torch.randn(4 * 32, 96, device=DEV) * 0.02)]
+    vec = [torch.nn.Parameter(torch.randn(300, device=DEV))]
+    emb = [torch.nn.Parameter(torch.randn(64, 48, device=DEV))]
+    groups = [dict(params=mats), dict(params=heads, num_heads=4),
+              dict(params=vec, algorithm="adamw", lr=0.003), dict(params=emb, algorithm="lion", lr=0.001)]
+    opt = getattr(dion, cls_name)(groups, lr=0.02, **kwargs)
+    return mats + heads + vec + emb, opt
+
+
+CASES = [("Muon", dict(nesterov=True)), ("Muon", dict(use_polar_express=False, cautious_wd=True)),
+         ("NorMuon", {}), ("Dion2", dict(fraction=0.25)), ("NorDion2", dict(fraction=0.5)),
+         ("Muon", dict(weight_decay=torch.tensor(0.02)))]
+
+
+@pytest.mark.parametrize("cls_name,kwargs", CASES)
+def test_replay_matches_eager_bit_for_bit(cls_name, kwargs):
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    p_e, o_e = _build(cls_name, dict(kwargs), 5)
+    p_g, inner = _build(cls_name, dict(kwargs), 5)
+    o_g = CudaGraphOptimizer(inner, warmup_steps=2)
+    s_e = torch.optim.lr_scheduler.LambdaLR(o_e, lambda s: 1.0 / (1 + 0.3 * s))
+    s_g = torch.optim.lr_scheduler.LambdaLR(inner, lambda s: 1.0 / (1 + 0.3 * s))
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    for p in p_e + p_g:
+        p.grad = torch.zeros_like(p)
+    for step in range(8):
+        for a, b in zip(p_e, p_g):
+            g = torch.randn(a.shape, device=DEV, generator=gen)
+            a.grad.copy_(g)
+            b.grad.copy_(g)  # in place: the captured graph reads these buffers
+        o_e.step()
+        o_g.step()
+        torch.cuda.synchronize()
+        # eager work of the test between replays
+        junk = torch.randn(256, 256, device=DEV) @ torch.randn(256, 256, device=DEV)
+        assert torch.isfinite(junk).all()
+        for i, (a, b) in enumerate(zip(p_e, p_g)):
+            assert torch.equal(a.data, b.data), (cls_name, step, i)
+        for a, b in zip(p_e, p_g):
+            for key in o_e.state[a]:
+                assert torch.equal(o_e.state[a][key], inner.state[b][key]), (cls_name, step, key)
+        s_e.step()
+        s_g.step()
+        o_g.zero_grad(set_to_none=False)
+    assert o_g._graph is not None
+    assert [g["step"] for g in inner.param_groups] == [g["step"] for g in o_e.param_groups]
+    assert float(inner.state[p_g[-2]]["step_dev"]) == 8.0
+    o_g.release()
+    assert o_g._graph is None
+
+
+def test_float_lr_assignment_reaches_the_graph_and_late_live_wd_is_refused():
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    p_e, o_e = _build("Muon", {}, 6)
+    p_g, inner = _build("Muon", {}, 6)
+    o_g = CudaGraphOptimizer(inner, warmup_steps=1)
+    gen = torch.Generator(device=DEV).manual_seed(10)
+    for p in p_e + p_g:
+        p.grad = torch.zeros_like(p)
+    for step in range(5):
+        for a, b in zip(p_e, p_g):
+            g = torch.randn(a.shape, device=DEV, generator=gen)
+            a.grad.copy_(g)
+            b.grad.copy_(g)
+        lr = 0.02 / (step + 1)
+        o_e.param_groups[0]["lr"] = lr      # the hand-rolled schedule idiom: a plain float
+        inner.param_groups[0]["lr"] = lr
+        o_e.step()
+        o_g.step()
+        for a, b in zip(p_e, p_g):
+            assert torch.equal(a.data, b.data), step
+    inner.param_groups[0]["weight_decay"] = torch.tensor(0.5, device=DEV)
+    with pytest.raises(RuntimeError, match="after the graph was captured"):
+        o_g.step()
+
+
+def test_capture_refuses_params_without_grad():
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    params, inner = _build("Muon", {}, 7)
+    opt = CudaGraphOptimizer(inner, warmup_steps=1)
+    for p in params[:-1]:
+        p.grad = torch.randn_like(p)
+    opt.step()  # warm-up step is eager and simply skips the param without a gradient
+    with pytest.raises(RuntimeError, match="grad=None at graph capture"):
+        opt.step()

@@ -172,3 +172,33 @@ def test_scalar_groups_keep_their_state_contract_and_have_no_cpu_path():
     b.grad = torch.randn(8)
     with pytest.raises(RuntimeError, match="no CPU path"):
         opt.step()
+
+
+def test_graph_wrapper_host_contract():
+    """The wrapper delegates the Optimizer API to the inner optimizer (dion/cuda_graph.py:88-181)."""
+    from dion.cuda_graph import CudaGraphOptimizer
+    from dion_amd import HipGraphOptimizer
+
+    assert CudaGraphOptimizer is HipGraphOptimizer
+    p = _params([(16, 32)])
+    inner = Muon(p, lr=0.02)
+    with pytest.raises(ValueError, match="warmup_steps"):
+        CudaGraphOptimizer(inner, warmup_steps=0)
+    opt = CudaGraphOptimizer(inner, warmup_steps=3)
+    assert isinstance(opt, torch.optim.Optimizer)
+    assert opt.param_groups is inner.param_groups and opt.state is inner.state
+    assert opt.state_dict()["param_groups"][0]["lr"] == pytest.approx(0.02)
+    sched = torch.optim.lr_scheduler.LambdaLR(opt, lambda s: 0.5)   # binds through the wrapper too
+    assert float(inner.param_groups[0]["lr"]) == pytest.approx(0.01)
+    assert sched is not None
+    p[0].grad = torch.ones_like(p[0])
+    with pytest.warns(RuntimeWarning, match="set_to_none"):
+        opt.zero_grad(set_to_none=True)
+    assert p[0].grad is not None and float(p[0].grad.abs().sum()) == 0.0
+    opt.add_param_group({"params": _params([(8, 8)])})
+    assert len(inner.param_groups) == 2 and opt._step_count == 0
+    opt.load_state_dict(inner.state_dict())
+    assert inner._hyperparam_tensors is inner._hyper_tensors
+    steps = [g["step"] for g in inner.param_groups]
+    inner._advance_host_step_counters()
+    assert [g["step"] for g in inner.param_groups] == [s + 1 for s in steps]
