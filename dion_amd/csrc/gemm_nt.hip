@@ -451,9 +451,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
 // ---------------------------------------------------------------------------------------------
 typedef TileCfg<256, 256, 64, 2, 2, 2> Cfg256;
 typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg128;
-typedef TileCfg<256, 256, 32, 2, 2, 4> Cfg256k32;
 typedef TileCfg<256, 256, 64, 2, 4, 2> Cfg256w8;   // 8 wavefronts, 128x64 each: two per SIMD
-typedef TileCfg<256, 256, 64, 4, 2, 2> Cfg256w8b;  // 8 wavefronts, 64x128 each
 typedef TileCfg<256, 256, 32, 2, 4, 4> Cfg256w8k32;  // 8 wavefronts, 4 x 32-deep slabs, spread refill
 typedef TileCfg<256, 256, 64, 2, 4, 2, true> Cfg256w8vg;  // 8 wavefronts, register-staged operands
 typedef TileCfg<128, 128, 64, 2, 2, 2, true> Cfg128vg;
@@ -538,9 +536,7 @@ hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) 
   switch (variant) {
     case 0: return launch_cfg<Cfg256>(p, stream);
     case 1: return launch_cfg<Cfg128>(p, stream);
-    case 2: return launch_cfg<Cfg256k32>(p, stream);
     case 3: return launch_cfg<Cfg256w8>(p, stream);
-    case 4: return launch_cfg<Cfg256w8b>(p, stream);
     case 5: return launch_cfg<Cfg256w8k32>(p, stream);
     case 6: return launch_cfg<Cfg256w8vg>(p, stream);
     case 8: return launch_cfg<Cfg128vg>(p, stream);
