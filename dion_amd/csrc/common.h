@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace dion {
 
 typedef uint16_t bf16_t;  // raw bfloat16 bits in memory
@@ -28,6 +30,20 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   v[0] = (__bf16)lo;
   v[1] = (__bf16)hi;
   return __builtin_bit_cast(uint32_t, v);
+}
+
+// Raises a kernel's dynamic-LDS limit once per device: the attribute belongs to the device that is
+// current when it is set, so `done` keeps one bit per device ordinal.
+static inline hipError_t set_max_dynamic_lds_once(const void* fn, int bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return e;
+  done.fetch_or(bit, std::memory_order_release);
+  return hipSuccess;
 }
 
 // One batched C = alpha * P * Q^T + beta * D problem, all operands row-major bf16 with the

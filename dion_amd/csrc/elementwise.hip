@@ -776,13 +776,9 @@ __global__ __launch_bounds__(1024) void dion2_compact_kernel(int dim, int k, int
 hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
                              int32_t* map, hipStream_t st) {
   const size_t shmem = (size_t)((dim + 3) / 4) * 16;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)dion2_rank_kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_done{0};
+  if (hipError_t e = set_max_dynamic_lds_once((const void*)dion2_rank_kernel, 160 * 1024 - 256, attr_done))
+    return e;
   hipLaunchKernelGGL(dion2_rank_kernel, dim3((dim + 255) / 256, n_mat), dim3(256), shmem, st, norms,
                      dim, k, map);
   hipLaunchKernelGGL(dion2_compact_kernel, dim3(n_mat), dim3(1024), 0, st, dim, k, idx, map);

@@ -458,14 +458,9 @@ typedef TileCfg<128, 128, 64, 2, 2, 2, true> Cfg128vg;
 
 template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false>
 static hipError_t launch_epi(const GemmParams& p, hipStream_t stream) {
-  static bool attr_set = false;
+  static std::atomic<uint64_t> attr_done{0};
   auto kern = gemm_nt_kernel<Cfg, HAS_D, HAS_C, HAS_CT, QK>;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       Cfg::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  if (hipError_t e = set_max_dynamic_lds_once((const void*)kern, Cfg::LDS_BYTES, attr_done)) return e;
   const int tilesM = p.M / Cfg::BM, tilesN = p.N / Cfg::BN;
   const int64_t per_mat = p.tri ? (int64_t)tilesM * (tilesM + 1) / 2 : (int64_t)tilesM * tilesN;
   const int64_t total = per_mat * p.batch;

@@ -263,16 +263,11 @@ hipError_t launch_ns_small(const void* in, int in_dtype, bf16_t* out, int batch,
   const int n = rows < cols ? cols : rows;
   const int n_pad = (n + 63) / 64 * 64;
   const size_t bytes = (size_t)64 * (n_pad * 2 + 16) + 2 * 64 * (64 * 2 + 16);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)ns_small_kernel<bf16_t>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute((const void*)ns_small_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            150 * 1024);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> done_bf16{0}, done_f32{0};
+  if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<bf16_t>, 150 * 1024, done_bf16))
+    return e;
+  if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<float>, 150 * 1024, done_f32))
+    return e;
   if (in_dtype == 0)
     hipLaunchKernelGGL(ns_small_kernel<bf16_t>, dim3(batch), dim3(256), bytes, st, (const bf16_t*)in, out, rows,
                        cols, n_pad, co, norm_scale, eps);
