@@ -1,4 +1,4 @@
-"""CPU oracle for the Muon / NorMuon / Dion2 optimizer-step hot path of microsoft/dion.
+"""CPU oracle for the Muon / NorMuon / Dion2 / NorDion2 optimizer-step hot path of microsoft/dion.
 
 TEST INFRASTRUCTURE ONLY.  This module restates the reference's algorithms on the CPU (numpy
 float64 for exact arithmetic, torch-CPU bfloat16/float32 for the rounding sequence of the eager
@@ -18,6 +18,12 @@ Pinning status (what fixes each function besides re-reading the formula):
     equal-row-energy input gives a multiple of U.                -> tests/test_oracle.py
   * dion2_pre / dion2_post: brute-force sort for the top-k set, fraction == 1 degenerate case,
     unselected entries exactly a*x.                               -> tests/test_oracle.py
+  * nordion2_normalize_selected / nordion2_step: every-row selection reduces to normuon_normalize,
+    unselected entries of V untouched, fraction == 1 and identity-orthogonalization closed
+    forms.                                                        -> tests/test_oracle.py
+  * adamw_update / lion_update: the reference's hand-computed cautious-decay vector
+    (tests/test_adamw_foreach.py:80-112), torch.optim.AdamW as an independent implementation,
+    first-step and blended-sign closed forms for Lion.            -> tests/test_oracle.py
   * gram_ns_fp64: PARITY UNPINNED against the third-party gram-newton-schulz==0.1.6 package
     (not in the reference tree, not installed); pinned only by equality with ns_fp64 in exact
     arithmetic.
