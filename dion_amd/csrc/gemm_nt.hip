@@ -168,7 +168,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
   if (p.tri) {
     tri_tile(t, tilesM, ti, tj);
   } else {
-    constexpr int GM = 4;
+    constexpr int GM = 8;
     const int per_group = GM * tilesN;
     const int g = t / per_group;
     const int first = g * GM;
