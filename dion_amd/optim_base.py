@@ -292,9 +292,12 @@ class OrthoOptimizer(Optimizer):
 
     # Shape groups are independent.  A group whose GEMMs cannot fill the GPU on their own (a few
     # hundred tiles) is run on one of a handful of side streams so that several such groups
-    # overlap; large groups run one after another on the caller's stream.  The reference reaches
+    # overlap; mid-sized groups (kernels of three or four rounds of workgroups) share two streams,
+    # which fills the partial last round of one group's kernels with the other's; large groups run
+    # one after another on the caller's stream, where a second stream only costs L2 locality.  The reference reaches
     # the same goal by interleaving up to three generator tasks (dion/megabatch_base.py:193).
-    _SMALL_GROUP_FLOP = 4e12
+    _SMALL_GROUP_FLOP = 4e12    # below: launches of a few microseconds, four streams
+    _MEDIUM_GROUP_FLOP = 3e13   # below: kernels of a few rounds of workgroups, two streams fill the tails
     _N_SIDE_STREAMS = 4
 
     @staticmethod
@@ -320,8 +323,8 @@ class OrthoOptimizer(Optimizer):
             for group, params in work:
                 self._update_shape_group(group, params)
             return
-        small = [w for w in work if self._group_flop(w[1]) < self._SMALL_GROUP_FLOP]
-        big = [w for w in work if self._group_flop(w[1]) >= self._SMALL_GROUP_FLOP]
+        small = [w for w in work if self._group_flop(w[1]) < self._MEDIUM_GROUP_FLOP]
+        big = [w for w in work if self._group_flop(w[1]) >= self._MEDIUM_GROUP_FLOP]
         # (Running the memory-bound phases of neighbouring large groups under these GEMMs on a
         # second stream was measured: no gain -- the chip is power-limited, not idle.)
         for group, params in big:
@@ -332,6 +335,8 @@ class OrthoOptimizer(Optimizer):
             return
         device = small[0][1][0].device
         pool = self._side_pool(device)
+        if any(self._group_flop(w[1]) >= self._SMALL_GROUP_FLOP for w in small):
+            pool = pool[:2]
         main = torch.cuda.current_stream(device)
         fork = main.record_event()
         used = []
