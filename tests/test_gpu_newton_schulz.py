@@ -1,6 +1,6 @@
 """GPU parity tests for the Newton-Schulz GEMM kernels and the whole orthogonalization, through
 the C ABI, against the CPU oracle.  Tolerances: bf16 orthogonalized outputs within relative
-Frobenius error 2e-2 of the bf16 reference path (BASELINE north star), GEMM kernels no worse than
+Frobenius error 2e-2 of the bf16 reference path, GEMM kernels no worse than
 a bf16 torch matmul measured against float64 (the recipe of the reference's
 tests/test_newton_shulz.py:79-125)."""
 import numpy as np
@@ -288,8 +288,8 @@ def test_gram_square_matrices_stay_in_band():
 
 @pytest.mark.parametrize("shape", [(768, 3072), (3072, 768), (96, 192)])
 def test_kj_newton_schulz_vs_oracle(shape):
-    """Single-matrix Muon NS with the fixed coefficients (BASELINE config 1:
-    dion/muon_reference.py:11-27)."""
+    """Single-matrix Muon NS with the fixed coefficients of dion/muon_reference.py:11-27 on a
+    768x3072 gradient (the reference's own CPU-runnable case)."""
     from dion_amd import zeropower_kj
 
     torch.manual_seed(11)
