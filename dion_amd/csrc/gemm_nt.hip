@@ -1,22 +1,24 @@
-// Batched bf16 "NT" GEMM for gfx950 (CDNA4):  C = alpha * P * Q^T + beta * D, fp32 accumulate.
+// Batched bf16 GEMM for gfx950 (CDNA4):  C = alpha * P * Q^T + beta * D (+ diag * I), fp32 accumulate.
 //
-// Every GEMM of the Newton-Schulz / Polar-Express iteration is expressed in this one form, with
-// both operands contiguous along the reduction dimension, by carrying X and X^T side by side:
+// Every GEMM of the Newton-Schulz / Polar-Express iteration is an instance of this one kernel:
 //   A  = X X^T                     P = Q = X            (tri: upper tiles + mirrored store)
 //   B  = c A A + b A + a I         P = Q = A (A = A^T)  (tri, D = A, a on the diagonal)
-//   X' = B X  (= a X + (B - aI) X)  P = B, Q = X^T, stores X' and (X')^T
-// A second operand form (QK) takes Q stored with the reduction index along rows, [K][N]: X' = B X
-// then reads X itself, its MFMA fragments come from ds_read_b64_tr_b16 (transposing LDS read), and
-// no X^T has to be kept or written.
+//   X' = B X  (= a X + (B - aI) X)  P = B, Q = X
+// P is always read with the reduction index contiguous ("K-contiguous" rows).  Q comes in two forms:
+// K-contiguous rows [N][K] like P (Q^T is then what multiplies P: the Gram products above, or
+// X' = B X given X^T, which also stores (X')^T for the next round), or -- QK -- stored with the
+// reduction index along rows, [K][N]: X' = B X then reads X as it lies, its MFMA fragments come from
+// ds_read_b64_tr_b16 (transposing LDS read), and no X^T has to be kept or written.  QK is the form
+// the orthogonalization driver uses.
 // This replaces the reference's ns_line_1 / ns_line_2 / ns_line_3
 // (dion/newton_schulz_triton.py:88-157, :206-287, :384-447) and the baddbmm of
 // dion/newton_schulz_triton.py:557-563.
 //
 // Kernel structure: one workgroup per BM x BN output tile, WM x WN wavefronts (64 lanes) each
 // owning a (BM/WM) x (BN/WN) sub-tile as 32x32 MFMA accumulators
-// (v_mfma_f32_32x32x16_bf16).  Operand tiles stream global -> LDS with the direct-to-LDS loads
-// (global_load_lds_dwordx4, no VGPR staging) into an NSTAGE ring; a 16-byte-chunk XOR swizzle
-// keeps both the DMA writes and the ds_read_b128 fragment reads bank-conflict free.
+// (v_mfma_f32_32x32x16_bf16).  Operand tiles reach a two-slot LDS ring either through the
+// direct-to-LDS loads (global_load_lds_dwordx4, no VGPR staging) or staged through registers
+// (TileCfg::VG); XOR swizzles keep the LDS writes and the fragment reads bank-conflict free.
 #include <stdlib.h>
 
 #include "common.h"
