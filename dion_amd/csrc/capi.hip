@@ -132,8 +132,9 @@ extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void
 // Whole orthogonalization
 // ---------------------------------------------------------------------------------------------
 namespace {
-// Rows of the workspace matrices are padded by kLdPad elements: a row pitch that is a multiple of
-// 4 KiB sends every row of a tile to the same L2 channel.
+// Optional padding (elements) of the rows of the workspace matrices, for experiments with row
+// pitches that are not powers of two.  Measured on MI355X: pitches of 4 KiB multiples cost nothing
+// (the L2 channel hash spreads them), so the default is 0.
 static int ld_pad() {
   static const int pad = [] {
     const char* e = getenv("DION_LD_PAD");
