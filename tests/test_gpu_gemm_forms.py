@@ -1,0 +1,108 @@
+"""The GEMM kernel through the C ABI (dion_ns_line_1/2/3) over the shapes that exercise every launch
+path: 128- and 256-wide tiles, ragged tile counts, triangular enumeration past one super-block, batch
+counts that do not divide the XCD count, and both forms of the second operand of X' = a X + B X
+(X^T with its reduction index contiguous, or X as it lies).  Each result is compared with the float64
+product of the same bf16 inputs (error no worse than a bf16 torch matmul's), and the two operand
+forms with each other bit for bit: they feed the MFMAs the same values in the same order."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _lib():
+    from dion_amd import _lib as L
+
+    return L.load(), L.check
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _err(res, ref64):
+    d = np.abs(res.float().cpu().numpy().astype(np.float64) - ref64)
+    return d.mean(), d.max()
+
+
+# (batch, m, n): m, n multiples of 128
+SHAPES = [(1, 128, 128), (3, 128, 384), (5, 384, 128), (2, 640, 1152), (9, 256, 512), (1, 2304, 256),
+          (7, 1280, 2560), (33, 512, 768), (2, 2560, 2304)]
+
+
+@pytest.mark.parametrize("batch,m,n", SHAPES)
+def test_line_1_and_2_all_tile_paths(batch, m, n):
+    lib, check = _lib()
+    torch.manual_seed(batch * 1000 + m + n)
+    X = torch.randn(batch, m, n, device=DEV).to(torch.bfloat16)
+    A = torch.empty(batch, m, m, device=DEV, dtype=torch.bfloat16)
+    check(lib.dion_ns_line_1(X.data_ptr(), A.data_ptr(), batch, m, n, _stream()), "line_1")
+    x64 = X.float().cpu().numpy().astype(np.float64)
+    ref = x64 @ np.swapaxes(x64, -2, -1)
+    mean, mx = _err(A, ref)
+    bmean, bmx = _err(X @ X.mT, ref)
+    assert mean <= bmean * 1.05 + 1e-6 and mx <= bmx * 1.5 + 1e-6
+    assert torch.equal(A, A.mT)
+
+    S = (A.float() / n ** 0.5).to(torch.bfloat16)  # symmetric, O(1) entries
+    S = torch.maximum(S, S.mT)                     # exactly symmetric after the rescale
+    B = torch.empty_like(S)
+    check(lib.dion_ns_line_2(S.data_ptr(), B.data_ptr(), batch, m, ctypes.c_float(0.73), ctypes.c_float(-1.31),
+                             _stream()), "line_2")
+    s64 = S.float().cpu().numpy().astype(np.float64)
+    ref2 = 0.73 * (s64 @ s64) - 1.31 * s64
+    mean, mx = _err(B, ref2)
+    bmean, bmx = _err(0.73 * (S @ S) - 1.31 * S, ref2)
+    assert mean <= bmean * 1.05 + 1e-6 and mx <= bmx * 1.5 + 1e-6
+    assert torch.equal(B, B.mT)
+
+
+@pytest.mark.parametrize("a", [0.0, 3.4445])
+@pytest.mark.parametrize("batch,m,n", SHAPES)
+def test_line_3_both_operand_forms(batch, m, n, a):
+    lib, check = _lib()
+    torch.manual_seed(batch * 77 + m + n)
+    X = torch.randn(batch, m, n, device=DEV).to(torch.bfloat16)
+    Xt = X.mT.contiguous()
+    Bm = torch.randn(batch, m, m, device=DEV)
+    Bm = ((Bm + Bm.mT) / 2).to(torch.bfloat16)
+    C_nt = torch.empty_like(X)
+    Ct_nt = torch.empty_like(Xt)
+    C_qk = torch.empty_like(X)
+    Ct_only = torch.empty_like(Xt)
+    st = _stream()
+    check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), Xt.data_ptr(), C_nt.data_ptr(), Ct_nt.data_ptr(), batch,
+                             m, n, ctypes.c_float(a), st), "line_3 (X^T given, both layouts out)")
+    check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), None, C_qk.data_ptr(), None, batch, m, n,
+                             ctypes.c_float(a), st), "line_3 (X as it lies)")
+    check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), Xt.data_ptr(), None, Ct_only.data_ptr(), batch, m, n,
+                             ctypes.c_float(a), st), "line_3 (transposed output only)")
+    x64 = X.float().cpu().numpy().astype(np.float64)
+    b64 = Bm.float().cpu().numpy().astype(np.float64)
+    ref = a * x64 + b64 @ x64
+    mean, mx = _err(C_nt, ref)
+    bmean, bmx = _err(a * X + Bm @ X, ref)
+    assert mean <= bmean * 1.05 + 1e-6 and mx <= bmx * 1.5 + 1e-6
+    assert torch.equal(Ct_nt, C_nt.mT)
+    assert torch.equal(C_qk, C_nt)
+    assert torch.equal(Ct_only, Ct_nt)
+
+
+def test_line_3_argument_errors():
+    lib, check = _lib()
+    from dion_amd._lib import DionHipError
+
+    X = torch.zeros(1, 128, 128, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises((DionHipError, ValueError)):
+        check(lib.dion_ns_line_3(X.data_ptr(), X.data_ptr(), None, None, None, 1, 128, 128, ctypes.c_float(0.0),
+                                 _stream()), "no output")
+    with pytest.raises((DionHipError, ValueError)):
+        check(lib.dion_ns_line_3(X.data_ptr(), X.data_ptr(), None, X.data_ptr(), X.data_ptr(), 1, 128, 128,
+                                 ctypes.c_float(0.0), _stream()), "Ct without Xt")
+    with pytest.raises((DionHipError, ValueError)):
+        check(lib.dion_ns_line_3(X.data_ptr(), X.data_ptr(), None, X.data_ptr(), None, 1, 100, 128,
+                                 ctypes.c_float(0.0), _stream()), "extent not a multiple of 128")
