@@ -103,6 +103,9 @@ def main() -> int:
     ap.add_argument("--optimizer", default="muon", choices=["muon", "normuon", "dion2", "nordion2"])
     ap.add_argument("--graph", action="store_true",
                     help="capture the step into a hipGraph during warm-up and time replays (needs --warmup >= 2)")
+    ap.add_argument("--breakdown", action="store_true",
+                    help="also time momentum / orthogonalization / update of every shape group on its own "
+                         "(adds a 'groups' list to the JSON line)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     args = ap.parse_args()
@@ -276,6 +279,53 @@ def main() -> int:
         }
         del X
         torch.cuda.empty_cache()
+
+    if args.breakdown:
+        # every shape group on its own: Muon's three phases, timed with events on the launch stream
+        from dion_amd import gram_newton_schulz, polar_express, zeropower_via_newtonschulz5
+
+        fn = {"polar_express": polar_express, "gram": gram_newton_schulz}.get(args.ns, zeropower_via_newtonschulz5)
+
+        def timed(f, iters):
+            f()
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                f()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / iters
+
+        lr_t = torch.tensor(0.02, device=dev)
+        rows_out = []
+        for name, rows, cols, count in spec:
+            Xs = [torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen) for _ in range(count)]
+            Gs = [torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen).to(torch.bfloat16)
+                  for _ in range(count)]
+            Ms = [torch.zeros(rows, cols, device=dev) for _ in range(count)]
+            n_el = count * rows * cols
+            it = 20 if n_el < 5e8 else 5
+            ms_pre = timed(lambda: ops.muon_pre(Gs, Ms, 0.95, True), it)
+            U = ops.muon_pre(Gs, Ms, 0.95, True)
+            ms_ns = timed(lambda: fn(U, 1e-8), max(3, it // 2))
+            O = fn(U, 1e-8)
+            ms_post = timed(lambda: ops.muon_post(Xs, O.view(count, -1), lr_t, 0.5, 0.01), it)
+            tf = count * ns_flops(rows, cols) / (ms_ns * 1e-3) * 1e-12
+            rows_out.append({
+                "group": f"{count}x({rows}x{cols}) {name}",
+                "ns_ms": round(ms_ns, 4), "ns_tflops": round(tf, 1),
+                "ns_pct_of_bf16_peak": round(100.0 * tf / PEAK_BF16_TFLOPS, 2),
+                "pre_ms": round(ms_pre, 4), "pre_GBps": round(n_el * 12 / (ms_pre * 1e-3) * 1e-9, 1),
+                "pre_pct_of_hbm_peak": round(100.0 * n_el * 12 / (ms_pre * 1e-3) / 8e12, 2),
+                "post_ms": round(ms_post, 4), "post_GBps": round(n_el * 10 / (ms_post * 1e-3) * 1e-9, 1),
+                "post_pct_of_hbm_peak": round(100.0 * n_el * 10 / (ms_post * 1e-3) / 8e12, 2),
+            })
+            del Xs, Gs, Ms, U, O
+            ops.release_workspaces()
+            torch.cuda.empty_cache()
+        result["groups"] = rows_out
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline("polar_express" if args.ns == "gram" else args.ns)
