@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libdion_hip.so")
-SOURCES = ["gemm_nt.hip", "elementwise.hip", "ns_small.hip", "scalar_opts.hip", "capi.hip"]
+SOURCES = ["gemm_nt.hip", "elementwise.hip", "select_scope.hip", "ns_small.hip", "scalar_opts.hip", "capi.hip"]
 
 # -packed-fp32-ops off: keep hipcc from forming v_pk_*_f32 out of scalar float code.
 HIPCC_FLAGS = [
@@ -21,7 +21,7 @@ HIPCC_FLAGS = [
 
 # The step kernels keep the reference's separate multiply / add roundings (mul_ then add_), so no
 # FMA contraction there; the GEMM epilogues may contract.
-EXTRA_FLAGS = {"elementwise.hip": ["-ffp-contract=off"], "scalar_opts.hip": ["-ffp-contract=off"]}
+EXTRA_FLAGS = {"elementwise.hip": ["-ffp-contract=off"], "select_scope.hip": ["-ffp-contract=off"], "scalar_opts.hip": ["-ffp-contract=off"]}
 
 
 def hipcc_path() -> str:

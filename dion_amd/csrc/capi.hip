@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 4; }
+extern "C" int dion_abi_version(void) { return 5; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -624,6 +624,100 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
                               row_scale ? row_scale + mat0 * k : nullptr, lr_dev, adj_ratio, wd_dev,
                               wd_host, vec4, (hipStream_t)stream),
             "dion_dion2_post");
+  }
+  return DION_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Whole-matrix selection: the sequence a rank runs on assembled matrices under
+// selection_scope="global" (dion/dion2.py:301-343, 565-659; dion/nordion2.py:291-335, 448-500)
+// ---------------------------------------------------------------------------------------------
+static int check_stacked(const char* who, int dtype, int n_mat, int rows, int cols, int select_dim) {
+  if (int rc = check_select_dim(who, select_dim)) return rc;
+  if (dtype != DION_BF16 && dtype != DION_F32) return fail(DION_E_INVALID, "%s: dtype", who);
+  if (n_mat < 0 || rows < 0 || cols < 0) return fail(DION_E_INVALID, "%s: bad size", who);
+  if (n_mat > 65535) return fail(DION_E_INVALID, "%s: more than 65535 matrices in one call", who);
+  return DION_OK;
+}
+
+extern "C" int dion_slice_l1(const void* U, int dtype, int n_mat, int rows, int cols, int select_dim,
+                             int round_bf16, float* norms, void* stream) {
+  if (int rc = check_stacked("dion_slice_l1", dtype, n_mat, rows, cols, select_dim)) return rc;
+  const int dim = select_dim == -2 ? rows : cols;
+  if (n_mat == 0 || dim == 0) return DION_OK;
+  if (!norms) return fail(DION_E_INVALID, "dion_slice_l1: null argument");
+  // empty slices (rows or cols == 0 on the other side) still launch: every norm comes out 0
+  if (!U && rows > 0 && cols > 0) return fail(DION_E_INVALID, "dion_slice_l1: null argument");
+  HIP_TRY(launch_slice_l1(U, dtype, n_mat, rows, cols, select_dim == -2, round_bf16, norms,
+                          (hipStream_t)stream),
+          "dion_slice_l1");
+  return DION_OK;
+}
+
+extern "C" int dion_gather_slices(const void* U, int dtype, int n_mat, int rows, int cols, int select_dim,
+                                  const int32_t* idx, int k, void* sub, void* stream) {
+  if (int rc = check_stacked("dion_gather_slices", dtype, n_mat, rows, cols, select_dim)) return rc;
+  const int dim = select_dim == -2 ? rows : cols;
+  if (k < 0 || k > dim) return fail(DION_E_INVALID, "dion_gather_slices: k outside [0, dim]");
+  if (n_mat == 0 || rows == 0 || cols == 0 || k == 0) return DION_OK;
+  if (!U || !idx || !sub) return fail(DION_E_INVALID, "dion_gather_slices: null argument");
+  HIP_TRY(launch_gather_slices(U, dtype, n_mat, rows, cols, select_dim == -2, idx, k, sub,
+                               (hipStream_t)stream),
+          "dion_gather_slices");
+  return DION_OK;
+}
+
+extern "C" int dion_scatter_slices(const void* sub, int dtype, int n_mat, int rows, int cols,
+                                   int select_dim, const int32_t* map, int k, void* out, void* stream) {
+  if (int rc = check_stacked("dion_scatter_slices", dtype, n_mat, rows, cols, select_dim)) return rc;
+  const int dim = select_dim == -2 ? rows : cols;
+  if (k < 0 || k > dim) return fail(DION_E_INVALID, "dion_scatter_slices: k outside [0, dim]");
+  if (n_mat == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!map || !out || (k > 0 && !sub)) return fail(DION_E_INVALID, "dion_scatter_slices: null argument");
+  HIP_TRY(launch_scatter_slices(sub, dtype, n_mat, rows, cols, select_dim == -2, map, k, out,
+                                (hipStream_t)stream),
+          "dion_scatter_slices");
+  return DION_OK;
+}
+
+extern "C" int dion_mask_index(const float* norms, int n_mat, int dim, int32_t* gate, void* stream) {
+  if (n_mat < 0 || dim < 0) return fail(DION_E_INVALID, "dion_mask_index: bad size");
+  if (n_mat == 0 || dim == 0) return DION_OK;
+  if (!norms || !gate) return fail(DION_E_INVALID, "dion_mask_index: null argument");
+  HIP_TRY(launch_mask_index(norms, n_mat, dim, gate, (hipStream_t)stream), "dion_mask_index");
+  return DION_OK;
+}
+
+extern "C" int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int n,
+                                      int mats_per_ptr, int rows, int cols, int select_dim,
+                                      const void* U, const float* norms, const float* row_scale,
+                                      const float* lr_dev, float adj_ratio, const float* wd_dev,
+                                      float wd_host, float ef_decay, void* stream) {
+  if (int rc = check_select_dim("dion_dion2_post_masked", select_dim)) return rc;
+  if (row_scale && select_dim != -2)
+    return fail(DION_E_INVALID, "dion_dion2_post_masked: row_scale needs select_dim == -2");
+  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0)
+    return fail(DION_E_INVALID, "dion_dion2_post_masked: bad size");
+  if (n == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!X_ptrs || !M_ptrs || !U || !norms || !lr_dev)
+    return fail(DION_E_INVALID, "dion_dion2_post_masked: null argument");
+  for (int i = 0; i < n; ++i)
+    if (!X_ptrs[i] || !M_ptrs[i])
+      return fail(DION_E_INVALID, "dion_dion2_post_masked: tensor %d has a null pointer", i);
+  const int dim = select_dim == -2 ? rows : cols;
+  const bool vec4 = (cols % 4 == 0) && table_aligned(X_ptrs, n) && table_aligned(M_ptrs, n) &&
+                    aligned16((uint64_t)U) && aligned16((uint64_t)norms);
+  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
+    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+    PtrTab x, m;
+    fill_tab(x, X_ptrs + i0, c);
+    fill_tab(m, M_ptrs + i0, c);
+    const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
+    HIP_TRY(launch_dion2_post_masked(x, m, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
+                                     (const bf16_t*)U + mat0 * rows * cols, norms + mat0 * dim,
+                                     row_scale ? row_scale + mat0 * rows : nullptr, lr_dev, adj_ratio,
+                                     wd_dev, wd_host, ef_decay, vec4, (hipStream_t)stream),
+            "dion_dion2_post_masked");
   }
   return DION_OK;
 }

@@ -57,6 +57,21 @@ hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int r
                              const float* row_scale, const float* lr_dev, float adj_ratio,
                              const float* wd_dev, float wd_host, bool vec4, hipStream_t st);
 
+// Whole-matrix selection (select_scope.hip): slice L1 norms of a stacked tensor, dense gather /
+// zero-filled scatter of the selected slices, and the update keyed off the non-zero slices.
+// dtype 0 = bf16, 1 = fp32.
+hipError_t launch_slice_l1(const void* U, int dtype, int n_mat, int rows, int cols, int select_rows,
+                           int round_bf16, float* norms, hipStream_t st);
+hipError_t launch_gather_slices(const void* U, int dtype, int n_mat, int rows, int cols, int select_rows,
+                                const int32_t* idx, int k, void* sub, hipStream_t st);
+hipError_t launch_scatter_slices(const void* sub, int dtype, int n_mat, int rows, int cols,
+                                 int select_rows, const int32_t* map, int k, void* out, hipStream_t st);
+hipError_t launch_mask_index(const float* norms, int n_mat, int dim, int32_t* gate, hipStream_t st);
+hipError_t launch_dion2_post_masked(const PtrTab& X, const PtrTab& M, int n_mat, int mats_per_ptr,
+                                    int rows, int cols, int select_rows, const bf16_t* U,
+                                    const float* norms, const float* row_scale, const float* lr_dev,
+                                    float adj_ratio, const float* wd_dev, float wd_host, float ef_decay,
+                                    bool vec4, hipStream_t st);
 
 // Multi-tensor AdamW / Lion (scalar_opts.hip): n <= kMtaTensors tensors per launch, host arrays of
 // device pointers and element counts.

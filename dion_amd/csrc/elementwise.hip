@@ -447,7 +447,9 @@ hipError_t launch_muon_post(const PtrTab& X, const void* U, int u_dtype, int n, 
 // ------------------------------------------------------------------------------------------
 // Row r of matrix mat keeps its second moment at V[mat][row_idx ? row_idx[mat][r] : r]; V holds
 // v_rows entries per matrix (v_rows == rows without row_idx).  The indirection serves updates made
-// of selected rows only (NorDion2, dion/nordion2.py:430-447).
+// of selected rows only (NorDion2, dion/nordion2.py:430-447).  A negative row_idx entry marks a row
+// that is not part of the update (an all-zero row of a masked full-size tensor,
+// dion/nordion2.py:485-497): its second moment is left alone and its scale is 0.
 // Pass 1: one wavefront per row.  V <- lerp(V, mean(u^2), w);  tmp[row] = sum(u^2).
 __global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restrict__ U, PtrTab V,
                                                            int mats_per_ptr, int rows, int cols,
@@ -480,11 +482,13 @@ __global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restr
   s = wave_sum(s);
   if (lane == 0) {
     const int vr = row_idx ? row_idx[(int64_t)mat * rows + row] : row;
-    float* v = (float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * v_rows + vr;
-    const float mean = s / (float)cols;
-    const float vo = *v;
-    *v = vo + w * (mean - vo);  // torch.lerp for weight < 0.5
-    rowsq[(int64_t)mat * rows + row] = s;
+    if (vr >= 0) {
+      float* v = (float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * v_rows + vr;
+      const float mean = s / (float)cols;
+      const float vo = *v;
+      *v = vo + w * (mean - vo);  // torch.lerp for weight < 0.5
+    }
+    rowsq[(int64_t)mat * rows + row] = vr >= 0 ? s : 0.f;
   }
 }
 
@@ -501,7 +505,8 @@ __global__ __launch_bounds__(1024) void normuon_scale_kernel(PtrTab V, int mats_
   float s1 = 0.f, s2 = 0.f;
   for (int r = threadIdx.x; r < rows; r += 1024) {
     const float q = sc[r];
-    const float inv = 1.0f / (sqrtf(v[ri ? ri[r] : r]) + 1e-8f);
+    const int vr = ri ? ri[r] : r;
+    const float inv = vr >= 0 ? 1.0f / (sqrtf(v[vr]) + 1e-8f) : 0.f;
     s1 += q;
     s2 += q * inv * inv;
   }
@@ -510,8 +515,8 @@ __global__ __launch_bounds__(1024) void normuon_scale_kernel(PtrTab V, int mats_
   const float ratio = sqrtf(s1) / fmaxf(sqrtf(s2), 1e-8f);
   __syncthreads();
   for (int r = threadIdx.x; r < rows; r += 1024) {
-    const float inv = 1.0f / (sqrtf(v[ri ? ri[r] : r]) + 1e-8f);
-    sc[r] = inv * ratio;
+    const int vr = ri ? ri[r] : r;
+    sc[r] = vr >= 0 ? (1.0f / (sqrtf(v[vr]) + 1e-8f)) * ratio : 0.f;
   }
 }
 

@@ -5,6 +5,7 @@ hands raw device pointers and the current stream to the library, and returns tor
 torch is used for device memory and streams only; all arithmetic happens in the HIP kernels.
 There is no CPU implementation behind these functions: CPU tensors raise.
 """
+import math
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -362,6 +363,131 @@ def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: 
         rs = row_scale.data_ptr()
     check(lib.dion_dion2_post(xp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(), k, imap.data_ptr(),
                               rs, lr_p, float(adj_ratio), wd_p, wd_h, _stream_handle(U.device)), "dion2_post")
+
+
+# ---------------------------------------------------------------------------------------------
+# whole-matrix selection (selection_scope="global"): select inside the orthogonalization call,
+# update keyed off the non-zero slices
+# ---------------------------------------------------------------------------------------------
+def _stacked(U: Tensor, name: str) -> Tuple[int, int, int, int]:
+    """(dtype code, n_mat, rows, cols) of a contiguous stacked ``[..., rows, cols]`` GPU tensor."""
+    _require_gpu(U, name)
+    if U.dim() < 2:
+        raise ValueError(f"{name} must have at least 2 dimensions, got shape {tuple(U.shape)}")
+    if not U.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    rows, cols = U.shape[-2], U.shape[-1]
+    n_mat = U.numel() // (rows * cols) if rows * cols else math.prod(U.shape[:-2])
+    return _dtype_code(U, name), n_mat, rows, cols
+
+
+def slice_l1(U: Tensor, select_dim: int, round_bf16: bool = False) -> Tensor:
+    """L1 norm of every slice of ``U [..., rows, cols]`` (bf16 or fp32) along ``select_dim``: fp32
+    ``[n_mat, dim]``.  ``round_bf16`` rounds the result to bf16 precision, which is what
+    ``X.norm(p=1, dim=...)`` returns for a bf16 ``X`` (dion/dion2.py:602)."""
+    if select_dim not in (-2, -1):
+        raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
+    code, n_mat, rows, cols = _stacked(U, "U")
+    dim = rows if select_dim == -2 else cols
+    norms = torch.empty(n_mat, dim, dtype=torch.float32, device=U.device)
+    lib = _lib.load()
+    check(lib.dion_slice_l1(U.data_ptr(), code, n_mat, rows, cols, select_dim, int(bool(round_bf16)),
+                            norms.data_ptr(), _stream_handle(U.device)), "slice_l1")
+    return norms
+
+
+def select_slices(U: Tensor, k: int, select_dim: int):
+    """Top-``k`` slices of every matrix of ``U [..., rows, cols]`` by L1 norm along ``select_dim``
+    (dion/dion2.py:600-610).  Returns (sub, idx int32 [n_mat, k] ascending, map int32 [n_mat, dim]);
+    ``sub`` is ``[..., k, cols]`` or ``[..., rows, k]`` in the dtype of ``U``."""
+    code, n_mat, rows, cols = _stacked(U, "U")
+    dim = rows if select_dim == -2 else cols
+    if not (0 <= k <= dim):
+        raise ValueError(f"k={k} outside [0, {dim}]")
+    norms = slice_l1(U, select_dim, round_bf16=U.dtype == torch.bfloat16)
+    dev = U.device
+    idx = torch.empty(n_mat, k, dtype=torch.int32, device=dev)
+    imap = torch.empty(n_mat, dim, dtype=torch.int32, device=dev)
+    sub_shape = (*U.shape[:-2], k, cols) if select_dim == -2 else (*U.shape[:-2], rows, k)
+    sub = torch.empty(sub_shape, dtype=U.dtype, device=dev)
+    lib = _lib.load()
+    st = _stream_handle(dev)
+    check(lib.dion_dion2_topk(norms.data_ptr(), n_mat, dim, k, idx.data_ptr(), imap.data_ptr(), st),
+          "dion2_topk")
+    check(lib.dion_gather_slices(U.data_ptr(), code, n_mat, rows, cols, select_dim, idx.data_ptr(), k,
+                                 sub.data_ptr(), st), "gather_slices")
+    return sub, idx, imap
+
+
+def scatter_slices(sub: Tensor, imap: Tensor, shape, select_dim: int) -> Tensor:
+    """Full-size tensor of ``shape [..., rows, cols]`` that holds ``sub`` at the slices ``imap`` marks and
+    zero elsewhere (dion/dion2.py:612-613)."""
+    if select_dim not in (-2, -1):
+        raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
+    code, n_mat, srows, scols = _stacked(sub, "sub")
+    rows, cols = shape[-2], shape[-1]
+    k = srows if select_dim == -2 else scols
+    if (select_dim == -2 and scols != cols) or (select_dim == -1 and srows != rows):
+        raise ValueError(f"sub {tuple(sub.shape)} does not fit into {tuple(shape)} along dim {select_dim}")
+    dim = rows if select_dim == -2 else cols
+    if imap.dtype != torch.int32 or not imap.is_contiguous() or imap.numel() != n_mat * dim:
+        raise ValueError("map must be a contiguous int32 tensor of n_mat * dim entries")
+    out = torch.empty(tuple(shape), dtype=sub.dtype, device=sub.device)
+    if out.numel() != n_mat * rows * cols:
+        raise ValueError(f"shape {tuple(shape)} does not hold {n_mat} matrices")
+    lib = _lib.load()
+    check(lib.dion_scatter_slices(sub.data_ptr(), code, n_mat, rows, cols, select_dim, imap.data_ptr(), k,
+                                  out.data_ptr(), _stream_handle(sub.device)), "scatter_slices")
+    return out
+
+
+def mask_index(norms: Tensor) -> Tensor:
+    """int32 ``[n_mat, dim]``: the slice's own index where its norm is > 0, -1 elsewhere."""
+    _require_gpu(norms, "norms")
+    if norms.dtype != torch.float32 or norms.dim() != 2 or not norms.is_contiguous():
+        raise ValueError("norms must be a contiguous float32 [n_mat, dim] tensor")
+    gate = torch.empty(norms.shape, dtype=torch.int32, device=norms.device)
+    lib = _lib.load()
+    check(lib.dion_mask_index(norms.data_ptr(), norms.shape[0], norms.shape[1], gate.data_ptr(),
+                              _stream_handle(norms.device)), "mask_index")
+    return gate
+
+
+def dion2_post_masked(X: List[Tensor], M: List[Tensor], U: Tensor, norms: Tensor, lr: Tensor,
+                      adj_ratio: float, weight_decay, ef_decay: float, select_dim: int,
+                      row_scale: Optional[Tensor] = None) -> None:
+    """``x = (1 - lr*wd)*x - lr*adj_ratio*u`` over every ``X[i]`` and ``m *= ef_decay`` on the slices of
+    ``M[i]`` whose entry of ``norms`` (``slice_l1(U)``) is > 0.  ``U [N, ..., rows, cols]`` bf16 is zero
+    off the selected slices.  Mirrors ``dion2_post_orthogonalize_masked`` (dion/dion2.py:623-659);
+    ``row_scale [n_mat, rows]`` (rows selected only) multiplies each row of ``U`` first."""
+    if select_dim not in (-2, -1):
+        raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
+    n = len(X)
+    assert n > 0 and len(M) == n
+    shape = X[0].shape
+    rows, cols = shape[-2], shape[-1]
+    numel = X[0].numel()
+    mats_per_ptr = numel // (rows * cols)
+    n_mat = n * mats_per_ptr
+    xp = _list_ptrs(X, "X", torch.float32, numel)
+    mp = _list_ptrs(M, "M", torch.float32, numel)
+    _check_bf16(U, "U")
+    if not U.is_contiguous() or U.numel() != n * numel:
+        raise ValueError("U must be a contiguous [N, *shape] arena")
+    dim = rows if select_dim == -2 else cols
+    if norms.dtype != torch.float32 or not norms.is_contiguous() or norms.numel() != n_mat * dim:
+        raise ValueError("norms must be a contiguous float32 tensor of n_mat * dim entries")
+    rs = None
+    if row_scale is not None:
+        if row_scale.dtype != torch.float32 or not row_scale.is_contiguous() or \
+                row_scale.numel() != n_mat * rows:
+            raise ValueError("row_scale must be a contiguous float32 tensor of n_mat * rows entries")
+        rs = row_scale.data_ptr()
+    lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, U.device)
+    lib = _lib.load()
+    check(lib.dion_dion2_post_masked(xp, mp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(),
+                                     norms.data_ptr(), rs, lr_p, float(adj_ratio), wd_p, wd_h,
+                                     float(ef_decay), _stream_handle(U.device)), "dion2_post_masked")
 
 
 # ---------------------------------------------------------------------------------------------

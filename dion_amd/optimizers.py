@@ -17,7 +17,7 @@ from typing import Callable, List, Optional, Tuple, Union
 import torch
 from torch import Tensor
 
-from . import ops
+from . import global_scope, ops
 from .optim_base import OrthoOptimizer, adjust_lr_ratio, split_lr_scales
 
 
@@ -170,9 +170,13 @@ class NorMuon(_MomentumOrtho):
 class Dion2(OrthoOptimizer):
     """Dion2 on one MI355X.  Same arguments as the reference ``Dion2`` (dion/dion2.py:60-79).
     ``triton_post_ortho`` is accepted and selects nothing (the fused single-rounding post kernel is
-    the only one); ``selection_scope`` only matters for sharded parameters and is validated only."""
+    the only one).  ``selection_scope="global"`` changes the sequence only for sharded parameters in
+    the reference (dion/dion2.py:284); with whole matrices it is the index-based sequence unless
+    ``assembled_selection`` is set, in which case the step runs what a rank runs on assembled
+    matrices: accumulate, select inside the orthogonalization call, masked update."""
 
     _printed = set()
+    assembled_selection = False
 
     def __init__(self, params, distributed_mesh=None, lr: float = 0.01, fraction: float = 0.25,
                  ef_decay: float = 0.95, betas: Tuple[float, float] = (0.9, 0.95),
@@ -232,6 +236,26 @@ class Dion2(OrthoOptimizer):
         M = [self._get_or_initialize_state(p, self._algo_name)["momentum"].view(mats, rows, cols)
              for p in params]
 
+        if self.assembled_selection and group["selection_scope"] == "global":
+            if flatten and len(shape) >= 3:
+                raise NotImplementedError("Dion2: whole-matrix selection with flatten=True is built for "
+                                          "2D parameters only.")
+            # accumulate -> select inside the orthogonalization call -> masked update
+            # (dion/dion2.py:301-343)
+            U_full = global_scope.dion2_pre_accumulate(G, M)
+            yield
+            _note_stream(U_full)
+            select_ns = global_scope.make_select_and_orthogonalize(
+                lambda t, epsilon=None: self._orthogonalize(t, float(epsilon)), group["fraction"], select_dim)
+            O = select_ns(U_full.view(n * mats, rows, cols), epsilon=float(group["epsilon"]))
+            del U_full
+            yield
+            _note_stream(O)
+            ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
+            global_scope.dion2_post_orthogonalize_masked(X, M, O.view(n, mats, rows, cols), group["lr"], ratio,
+                                                         group["weight_decay"], group["ef_decay"], select_dim)
+            return
+
         U_sel, _idx, imap = ops.dion2_select(G, M, k, select_dim, group["ef_decay"])
         sel_rows, sel_cols = U_sel.shape[-2], U_sel.shape[-1]
         yield
@@ -258,7 +282,10 @@ class NorDion2(OrthoOptimizer):
     branch): ``M += G``; the ``ceil(fraction * rows)`` rows of largest L1 norm are selected (always
     rows, so that a selected slice is a whole neuron); those rows of ``M`` decay by ``mu``; the
     selected block is orthogonalized; NorMuon's per-row second-moment normalisation runs on it
-    against the selected entries of ``variance_neuron``; the scaled rows update ``X``."""
+    against the selected entries of ``variance_neuron``; the scaled rows update ``X``.
+    ``assembled_selection`` as for ``Dion2``."""
+
+    assembled_selection = False
 
     def __init__(self, params, distributed_mesh=None, lr: float = 0.01, fraction: float = 0.25,
                  mu: float = 0.95, muon_beta2: float = 0.95, betas: Tuple[float, float] = (0.9, 0.95),
@@ -318,6 +345,24 @@ class NorDion2(OrthoOptimizer):
         states = [self._get_or_initialize_state(p, self._algo_name) for p in params]
         M = [s["momentum"].view(mats, rows, cols) for s in states]
         V = [s["variance_neuron"].view(mats, rows, 1) for s in states]
+
+        if self.assembled_selection and group["selection_scope"] == "global":
+            # accumulate -> select inside the orthogonalization call -> masked normalisation and update
+            # (dion/nordion2.py:291-335)
+            U_full = global_scope.dion2_pre_accumulate(G, M)
+            yield
+            _note_stream(U_full)
+            select_ns = global_scope.make_select_and_orthogonalize(
+                lambda t, epsilon=None: self._orthogonalize(t, float(epsilon)), group["fraction"], select_dim)
+            O = select_ns(U_full.view(n * mats, rows, cols), epsilon=float(group["epsilon"]))
+            del U_full
+            yield
+            _note_stream(O)
+            ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
+            global_scope.nordion2_post_orthogonalize_masked(
+                X, M, V, O.view(n, mats, rows, cols), group["lr"], ratio, group["weight_decay"], group["mu"],
+                group["muon_beta2"], select_dim)
+            return
 
         # error-feedback decay of the selected rows is the momentum factor (dion/nordion2.py:352-359)
         U_sel, idx, imap = ops.dion2_select(G, M, k, select_dim, group["mu"])

@@ -173,6 +173,49 @@ int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, i
                     float wd_host, void* stream);
 
 /* --------------------------------------------------------------------------------------------
+ * Whole-matrix selection: what a rank runs on assembled matrices when the top-k is taken inside
+ * the orthogonalization call and the update only sees a full-size tensor that is zero outside the
+ * selected slices (selection_scope="global").  Stacked tensors are contiguous [n_mat, rows, cols];
+ * dtype is DION_BF16 or DION_F32; n_mat <= 65535.
+ * ------------------------------------------------------------------------------------------ */
+
+/* norms[i][s] = sum |U_i[slice s]| (fp32 accumulate; round_bf16 != 0 rounds the result to bf16,
+ * which is what a bf16 input gets from Tensor.norm).  norms out [n_mat, dim] fp32.
+ * Replaces X.norm(p=1, dim=norm_dim) at dion/dion2.py:602 and the non-zero test
+ * u.abs().sum(dim) > 0 at dion/dion2.py:648, dion/nordion2.py:487. */
+int dion_slice_l1(const void* U, int dtype, int n_mat, int rows, int cols, int select_dim,
+                  int round_bf16, float* norms, void* stream);
+
+/* sub_i = U_i[selected slices], idx [n_mat, k] int32 as written by dion_dion2_topk;
+ * sub [n_mat, k, cols] (select_dim -2) or [n_mat, rows, k] (select_dim -1), same dtype as U.
+ * Replaces torch.gather at dion/dion2.py:604-610. */
+int dion_gather_slices(const void* U, int dtype, int n_mat, int rows, int cols, int select_dim,
+                       const int32_t* idx, int k, void* sub, void* stream);
+
+/* out_i = zeros;  out_i[selected slices] = sub_i.  map [n_mat, dim] int32 is the dense inverse map
+ * of dion_dion2_topk; every element of out is written (no prior clear needed).
+ * Replaces zeros_like + scatter_ at dion/dion2.py:612-613. */
+int dion_scatter_slices(const void* sub, int dtype, int n_mat, int rows, int cols, int select_dim,
+                        const int32_t* map, int k, void* out, void* stream);
+
+/* gate[i][s] = s where norms[i][s] > 0, else -1: the row_idx form dion_normuon_stats_selected takes,
+ * in which a negative entry leaves that row's second moment untouched and gives it scale 0
+ * (torch.where(sel, v_new, v) at dion/nordion2.py:494). */
+int dion_mask_index(const float* norms, int n_mat, int dim, int32_t* gate, void* stream);
+
+/* Masked Dion2 / NorDion2 update, single rounding of the sum:
+ *   x = (1 - lr wd) x - lr adj_ratio u   everywhere (u [n_mat, rows, cols] bf16, zero off the
+ *   selected slices);   m *= ef_decay   on slices with norms[i][s] > 0
+ * norms as written by dion_slice_l1 on U.  row_scale (nullable, select_dim -2 only): device
+ * [n_mat, rows] fp32, row r of u is multiplied by row_scale[i][r] first.
+ * Replaces dion2_post_orthogonalize_masked (dion/dion2.py:623-659) and, with row_scale, the update
+ * half of nordion2_post_orthogonalize_masked (dion/nordion2.py:448-500). */
+int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int n, int mats_per_ptr,
+                           int rows, int cols, int select_dim, const void* U, const float* norms,
+                           const float* row_scale, const float* lr_dev, float adj_ratio,
+                           const float* wd_dev, float wd_host, float ef_decay, void* stream);
+
+/* --------------------------------------------------------------------------------------------
  * Multi-tensor AdamW / Lion for the non-matrix parameter groups (algorithm "adamw" / "lion").
  * X_ptrs, G_ptrs, M_ptrs, V_ptrs: host ptr tables of n device pointers; tensor i has numels[i]
  * elements (host array); X, M, V fp32, G bf16 or fp32 per g_dtype (one dtype per call).

@@ -21,6 +21,12 @@ Pinning status (what fixes each function besides re-reading the formula):
   * nordion2_normalize_selected / nordion2_step: every-row selection reduces to normuon_normalize,
     unselected entries of V untouched, fraction == 1 and identity-orthogonalization closed
     forms.                                                        -> tests/test_oracle.py
+  * dion2_pre_accumulate / select_and_orthogonalize / dion2_post_masked / nordion2_post_masked
+    (the whole-matrix "global" selection sequence): the reference's own padded-matrix case
+    (17 real + 3 zero rows, fraction 0.35 -> 6 selected, tests/test_dion2_selection_scope.py:138-169),
+    brute-force top-k, and equality of the masked sequence with the index-based one (dion2_pre /
+    dion2_post / nordion2_step, written separately) whenever both pick the same slices.
+                                                                  -> tests/test_oracle.py
   * adamw_update / lion_update: the reference's hand-computed cautious-decay vector
     (tests/test_adamw_foreach.py:80-112), torch.optim.AdamW as an independent implementation,
     first-step and blended-sign closed forms for Lion.            -> tests/test_oracle.py
@@ -302,6 +308,68 @@ def dion2_post(X: torch.Tensor, U: torch.Tensor, idx: torch.Tensor, lr: float, a
         full[:, idx] = U.to(torch.float64)
     out = a.double() * X.double() - b.double() * full
     return out.to(torch.float32)
+
+
+def dion2_pre_accumulate(G: torch.Tensor, M: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dion/dion2.py:546-563 for one matrix: returns (M + G, its bf16 copy)."""
+    M_new = M + G.to(M.dtype)
+    return M_new, M_new.to(torch.bfloat16)
+
+
+def select_and_orthogonalize(X: torch.Tensor, fraction: float, select_dim: int, ns,
+                             global_select_size: Optional[int] = None):
+    """dion/dion2.py:596-614 for one matrix X [rows, cols]: top-k slices by L1 norm (the norm of a
+    bf16 tensor is itself bf16), ``ns`` on the dense block, scattered into zeros.  Ties go to the
+    lower index.  Returns (full-size result in X.dtype, sorted index tensor)."""
+    have = X.size(select_dim)
+    num_select = have if global_select_size is None else global_select_size
+    k = min(max(1, int(math.ceil(fraction * num_select))), have)
+    norm_dim = -1 if select_dim == -2 else -2
+    norms = X.float().abs().sum(dim=norm_dim).to(X.dtype)
+    order = sorted(range(have), key=lambda i: (-float(norms[i]), i))
+    idx = torch.tensor(sorted(order[:k]), dtype=torch.long)
+    sub = X[idx, :] if select_dim == -2 else X[:, idx]
+    ortho = ns(sub).to(X.dtype)
+    out = torch.zeros_like(X)
+    if select_dim == -2:
+        out[idx, :] = ortho
+    else:
+        out[:, idx] = ortho
+    return out, idx
+
+
+def _nonzero_slices(U: torch.Tensor, select_dim: int) -> torch.Tensor:
+    """dion/dion2.py:648: boolean mask, keepdim, over the slices of U that are not all zero."""
+    norm_dim = -1 if select_dim == -2 else -2
+    return U.to(torch.float32).abs().sum(dim=norm_dim, keepdim=True) > 0
+
+
+def dion2_post_masked(X: torch.Tensor, M: torch.Tensor, U: torch.Tensor, lr: float, adj_ratio: float, wd: float,
+                      ef_decay: float, select_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dion/dion2.py:623-659 for one matrix, the weight update in the single-rounding form of
+    ``dion2_post``.  Returns (X_new, M_new)."""
+    sel = _nonzero_slices(U, select_dim)
+    M_new = M * torch.where(sel, torch.tensor(ef_decay, dtype=M.dtype), torch.ones((), dtype=M.dtype))
+    lr_t = torch.tensor(lr, dtype=torch.float32)
+    a = 1 - lr_t * torch.tensor(wd, dtype=torch.float32)
+    b = lr_t * torch.tensor(adj_ratio, dtype=torch.float32)
+    X_new = (a.double() * X.double() - b.double() * U.double()).to(torch.float32)
+    return X_new, M_new
+
+
+def nordion2_post_masked(X: torch.Tensor, M: torch.Tensor, V: torch.Tensor, U: torch.Tensor, lr: float,
+                         adj_ratio: float, wd: float, ef_decay: float, beta2: float):
+    """dion/nordion2.py:448-500 for one matrix (rows selected): NorMuon normalisation over the full,
+    mostly-zero U; V written back on the non-zero rows only.  Returns (X_new, M_new, V_new)."""
+    sel = _nonzero_slices(U, -2)
+    M_new = M * torch.where(sel, torch.tensor(ef_decay, dtype=M.dtype), torch.ones((), dtype=M.dtype))
+    nU, v_new = normuon_normalize(U, V.float(), beta2)
+    V_new = torch.where(sel, v_new.to(V.dtype), V)
+    lr_t = torch.tensor(lr, dtype=torch.float32)
+    a = 1 - lr_t * torch.tensor(wd, dtype=torch.float32)
+    b = lr_t * torch.tensor(adj_ratio, dtype=torch.float32)
+    X_new = (a.double() * X.double() - b.double() * nU.double()).to(torch.float32)
+    return X_new, M_new, V_new
 
 
 def nordion2_normalize_selected(U: torch.Tensor, V_full: torch.Tensor, idx: torch.Tensor, beta2: float):

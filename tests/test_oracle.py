@@ -253,6 +253,80 @@ def test_nordion2_step_closed_cases():
     assert torch.equal(m3[mask], acc[mask]) and torch.equal(x3[mask], (x * torch.tensor(1 - 0.02 * 0.01))[mask])
 
 
+def test_whole_matrix_selection_known_answer_and_bruteforce():
+    """The reference's padded case (tests/test_dion2_selection_scope.py:138-169): 17 real rows + 3 zero
+    rows, fraction 0.35 and the true size 17 -> 6 rows selected, none of them padding; without the true
+    size it would be 7.  Then brute force: the selected slices are the k largest by L1 norm, the result
+    equals ns(sub) there and is exactly zero elsewhere."""
+    torch.manual_seed(0)
+    X = torch.cat([torch.randn(17, 6), torch.zeros(3, 6)], dim=0)
+    ident = lambda t: t
+    out, idx = o.select_and_orthogonalize(X, 0.35, -2, ident, global_select_size=17)
+    assert int((out.abs().sum(-1) > 0).sum()) == math.ceil(0.35 * 17) == 6
+    assert float(out[17:].abs().sum()) == 0.0 and int(idx.max()) < 17
+    out7, _ = o.select_and_orthogonalize(X, 0.35, -2, ident)
+    assert int((out7.abs().sum(-1) > 0).sum()) == 7
+    # k never exceeds what the matrix holds
+    out_all, idx_all = o.select_and_orthogonalize(X[:4], 0.9, -2, ident, global_select_size=100)
+    assert idx_all.numel() == 4 and torch.equal(out_all, X[:4])
+    for sd, dim in [(-2, 20), (-1, 6)]:
+        Y = torch.randn(20, 6)
+        dbl = lambda t: 2 * t
+        out, idx = o.select_and_orthogonalize(Y, 0.5, sd, dbl)
+        k = math.ceil(0.5 * dim)
+        norms = Y.abs().sum(dim=1 if sd == -2 else 0)
+        top = set(torch.sort(norms, descending=True).indices[:k].tolist())
+        assert set(idx.tolist()) == top
+        mask = torch.zeros(dim, dtype=torch.bool)
+        mask[idx] = True
+        if sd == -2:
+            assert torch.equal(out[mask], 2 * Y[mask]) and float(out[~mask].abs().sum()) == 0.0
+        else:
+            assert torch.equal(out[:, mask], 2 * Y[:, mask]) and float(out[:, ~mask].abs().sum()) == 0.0
+    # bf16 input: norms are compared at bf16 precision, ties go to the lower index
+    Z = torch.ones(4, 256, dtype=torch.bfloat16)
+    Z[2, 0] = 1.5  # 256.5 rounds to 256 in bf16: a four-way tie
+    _, idx = o.select_and_orthogonalize(Z, 0.5, -2, ident)
+    assert idx.tolist() == [0, 1]
+
+
+def test_masked_sequence_equals_index_sequence():
+    """accumulate -> select inside -> masked update gives the same X, M (and V) as the index-based
+    dion2_pre -> dion2_post (nordion2_step), which are written separately, whenever both pick the same
+    slices: here the slice norms are far apart, so they do."""
+    torch.manual_seed(11)
+    scale = torch.tensor([1.0, 3.0, 0.2, 5.0, 0.5, 2.0, 0.1, 4.0])
+    for sd in (-2, -1):
+        shape = (8, 12) if sd == -2 else (12, 8)
+        g = torch.randn(shape)
+        g = (g * (scale[:, None] if sd == -2 else scale[None, :])).to(torch.bfloat16)
+        m = torch.randn(shape) * 0.01
+        x = torch.randn(shape) * 0.02
+        ns = lambda u: (u.float() * 0.5).to(torch.bfloat16)
+        m_idx, u_sel, idx = o.dion2_pre(g, m, 0.25, 0.9, sd)
+        x_idx = o.dion2_post(x, ns(u_sel), idx, 0.02, 1.5, 0.1, sd)
+        m_acc, u_full = o.dion2_pre_accumulate(g, m)
+        full, idx2 = o.select_and_orthogonalize(u_full, 0.25, sd, ns)
+        assert torch.equal(idx, idx2) and idx.numel() == 2
+        x_msk, m_msk = o.dion2_post_masked(x, m_acc, full, 0.02, 1.5, 0.1, 0.9, sd)
+        assert torch.equal(x_idx, x_msk) and torch.equal(m_idx, m_msk)
+    # NorDion2 (rows): same comparison including the second moments
+    g = (torch.randn(8, 12) * scale[:, None]).to(torch.bfloat16)
+    m = torch.randn(8, 12) * 0.01
+    x = torch.randn(8, 12) * 0.02
+    v = torch.rand(8, 1) * 1e-2
+    ns = lambda u: (u.float() * 0.5).to(torch.bfloat16)
+    x_idx, m_idx, v_idx, idx = o.nordion2_step(x, g, m, v, 0.02, 0.25, 0.95, 0.9, 0.1, "spectral_norm", ns=ns)
+    m_acc, u_full = o.dion2_pre_accumulate(g, m)
+    full, idx2 = o.select_and_orthogonalize(u_full, 0.25, -2, ns)
+    assert torch.equal(idx, idx2)
+    x_msk, m_msk, v_msk = o.nordion2_post_masked(x, m_acc, v, full, 0.02, o.adjust_lr_ratio(x.shape, "spectral_norm"),
+                                                 0.1, 0.95, 0.9)
+    assert torch.equal(m_idx, m_msk)
+    assert torch.allclose(v_idx, v_msk, rtol=1e-6, atol=0) and torch.equal(v_msk[[0, 2, 4, 6]], v[[0, 2, 4, 6]])
+    assert torch.allclose(x_idx, x_msk, rtol=1e-5, atol=1e-8)
+
+
 def test_adamw_restatement_known_answers():
     """The reference's hand-computed cautious-weight-decay vector (tests/test_adamw_foreach.py:80-112):
     mask [1, 0, 0, 1], two positions decayed, two not.  Plus torch.optim.AdamW as an independent
