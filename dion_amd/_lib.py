@@ -44,8 +44,9 @@ SIGNATURES = {
     "dion_dion2_topk": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "dion_dion2_gather": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
                                   c_void_p, c_void_p]),
-    "dion_dion2_post": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
-                                c_void_p, c_void_p, c_float, c_void_p, c_float, c_void_p]),
+    "dion_dion2_post": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p,
+                                c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float, c_void_p]),
+    "dion_dion2_index_map": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "dion_slice_l1": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "dion_gather_slices": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
                                    c_void_p]),
@@ -53,7 +54,8 @@ SIGNATURES = {
                                     c_void_p]),
     "dion_mask_index": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "dion_dion2_post_masked": (c_int, [_u64p, _u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
-                                       c_void_p, c_void_p, c_float, c_void_p, c_float, c_float, c_void_p]),
+                                       c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float, c_float,
+                                       c_void_p]),
     "dion_adamw_step": (c_int, [_u64p, _u64p, c_int, _u64p, _u64p, _u64p, _i64p, c_int, c_void_p, c_float,
                                 c_float, c_float, c_void_p, c_float, c_int, c_void_p]),
     "dion_lion_step": (c_int, [_u64p, _u64p, c_int, _u64p, _i64p, c_int, c_void_p, c_float, c_float,

@@ -599,10 +599,11 @@ extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr
 }
 
 extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, int cols,
-                               int select_dim, const void* U_sel, int k, const int32_t* map,
-                               const float* row_scale, const float* lr_dev, float adj_ratio,
-                               const float* wd_dev, float wd_host, void* stream) {
+                               int select_dim, const void* U_sel, int u_dtype, int k, const int32_t* map,
+                               const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
+                               float adj_ratio, const float* wd_dev, float wd_host, void* stream) {
   if (int rc = check_select_dim("dion_dion2_post", select_dim)) return rc;
+  if (u_dtype != DION_BF16 && u_dtype != DION_F32) return fail(DION_E_INVALID, "dion_dion2_post: u_dtype");
   if (row_scale && select_dim != -2)
     return fail(DION_E_INVALID, "dion_dion2_post: row_scale needs select_dim == -2");
   if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || k < 0)
@@ -612,6 +613,7 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
     return fail(DION_E_INVALID, "dion_dion2_post: null argument");
   const int dim = select_dim == -2 ? rows : cols;
   const int64_t sel_numel = select_dim == -2 ? (int64_t)k * cols : (int64_t)rows * k;
+  const int es = u_dtype == DION_BF16 ? 2 : 4;
   const bool vec4 = (cols % 4 == 0) && table_aligned(X_ptrs, n) && aligned16((uint64_t)U_sel) &&
                     aligned16((uint64_t)map);
   for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
@@ -620,11 +622,20 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
     fill_tab(x, X_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
     HIP_TRY(launch_dion2_post(x, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
-                              (const bf16_t*)U_sel + mat0 * sel_numel, k, map + mat0 * dim,
-                              row_scale ? row_scale + mat0 * k : nullptr, lr_dev, adj_ratio, wd_dev,
-                              wd_host, vec4, (hipStream_t)stream),
+                              (const char*)U_sel + mat0 * sel_numel * es, u_dtype == DION_BF16 ? 0 : 1, k,
+                              map + mat0 * dim, row_scale ? row_scale + mat0 * k : nullptr, lr_dev,
+                              adj_lr_dev, adj_ratio, wd_dev, wd_host, vec4, (hipStream_t)stream),
             "dion_dion2_post");
   }
+  return DION_OK;
+}
+
+extern "C" int dion_dion2_index_map(const int64_t* idx, int n_mat, int k, int dim, int32_t* map,
+                                    void* stream) {
+  if (n_mat < 0 || k < 0 || dim < 0 || k > dim) return fail(DION_E_INVALID, "dion_dion2_index_map: bad size");
+  if (n_mat == 0 || dim == 0) return DION_OK;
+  if (!map || (k > 0 && !idx)) return fail(DION_E_INVALID, "dion_dion2_index_map: null argument");
+  HIP_TRY(launch_dion2_index_map(idx, n_mat, k, dim, map, (hipStream_t)stream), "dion_dion2_index_map");
   return DION_OK;
 }
 
@@ -691,8 +702,8 @@ extern "C" int dion_mask_index(const float* norms, int n_mat, int dim, int32_t* 
 extern "C" int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int n,
                                       int mats_per_ptr, int rows, int cols, int select_dim,
                                       const void* U, const float* norms, const float* row_scale,
-                                      const float* lr_dev, float adj_ratio, const float* wd_dev,
-                                      float wd_host, float ef_decay, void* stream) {
+                                      const float* lr_dev, const float* adj_lr_dev, float adj_ratio,
+                                      const float* wd_dev, float wd_host, float ef_decay, void* stream) {
   if (int rc = check_select_dim("dion_dion2_post_masked", select_dim)) return rc;
   if (row_scale && select_dim != -2)
     return fail(DION_E_INVALID, "dion_dion2_post_masked: row_scale needs select_dim == -2");
@@ -715,8 +726,8 @@ extern "C" int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
     HIP_TRY(launch_dion2_post_masked(x, m, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
                                      (const bf16_t*)U + mat0 * rows * cols, norms + mat0 * dim,
-                                     row_scale ? row_scale + mat0 * rows : nullptr, lr_dev, adj_ratio,
-                                     wd_dev, wd_host, ef_decay, vec4, (hipStream_t)stream),
+                                     row_scale ? row_scale + mat0 * rows : nullptr, lr_dev, adj_lr_dev,
+                                     adj_ratio, wd_dev, wd_host, ef_decay, vec4, (hipStream_t)stream),
             "dion_dion2_post_masked");
   }
   return DION_OK;

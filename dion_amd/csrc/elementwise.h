@@ -53,9 +53,12 @@ hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int
                                int select_rows, const int32_t* idx, int k, float ef_decay, bf16_t* U,
                                bool vec4, hipStream_t st);
 hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
-                             int select_rows, const bf16_t* U, int k, const int32_t* map,
-                             const float* row_scale, const float* lr_dev, float adj_ratio,
-                             const float* wd_dev, float wd_host, bool vec4, hipStream_t st);
+                             int select_rows, const void* U, int u_dtype, int k, const int32_t* map,
+                             const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
+                             float adj_ratio, const float* wd_dev, float wd_host, bool vec4,
+                             hipStream_t st);
+hipError_t launch_dion2_index_map(const int64_t* idx, int n_mat, int k, int dim, int32_t* map,
+                                  hipStream_t st);
 
 // Whole-matrix selection (select_scope.hip): slice L1 norms of a stacked tensor, dense gather /
 // zero-filled scatter of the selected slices, and the update keyed off the non-zero slices.
@@ -70,8 +73,8 @@ hipError_t launch_mask_index(const float* norms, int n_mat, int dim, int32_t* ga
 hipError_t launch_dion2_post_masked(const PtrTab& X, const PtrTab& M, int n_mat, int mats_per_ptr,
                                     int rows, int cols, int select_rows, const bf16_t* U,
                                     const float* norms, const float* row_scale, const float* lr_dev,
-                                    float adj_ratio, const float* wd_dev, float wd_host, float ef_decay,
-                                    bool vec4, hipStream_t st);
+                                    const float* adj_lr_dev, float adj_ratio, const float* wd_dev,
+                                    float wd_host, float ef_decay, bool vec4, hipStream_t st);
 
 // Multi-tensor AdamW / Lion (scalar_opts.hip): n <= kMtaTensors tensors per launch, host arrays of
 // device pointers and element counts.

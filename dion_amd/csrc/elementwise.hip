@@ -852,14 +852,29 @@ hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int
 }
 
 // x = a*x - b*u[map] on selected slices, x = a*x elsewhere; one rounding of the sum.
-// Block (row group of 8, mat); 4 columns per thread on the vector path.
-template <bool VEC>
+// Block (row group of 8, mat); 4 columns per thread on the vector path.  u is bf16 or fp32 (UT).
+template <typename UT>
+static __device__ __forceinline__ float u_load(const UT* u, int64_t i) {
+  return sizeof(UT) == 2 ? bf16_to_f32(((const bf16_t*)u)[i]) : ((const float*)u)[i];
+}
+template <typename UT>
+static __device__ __forceinline__ float4 u_load4(const UT* u, int64_t i) {
+  if (sizeof(UT) == 2) {
+    const uint2 raw = *(const uint2*)((const bf16_t*)u + i);
+    return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                       __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u));
+  }
+  return *(const float4*)((const float*)u + i);
+}
+
+template <bool VEC, typename UT>
 __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_ptr, int rows,
                                                          int cols, int select_rows,
-                                                         const bf16_t* __restrict__ U, int k,
+                                                         const UT* __restrict__ U, int k,
                                                          const int32_t* __restrict__ map,
                                                          const float* __restrict__ row_scale,
                                                          const float* __restrict__ lr_dev,
+                                                         const float* __restrict__ adj_lr_dev,
                                                          float adj_ratio,
                                                          const float* __restrict__ wd_dev,
                                                          float wd_host) {
@@ -868,30 +883,24 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
   const float lr = *lr_dev;
   const float wd = wd_dev ? *wd_dev : wd_host;
   const float a = __fsub_rn(1.0f, __fmul_rn(lr, wd));
-  const float b0 = __fmul_rn(lr, adj_ratio);
+  const float b0 = __fmul_rn(adj_lr_dev ? *adj_lr_dev : lr, adj_ratio);
   float b = b0;
   const int dim = select_rows ? rows : cols;
   const int32_t* mp = map + (int64_t)mat * dim;
-  const bf16_t* u = U + (int64_t)mat * (select_rows ? (int64_t)k * cols : (int64_t)rows * k);
+  const UT* u = U + (int64_t)mat * (select_rows ? (int64_t)k * cols : (int64_t)rows * k);
   const int r_end = (blockIdx.x * 8 + 8) < rows ? (blockIdx.x * 8 + 8) : rows;
   for (int r = blockIdx.x * 8; r < r_end; ++r) {
     float* xr = x + (int64_t)r * cols;
     if (select_rows) {
       const int j = mp[r];
-      const bf16_t* ur = u + (int64_t)(j < 0 ? 0 : j) * cols;
+      const UT* ur = u + (int64_t)(j < 0 ? 0 : j) * cols;
       // per-row scale of the selected slice (rows selected only): u is multiplied by it first
       if (row_scale && j >= 0) b = __fmul_rn(b0, row_scale[(int64_t)mat * k + j]);
       if (VEC) {
         for (int c = threadIdx.x * 4; c < cols; c += 1024) {
           float4 v = *(const float4*)(xr + c);
           float4 uv = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (j >= 0) {
-            const uint2 raw = *(const uint2*)(ur + c);
-            uv.x = __uint_as_float(raw.x << 16);
-            uv.y = __uint_as_float(raw.x & 0xffff0000u);
-            uv.z = __uint_as_float(raw.y << 16);
-            uv.w = __uint_as_float(raw.y & 0xffff0000u);
-          }
+          if (j >= 0) uv = u_load4<UT>(ur, c);
           v.x = fmaf(a, v.x, -(b * uv.x));
           v.y = fmaf(a, v.y, -(b * uv.y));
           v.z = fmaf(a, v.z, -(b * uv.z));
@@ -900,20 +909,20 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
         }
       } else {
         for (int c = threadIdx.x; c < cols; c += 256) {
-          const float uv = j >= 0 ? bf16_to_f32(ur[c]) : 0.f;
+          const float uv = j >= 0 ? u_load<UT>(ur, c) : 0.f;
           xr[c] = fmaf(a, xr[c], -(b * uv));
         }
       }
     } else {
-      const bf16_t* ur = u + (int64_t)r * k;
+      const UT* ur = u + (int64_t)r * k;
       if (VEC) {
         for (int c = threadIdx.x * 4; c < cols; c += 1024) {
           float4 v = *(const float4*)(xr + c);
           const int4 j4 = *(const int4*)(mp + c);
-          const float u0 = j4.x >= 0 ? bf16_to_f32(ur[j4.x]) : 0.f;
-          const float u1 = j4.y >= 0 ? bf16_to_f32(ur[j4.y]) : 0.f;
-          const float u2 = j4.z >= 0 ? bf16_to_f32(ur[j4.z]) : 0.f;
-          const float u3 = j4.w >= 0 ? bf16_to_f32(ur[j4.w]) : 0.f;
+          const float u0 = j4.x >= 0 ? u_load<UT>(ur, j4.x) : 0.f;
+          const float u1 = j4.y >= 0 ? u_load<UT>(ur, j4.y) : 0.f;
+          const float u2 = j4.z >= 0 ? u_load<UT>(ur, j4.z) : 0.f;
+          const float u3 = j4.w >= 0 ? u_load<UT>(ur, j4.w) : 0.f;
           v.x = fmaf(a, v.x, -(b * u0));
           v.y = fmaf(a, v.y, -(b * u1));
           v.z = fmaf(a, v.z, -(b * u2));
@@ -923,7 +932,7 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
       } else {
         for (int c = threadIdx.x; c < cols; c += 256) {
           const int j = mp[c];
-          const float uv = j >= 0 ? bf16_to_f32(ur[j]) : 0.f;
+          const float uv = j >= 0 ? u_load<UT>(ur, j) : 0.f;
           xr[c] = fmaf(a, xr[c], -(b * uv));
         }
       }
@@ -932,16 +941,42 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
 }
 
 hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
-                             int select_rows, const bf16_t* U, int k, const int32_t* map,
-                             const float* row_scale, const float* lr_dev, float adj_ratio,
-                             const float* wd_dev, float wd_host, bool vec4, hipStream_t st) {
+                             int select_rows, const void* U, int u_dtype, int k, const int32_t* map,
+                             const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
+                             float adj_ratio, const float* wd_dev, float wd_host, bool vec4,
+                             hipStream_t st) {
   dim3 grid((rows + 7) / 8, n_mat);
-  if (vec4)
-    hipLaunchKernelGGL(dion2_post_kernel<true>, grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols,
-                       select_rows, U, k, map, row_scale, lr_dev, adj_ratio, wd_dev, wd_host);
-  else
-    hipLaunchKernelGGL(dion2_post_kernel<false>, grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols,
-                       select_rows, U, k, map, row_scale, lr_dev, adj_ratio, wd_dev, wd_host);
+#define D2POST_LAUNCH(V, UT)                                                                        \
+  hipLaunchKernelGGL((dion2_post_kernel<V, UT>), grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols, \
+                     select_rows, (const UT*)U, k, map, row_scale, lr_dev, adj_lr_dev, adj_ratio,     \
+                     wd_dev, wd_host)
+  if (u_dtype == 0) {
+    if (vec4) D2POST_LAUNCH(true, bf16_t); else D2POST_LAUNCH(false, bf16_t);
+  } else {
+    if (vec4) D2POST_LAUNCH(true, float); else D2POST_LAUNCH(false, float);
+  }
+#undef D2POST_LAUNCH
+  return hipGetLastError();
+}
+
+// map[m][idx[m][j]] = j for the k (distinct, unordered) int64 indices of every matrix, -1 elsewhere.
+// One block per matrix: the fill and the scatter are separated by a block barrier.
+__global__ __launch_bounds__(256) void dion2_index_map_kernel(const int64_t* __restrict__ idx, int k,
+                                                              int dim, int32_t* __restrict__ map) {
+  const int mat = blockIdx.x;
+  int32_t* mp = map + (int64_t)mat * dim;
+  for (int i = threadIdx.x; i < dim; i += 256) mp[i] = -1;
+  __syncthreads();
+  const int64_t* id = idx + (int64_t)mat * k;
+  for (int j = threadIdx.x; j < k; j += 256) {
+    const int64_t i = id[j];
+    if (i >= 0 && i < dim) mp[i] = j;
+  }
+}
+
+hipError_t launch_dion2_index_map(const int64_t* idx, int n_mat, int k, int dim, int32_t* map,
+                                  hipStream_t st) {
+  hipLaunchKernelGGL(dion2_index_map_kernel, dim3(n_mat), dim3(256), 0, st, idx, k, dim, map);
   return hipGetLastError();
 }
 

@@ -253,6 +253,7 @@ __global__ __launch_bounds__(256) void dion2_post_masked_kernel(PtrTab X, PtrTab
                                                                 const float* __restrict__ norms,
                                                                 const float* __restrict__ row_scale,
                                                                 const float* __restrict__ lr_dev,
+                                                                const float* __restrict__ adj_lr_dev,
                                                                 float adj_ratio,
                                                                 const float* __restrict__ wd_dev,
                                                                 float wd_host, float ef_decay) {
@@ -264,7 +265,7 @@ __global__ __launch_bounds__(256) void dion2_post_masked_kernel(PtrTab X, PtrTab
   const float lr = *lr_dev;
   const float wd = wd_dev ? *wd_dev : wd_host;
   const float a = __fsub_rn(1.0f, __fmul_rn(lr, wd));
-  const float b0 = __fmul_rn(lr, adj_ratio);
+  const float b0 = __fmul_rn(adj_lr_dev ? *adj_lr_dev : lr, adj_ratio);
   const int dim = select_rows ? rows : cols;
   const float* nm = norms + (int64_t)mat * dim;
   const int r_end = (blockIdx.x * 8 + 8) < rows ? (blockIdx.x * 8 + 8) : rows;
@@ -332,17 +333,17 @@ __global__ __launch_bounds__(256) void dion2_post_masked_kernel(PtrTab X, PtrTab
 hipError_t launch_dion2_post_masked(const PtrTab& X, const PtrTab& M, int n_mat, int mats_per_ptr,
                                     int rows, int cols, int select_rows, const bf16_t* U,
                                     const float* norms, const float* row_scale, const float* lr_dev,
-                                    float adj_ratio, const float* wd_dev, float wd_host, float ef_decay,
-                                    bool vec4, hipStream_t st) {
+                                    const float* adj_lr_dev, float adj_ratio, const float* wd_dev,
+                                    float wd_host, float ef_decay, bool vec4, hipStream_t st) {
   dim3 grid((rows + 7) / 8, n_mat);
   if (vec4)
     hipLaunchKernelGGL(dion2_post_masked_kernel<true>, grid, dim3(256), 0, st, X, M, mats_per_ptr, rows,
-                       cols, select_rows, U, norms, row_scale, lr_dev, adj_ratio, wd_dev, wd_host,
-                       ef_decay);
+                       cols, select_rows, U, norms, row_scale, lr_dev, adj_lr_dev, adj_ratio, wd_dev,
+                       wd_host, ef_decay);
   else
     hipLaunchKernelGGL(dion2_post_masked_kernel<false>, grid, dim3(256), 0, st, X, M, mats_per_ptr, rows,
-                       cols, select_rows, U, norms, row_scale, lr_dev, adj_ratio, wd_dev, wd_host,
-                       ef_decay);
+                       cols, select_rows, U, norms, row_scale, lr_dev, adj_lr_dev, adj_ratio, wd_dev,
+                       wd_host, ef_decay);
   return hipGetLastError();
 }
 

@@ -71,19 +71,22 @@ def _arena(U, n: int) -> Tensor:
 
 
 def dion2_post_orthogonalize_masked(X: List[Tensor], M: List[Tensor], U, base_lr: Tensor, adj_ratio: float,
-                                    weight_decay, ef_decay: float, select_dim: int) -> None:
+                                    weight_decay, ef_decay: float, select_dim: int,
+                                    adjusted_lr: Optional[Tensor] = None) -> None:
     """``X[i] <- (1 - lr*wd) X[i] - lr*adj_ratio*U[i]``; the slices of ``M[i]`` at which ``U[i]`` is not all
     zero decay by ``ef_decay``.  ``U``: bf16 arena ``[N, *shape]`` (or a list of N tensors), zero off the
     selected slices.  ``base_lr`` is the 0-d device tensor of the group, the adjusted rate is
-    ``base_lr * adj_ratio`` (dion/dion2.py:623-659)."""
+    ``base_lr * adj_ratio``, or ``adjusted_lr * adj_ratio`` when that 0-d device tensor is given
+    (dion/dion2.py:623-659)."""
     U = _arena(U, len(X))
     norms = ops.slice_l1(U, select_dim)
-    ops.dion2_post_masked(X, M, U, norms, base_lr, adj_ratio, weight_decay, ef_decay, select_dim)
+    ops.dion2_post_masked(X, M, U, norms, base_lr, adj_ratio, weight_decay, ef_decay, select_dim,
+                          adjusted_lr=adjusted_lr)
 
 
 def nordion2_post_orthogonalize_masked(X: List[Tensor], M: List[Tensor], V: List[Tensor], U, base_lr: Tensor,
                                        adj_ratio: float, weight_decay, ef_decay: float, muon_beta2: float,
-                                       select_dim: int = -2) -> None:
+                                       select_dim: int = -2, adjusted_lr: Optional[Tensor] = None) -> None:
     """As ``dion2_post_orthogonalize_masked`` with NorMuon's per-row normalisation in between: the second
     moments ``V[i] [..., rows, 1]`` are updated on the selected (non-zero) rows only and the Frobenius
     norm of the update is kept (dion/nordion2.py:448-500).  Rows only."""
@@ -93,4 +96,5 @@ def nordion2_post_orthogonalize_masked(X: List[Tensor], M: List[Tensor], V: List
     norms = ops.slice_l1(U, -2)
     gate = ops.mask_index(norms)
     row_scale = ops.normuon_stats_selected(U, V, gate, muon_beta2)
-    ops.dion2_post_masked(X, M, U, norms, base_lr, adj_ratio, weight_decay, ef_decay, -2, row_scale=row_scale)
+    ops.dion2_post_masked(X, M, U, norms, base_lr, adj_ratio, weight_decay, ef_decay, -2, row_scale=row_scale,
+                          adjusted_lr=adjusted_lr)

@@ -338,10 +338,11 @@ def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_d
 
 
 def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: float, weight_decay,
-               select_dim: int, row_scale: Optional[Tensor] = None) -> None:
+               select_dim: int, row_scale: Optional[Tensor] = None, adjusted_lr: Optional[Tensor] = None) -> None:
     """Fused ``x = (1 - lr*wd)*x - lr*adj_ratio*u[map]`` over every ``X[i]``.  Mirrors
-    ``dion2_post_orthogonalize_triton`` (dion/dion2_triton.py:147-242).  ``row_scale [n_mat, k]``
-    (rows selected only) multiplies each selected row of ``U`` first."""
+    ``dion2_post_orthogonalize_triton`` (dion/dion2_triton.py:147-242).  ``U`` bf16 or fp32 arena.
+    ``row_scale [n_mat, k]`` (rows selected only) multiplies each selected row of ``U`` first;
+    ``adjusted_lr`` (0-d fp32 device tensor) replaces ``lr`` in the update term."""
     if select_dim not in (-2, -1):
         raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
     n = len(X)
@@ -351,7 +352,9 @@ def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: 
     numel = X[0].numel()
     mats_per_ptr = numel // (rows * cols)
     xp = _list_ptrs(X, "X", torch.float32, numel)
-    _check_bf16(U, "U")
+    _require_gpu(U, "U")
+    if not U.is_contiguous():
+        raise ValueError("U must be contiguous")
     k = U.shape[-2] if select_dim == -2 else U.shape[-1]
     lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, U.device)
     lib = _lib.load()
@@ -361,8 +364,52 @@ def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: 
                 row_scale.numel() != n * mats_per_ptr * k:
             raise ValueError("row_scale must be a contiguous float32 tensor of n_mat * k entries")
         rs = row_scale.data_ptr()
-    check(lib.dion_dion2_post(xp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(), k, imap.data_ptr(),
-                              rs, lr_p, float(adj_ratio), wd_p, wd_h, _stream_handle(U.device)), "dion2_post")
+    alr = None
+    if adjusted_lr is not None:
+        if not (adjusted_lr.is_cuda and adjusted_lr.dtype == torch.float32 and adjusted_lr.numel() == 1):
+            raise TypeError("adjusted_lr must be a 0-d float32 GPU tensor")
+        alr = adjusted_lr.data_ptr()
+    check(lib.dion_dion2_post(xp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(), _dtype_code(U, "U"), k,
+                              imap.data_ptr(), rs, lr_p, alr, float(adj_ratio), wd_p, wd_h,
+                              _stream_handle(U.device)), "dion2_post")
+
+
+def dion2_index_map(indices: Tensor, dim: int) -> Tensor:
+    """int32 ``[n_mat, dim]`` inverse map of ``indices [..., k]`` (int64, distinct, any order): position of
+    each slice in the list, -1 where not listed.  Mirrors ``_build_index_map``
+    (dion/dion2_triton.py:30-47)."""
+    _require_gpu(indices, "indices")
+    if indices.dtype != torch.int64:
+        raise TypeError(f"indices must be int64, got {indices.dtype}")
+    k = indices.shape[-1]
+    idx = indices.reshape(-1, k).contiguous()
+    imap = torch.empty(idx.shape[0], dim, dtype=torch.int32, device=indices.device)
+    lib = _lib.load()
+    check(lib.dion_dion2_index_map(idx.data_ptr(), idx.shape[0], k, dim, imap.data_ptr(),
+                                   _stream_handle(indices.device)), "dion2_index_map")
+    return imap
+
+
+def dion2_post_orthogonalize_triton(X: List[Tensor], U: List[Tensor], indices: List[Tensor], base_lr: Tensor,
+                                    adjusted_lr: Tensor, weight_decay, select_dim: int) -> None:
+    """Same call as the reference's ``dion2_post_orthogonalize_triton`` (dion/dion2_triton.py:147-155):
+    per tensor ``x`` ``[*leading, M, N]`` fp32 contiguous, ``u`` the selected slices (bf16 or fp32),
+    ``indices [*leading, k]`` int64; ``selected: x = (1 - base_lr*wd)*x - adjusted_lr*u``, unselected:
+    ``x = (1 - base_lr*wd)*x``.  ``base_lr`` / ``adjusted_lr`` are 0-d fp32 device tensors read in the
+    kernel.  Empty tensors are skipped; non-contiguous ``x`` raises ``ValueError``."""
+    if select_dim not in (-2, -1):
+        raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
+    for x, u, idx in zip(X, U, indices):
+        if x.numel() == 0:
+            continue
+        if not x.is_contiguous():
+            raise ValueError("dion2_post_orthogonalize_triton requires contiguous X tensors")
+        if u.dtype not in (torch.bfloat16, torch.float32):
+            u = u.float()
+        dim = x.shape[select_dim]
+        imap = dion2_index_map(idx, dim)
+        dion2_post([x], u.contiguous().unsqueeze(0), imap, base_lr, 1.0, weight_decay, select_dim,
+                   adjusted_lr=adjusted_lr)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -455,11 +502,12 @@ def mask_index(norms: Tensor) -> Tensor:
 
 def dion2_post_masked(X: List[Tensor], M: List[Tensor], U: Tensor, norms: Tensor, lr: Tensor,
                       adj_ratio: float, weight_decay, ef_decay: float, select_dim: int,
-                      row_scale: Optional[Tensor] = None) -> None:
+                      row_scale: Optional[Tensor] = None, adjusted_lr: Optional[Tensor] = None) -> None:
     """``x = (1 - lr*wd)*x - lr*adj_ratio*u`` over every ``X[i]`` and ``m *= ef_decay`` on the slices of
     ``M[i]`` whose entry of ``norms`` (``slice_l1(U)``) is > 0.  ``U [N, ..., rows, cols]`` bf16 is zero
     off the selected slices.  Mirrors ``dion2_post_orthogonalize_masked`` (dion/dion2.py:623-659);
-    ``row_scale [n_mat, rows]`` (rows selected only) multiplies each row of ``U`` first."""
+    ``row_scale [n_mat, rows]`` (rows selected only) multiplies each row of ``U`` first; ``adjusted_lr``
+    (0-d fp32 device tensor) replaces ``lr`` in the update term."""
     if select_dim not in (-2, -1):
         raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
     n = len(X)
@@ -484,9 +532,14 @@ def dion2_post_masked(X: List[Tensor], M: List[Tensor], U: Tensor, norms: Tensor
             raise ValueError("row_scale must be a contiguous float32 tensor of n_mat * rows entries")
         rs = row_scale.data_ptr()
     lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, U.device)
+    alr = None
+    if adjusted_lr is not None:
+        if not (adjusted_lr.is_cuda and adjusted_lr.dtype == torch.float32 and adjusted_lr.numel() == 1):
+            raise TypeError("adjusted_lr must be a 0-d float32 GPU tensor")
+        alr = adjusted_lr.data_ptr()
     lib = _lib.load()
     check(lib.dion_dion2_post_masked(xp, mp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(),
-                                     norms.data_ptr(), rs, lr_p, float(adj_ratio), wd_p, wd_h,
+                                     norms.data_ptr(), rs, lr_p, alr, float(adj_ratio), wd_p, wd_h,
                                      float(ef_decay), _stream_handle(U.device)), "dion2_post_masked")
 
 

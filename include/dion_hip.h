@@ -162,15 +162,23 @@ int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr, int rows,
                       void* stream);
 
 /* Dion2 fused weight decay + selective update, single rounding:
- *   x = (1 - lr wd) x - lr adj_ratio u[map]   on selected slices,  x = (1 - lr wd) x elsewhere
+ *   x = (1 - lr wd) x - b u[map]   on selected slices,  x = (1 - lr wd) x elsewhere
+ *   b = lr * adj_ratio, or (*adj_lr_dev) * adj_ratio when adj_lr_dev (nullable, device fp32 scalar:
+ *   the reference's `adjusted_lr` tensor) is given
+ * U_sel [n_mat, k, cols] / [n_mat, rows, k] in u_dtype (DION_BF16 or DION_F32).
  * row_scale (nullable, select_dim -2 only): device [n_mat, k] fp32; selected row j of U_sel is
  * multiplied by row_scale[i][j] first (NorDion2's normalised update).
  * Replaces dion2_post_orthogonalize_triton (dion/dion2_triton.py:147-242, kernel :57-144),
  * dion2_post_orthogonalize (dion/dion2.py:666-697) and its use at dion/nordion2.py:403-425. */
 int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, int cols,
-                    int select_dim, const void* U_sel, int k, const int32_t* map,
-                    const float* row_scale, const float* lr_dev, float adj_ratio, const float* wd_dev,
-                    float wd_host, void* stream);
+                    int select_dim, const void* U_sel, int u_dtype, int k, const int32_t* map,
+                    const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
+                    float adj_ratio, const float* wd_dev, float wd_host, void* stream);
+
+/* Dense inverse map of k distinct (unordered) int64 slice indices per matrix: map[i][idx[i][j]] = j,
+ * -1 elsewhere.  idx [n_mat, k] int64, map out [n_mat, dim] int32.
+ * Replaces _build_index_map (dion/dion2_triton.py:30-47). */
+int dion_dion2_index_map(const int64_t* idx, int n_mat, int k, int dim, int32_t* map, void* stream);
 
 /* --------------------------------------------------------------------------------------------
  * Whole-matrix selection: what a rank runs on assembled matrices when the top-k is taken inside
@@ -204,16 +212,17 @@ int dion_scatter_slices(const void* sub, int dtype, int n_mat, int rows, int col
 int dion_mask_index(const float* norms, int n_mat, int dim, int32_t* gate, void* stream);
 
 /* Masked Dion2 / NorDion2 update, single rounding of the sum:
- *   x = (1 - lr wd) x - lr adj_ratio u   everywhere (u [n_mat, rows, cols] bf16, zero off the
- *   selected slices);   m *= ef_decay   on slices with norms[i][s] > 0
+ *   x = (1 - lr wd) x - b u   everywhere (u [n_mat, rows, cols] bf16, zero off the selected
+ *   slices; b as in dion_dion2_post);   m *= ef_decay   on slices with norms[i][s] > 0
  * norms as written by dion_slice_l1 on U.  row_scale (nullable, select_dim -2 only): device
  * [n_mat, rows] fp32, row r of u is multiplied by row_scale[i][r] first.
  * Replaces dion2_post_orthogonalize_masked (dion/dion2.py:623-659) and, with row_scale, the update
  * half of nordion2_post_orthogonalize_masked (dion/nordion2.py:448-500). */
 int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int n, int mats_per_ptr,
                            int rows, int cols, int select_dim, const void* U, const float* norms,
-                           const float* row_scale, const float* lr_dev, float adj_ratio,
-                           const float* wd_dev, float wd_host, float ef_decay, void* stream);
+                           const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
+                           float adj_ratio, const float* wd_dev, float wd_host, float ef_decay,
+                           void* stream);
 
 /* --------------------------------------------------------------------------------------------
  * Multi-tensor AdamW / Lion for the non-matrix parameter groups (algorithm "adamw" / "lion").
