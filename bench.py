@@ -101,6 +101,9 @@ def main() -> int:
     ap.add_argument("--workload", default="llama3_8b", choices=sorted(WORKLOADS))
     ap.add_argument("--ns", default="ns5", choices=["ns5", "polar_express", "gram"])
     ap.add_argument("--optimizer", default="muon", choices=["muon", "normuon", "dion2", "nordion2"])
+    ap.add_argument("--selection-scope", default="local", choices=["local", "global"],
+                    help="dion2 / nordion2: 'global' runs the whole-matrix sequence (accumulate, select inside the "
+                         "orthogonalization call, masked update) that a rank runs on assembled matrices")
     ap.add_argument("--graph", action="store_true",
                     help="capture the step into a hipGraph during warm-up and time replays (needs --warmup >= 2)")
     ap.add_argument("--breakdown", action="store_true",
@@ -162,10 +165,15 @@ def main() -> int:
                       adjust_lr="spectral_norm", **ns_kw)
     elif args.optimizer == "nordion2":
         opt = NorDion2(groups, lr=0.02, fraction=fraction, mu=0.95, muon_beta2=0.95, weight_decay=0.01,
-                       adjust_lr="spectral_norm", **ns_kw)
+                       adjust_lr="spectral_norm", selection_scope=args.selection_scope, **ns_kw)
     else:
         opt = Dion2(groups, lr=0.02, fraction=fraction, ef_decay=0.95, weight_decay=0.01,
-                    adjust_lr="spectral_norm", **ns_kw)
+                    adjust_lr="spectral_norm", selection_scope=args.selection_scope, **ns_kw)
+    if args.selection_scope == "global":
+        if args.optimizer not in ("dion2", "nordion2"):
+            print("bench.py: --selection-scope applies to dion2 / nordion2", file=sys.stderr)
+            return 2
+        opt.assembled_selection = True
 
     if args.graph:
         if args.warmup < 2:
@@ -202,6 +210,7 @@ def main() -> int:
                         + ("hipGraph replay, " if args.graph else "") + f"{args.ns}, wd 0.01, lr 0.02"
                         + ({"dion2": ", fraction 0.25, ef_decay 0.95", "nordion2": ", fraction 0.25, mu 0.95"}
                            .get(args.optimizer, ", nesterov mu=0.95"))
+                        + (", whole-matrix selection" if args.selection_scope == "global" else "")
                         + (", muon_beta2 0.95" if args.optimizer in ("normuon", "nordion2") else "") + ") over "
                         + ", ".join(f"{c}x({r}x{k})" for _n, r, k, c in spec),
             "matrices": sum(c for *_x, c in spec),

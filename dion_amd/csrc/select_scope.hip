@@ -50,12 +50,12 @@ __global__ __launch_bounds__(256) void slice_l1_rows_kernel(const T* __restrict_
   if (lane == 0) norms[(int64_t)mat * rows + row] = round_bf16 ? through_bf16(s) : s;
 }
 
-// Columns: a block owns 64*W columns (W consecutive ones per thread) and walks all rows, four row
-// lanes at a time.
-template <typename T, int W>
-__global__ __launch_bounds__(256) void slice_l1_cols_kernel(const T* __restrict__ U, int rows, int cols,
-                                                            int round_bf16, float* __restrict__ norms) {
-  __shared__ float red[4][64 * W];
+// Columns: a block owns 64*W columns (W consecutive ones per thread) and walks all rows, RL row
+// lanes (wavefronts) at a time; the lanes' partial sums are added in lane order.
+template <typename T, int W, int RL>
+__global__ __launch_bounds__(64 * RL) void slice_l1_cols_kernel(const T* __restrict__ U, int rows, int cols,
+                                                                int round_bf16, float* __restrict__ norms) {
+  __shared__ float red[RL][64 * W];
   const int mat = blockIdx.y;
   const int t = threadIdx.x & 63, ry = threadIdx.x >> 6;
   const int c = (blockIdx.x * 64 + t) * W;
@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void slice_l1_cols_kernel(const T* __restrict_
   for (int e = 0; e < W; ++e) s[e] = 0.f;
   if (c < cols) {
 #pragma unroll 4
-    for (int r = ry; r < rows; r += 4) {
+    for (int r = ry; r < rows; r += RL) {
       const int64_t i = (int64_t)r * cols + c;
       if (W == 4 && sizeof(T) == 2) {
         const uint2 raw = *(const uint2*)((const bf16_t*)u + i);
@@ -92,9 +92,30 @@ __global__ __launch_bounds__(256) void slice_l1_cols_kernel(const T* __restrict_
 #pragma unroll
     for (int e = 0; e < W; ++e) {
       const int q = t * W + e;
-      const float v = (red[0][q] + red[1][q]) + (red[2][q] + red[3][q]);
+      float v = red[0][q];
+#pragma unroll
+      for (int l = 1; l < RL; ++l) v += red[l][q];
       norms[(int64_t)mat * cols + c + e] = round_bf16 ? through_bf16(v) : v;
     }
+  }
+}
+
+template <typename T>
+static void launch_slice_l1_cols(const T* U, int n_mat, int rows, int cols, int round_bf16, float* norms,
+                                 bool vec, hipStream_t st) {
+  if (vec) {
+    dim3 grid((cols / 4 + 63) / 64, n_mat);
+    // few column blocks and many rows: 16 wavefronts per block keep enough loads in flight
+    if ((int64_t)grid.x * grid.y < 1024 && rows >= 256)
+      hipLaunchKernelGGL((slice_l1_cols_kernel<T, 4, 16>), grid, dim3(1024), 0, st, U, rows, cols,
+                         round_bf16, norms);
+    else
+      hipLaunchKernelGGL((slice_l1_cols_kernel<T, 4, 4>), grid, dim3(256), 0, st, U, rows, cols, round_bf16,
+                         norms);
+  } else {
+    dim3 grid((cols + 63) / 64, n_mat);
+    hipLaunchKernelGGL((slice_l1_cols_kernel<T, 1, 4>), grid, dim3(256), 0, st, U, rows, cols, round_bf16,
+                       norms);
   }
 }
 
@@ -111,23 +132,10 @@ hipError_t launch_slice_l1(const void* U, int dtype, int n_mat, int rows, int co
   } else {
     const int es = dtype == 0 ? 2 : 4;
     const bool vec = (cols % 4) == 0 && (((uintptr_t)U) % (4 * es)) == 0;
-    if (vec) {
-      dim3 grid((cols / 4 + 63) / 64, n_mat);
-      if (dtype == 0)
-        hipLaunchKernelGGL((slice_l1_cols_kernel<bf16_t, 4>), grid, dim3(256), 0, st, (const bf16_t*)U,
-                           rows, cols, round_bf16, norms);
-      else
-        hipLaunchKernelGGL((slice_l1_cols_kernel<float, 4>), grid, dim3(256), 0, st, (const float*)U,
-                           rows, cols, round_bf16, norms);
-    } else {
-      dim3 grid((cols + 63) / 64, n_mat);
-      if (dtype == 0)
-        hipLaunchKernelGGL((slice_l1_cols_kernel<bf16_t, 1>), grid, dim3(256), 0, st, (const bf16_t*)U,
-                           rows, cols, round_bf16, norms);
-      else
-        hipLaunchKernelGGL((slice_l1_cols_kernel<float, 1>), grid, dim3(256), 0, st, (const float*)U,
-                           rows, cols, round_bf16, norms);
-    }
+    if (dtype == 0)
+      launch_slice_l1_cols<bf16_t>((const bf16_t*)U, n_mat, rows, cols, round_bf16, norms, vec, st);
+    else
+      launch_slice_l1_cols<float>((const float*)U, n_mat, rows, cols, round_bf16, norms, vec, st);
   }
   return hipGetLastError();
 }
@@ -137,7 +145,7 @@ hipError_t launch_slice_l1(const void* U, int dtype, int n_mat, int rows, int co
 // tensor that is zero elsewhere.  Pure data movement on 2- or 4-byte elements (E).
 // ------------------------------------------------------------------------------------------
 // Rows: block (j, mat) copies row idx[j] of the source to row j of the block.
-// Columns: block (row, mat) gathers the k selected columns of that row.
+// Columns: block (row group of 8, mat) gathers the k selected columns of each of its rows.
 template <typename E>
 __global__ __launch_bounds__(256) void gather_slices_kernel(const E* __restrict__ U, int rows, int cols,
                                                             int select_rows,
@@ -157,24 +165,27 @@ __global__ __launch_bounds__(256) void gather_slices_kernel(const E* __restrict_
       for (int c = threadIdx.x; c < cols; c += 256) dst[c] = src[c];
     }
   } else {
-    const int r = blockIdx.x;
-    const E* src = u + (int64_t)r * cols;
-    E* dst = sub + ((int64_t)mat * rows + r) * k;
-    for (int j = threadIdx.x; j < k; j += 256) dst[j] = src[id[j]];
+    const int r_end = (blockIdx.x * 8 + 8) < rows ? (blockIdx.x * 8 + 8) : rows;
+    for (int r = blockIdx.x * 8; r < r_end; ++r) {
+      const E* src = u + (int64_t)r * cols;
+      E* dst = sub + ((int64_t)mat * rows + r) * k;
+      for (int j = threadIdx.x; j < k; j += 256) dst[j] = src[id[j]];
+    }
   }
 }
 
-// Block (row, mat) writes one full row of the output: the block's row map[row] (rows selected) or
-// the block's entries map[c] (columns selected) where the map is >= 0, zero elsewhere.
+// Rows selected: block (row, mat) writes one full row of the output, the block's row map[row] or zeros.
+// Columns selected: block (row group of 8, mat); per row, entry c is the block's entry map[c] where the
+// map is >= 0, zero elsewhere.
 template <typename E>
 __global__ __launch_bounds__(256) void scatter_slices_kernel(const E* __restrict__ sub, int rows, int cols,
                                                              int select_rows,
                                                              const int32_t* __restrict__ map, int k,
                                                              E* __restrict__ out, int vec16) {
   const int mat = blockIdx.y;
-  const int r = blockIdx.x;
-  E* dst = out + ((int64_t)mat * rows + r) * cols;
   if (select_rows) {
+    const int r = blockIdx.x;
+    E* dst = out + ((int64_t)mat * rows + r) * cols;
     const int j = map[(int64_t)mat * rows + r];
     const E* src = sub + ((int64_t)mat * k + (j < 0 ? 0 : j)) * cols;
     if (vec16) {
@@ -184,12 +195,48 @@ __global__ __launch_bounds__(256) void scatter_slices_kernel(const E* __restrict
     } else {
       for (int c = threadIdx.x; c < cols; c += 256) dst[c] = j >= 0 ? src[c] : (E)0;
     }
+    return;
+  }
+  const int32_t* mp = map + (int64_t)mat * cols;
+  const int r_end = (blockIdx.x * 8 + 8) < rows ? (blockIdx.x * 8 + 8) : rows;
+  if (vec16) {
+    // V columns per thread: V map entries in (kept across the block's rows), one 16-byte store out
+    constexpr int V = 16 / (int)sizeof(E);
+    for (int c = threadIdx.x * V; c < cols; c += 256 * V) {
+      int j[V];
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        const int4 m4 = *(const int4*)(mp + c + 4 * q);
+        j[4 * q] = m4.x;
+        j[4 * q + 1] = m4.y;
+        j[4 * q + 2] = m4.z;
+        j[4 * q + 3] = m4.w;
+      }
+      for (int r = blockIdx.x * 8; r < r_end; ++r) {
+        const E* src = sub + ((int64_t)mat * rows + r) * k;
+        uint32_t w[4];
+        if (sizeof(E) == 2) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint32_t lo = j[2 * q] >= 0 ? (uint32_t)src[j[2 * q]] : 0u;
+            const uint32_t hi = j[2 * q + 1] >= 0 ? (uint32_t)src[j[2 * q + 1]] : 0u;
+            w[q] = lo | (hi << 16);
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) w[q] = j[q] >= 0 ? (uint32_t)src[j[q]] : 0u;
+        }
+        *(uint4*)(out + ((int64_t)mat * rows + r) * cols + c) = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    }
   } else {
-    const int32_t* mp = map + (int64_t)mat * cols;
-    const E* src = sub + ((int64_t)mat * rows + r) * k;
-    for (int c = threadIdx.x; c < cols; c += 256) {
-      const int j = mp[c];
-      dst[c] = j >= 0 ? src[j] : (E)0;
+    for (int r = blockIdx.x * 8; r < r_end; ++r) {
+      const E* src = sub + ((int64_t)mat * rows + r) * k;
+      E* dst = out + ((int64_t)mat * rows + r) * cols;
+      for (int c = threadIdx.x; c < cols; c += 256) {
+        const int j = mp[c];
+        dst[c] = j >= 0 ? src[j] : (E)0;
+      }
     }
   }
 }
@@ -202,7 +249,7 @@ hipError_t launch_gather_slices(const void* U, int dtype, int n_mat, int rows, i
                                 const int32_t* idx, int k, void* sub, hipStream_t st) {
   const int es = dtype == 0 ? 2 : 4;
   const int vec16 = select_rows && rows_vec16(U, sub, cols, es);
-  dim3 grid(select_rows ? k : rows, n_mat);
+  dim3 grid(select_rows ? k : (rows + 7) / 8, n_mat);
   if (es == 2)
     hipLaunchKernelGGL(gather_slices_kernel<uint16_t>, grid, dim3(256), 0, st, (const uint16_t*)U, rows,
                        cols, select_rows, idx, k, (uint16_t*)sub, vec16);
@@ -215,8 +262,11 @@ hipError_t launch_gather_slices(const void* U, int dtype, int n_mat, int rows, i
 hipError_t launch_scatter_slices(const void* sub, int dtype, int n_mat, int rows, int cols,
                                  int select_rows, const int32_t* map, int k, void* out, hipStream_t st) {
   const int es = dtype == 0 ? 2 : 4;
-  const int vec16 = select_rows && rows_vec16(sub, out, cols, es);
-  dim3 grid(rows, n_mat);
+  // rows: both sides move whole 16-byte chunks; columns: the output row and the map do
+  const int vec16 = select_rows ? rows_vec16(sub, out, cols, es)
+                                : (rows_vec16(out, out, cols, es) && (cols % 8) == 0 &&
+                                   (((uintptr_t)map) & 15) == 0);
+  dim3 grid(select_rows ? rows : (rows + 7) / 8, n_mat);
   if (es == 2)
     hipLaunchKernelGGL(scatter_slices_kernel<uint16_t>, grid, dim3(256), 0, st, (const uint16_t*)sub,
                        rows, cols, select_rows, map, k, (uint16_t*)out, vec16);
