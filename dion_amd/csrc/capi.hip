@@ -210,6 +210,11 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
             "small-matrix Newton-Schulz");
     return DION_OK;
   }
+  if (batch > 65535)
+    return fail(DION_E_INVALID,
+                "dion_ns_orthogonalize: %d matrices in one call (at most 65535 outside the small-matrix "
+                "kernel): split the batch",
+                batch);
   const NsPlan pl = make_plan(batch, rows, cols, flags);
   if (!workspace || workspace_bytes < pl.total)
     return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize: workspace %zu < %zu bytes", workspace_bytes,

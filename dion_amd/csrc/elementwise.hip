@@ -184,10 +184,11 @@ __global__ __launch_bounds__(256) void ns_prepare_vec_kernel(const T* __restrict
 __global__ __launch_bounds__(256) void unpad_kernel(const bf16_t* __restrict__ src, int64_t src_stride,
                                                     int ld, bf16_t* __restrict__ dst, int R, int C) {
   const int b = blockIdx.z;
-  const int r = blockIdx.y;
-  const bf16_t* s = src + (int64_t)b * src_stride + (int64_t)r * ld;
-  bf16_t* d = dst + ((int64_t)b * R + r) * C;
-  for (int c = blockIdx.x * 256 + threadIdx.x; c < C; c += gridDim.x * 256) d[c] = s[c];
+  for (int r = blockIdx.y; r < R; r += gridDim.y) {
+    const bf16_t* s = src + (int64_t)b * src_stride + (int64_t)r * ld;
+    bf16_t* d = dst + ((int64_t)b * R + r) * C;
+    for (int c = blockIdx.x * 256 + threadIdx.x; c < C; c += gridDim.x * 256) d[c] = s[c];
+  }
 }
 
 hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t numel,
@@ -238,8 +239,8 @@ hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* d
                         int C, hipStream_t st) {
   int gx = (C + 255) / 256;
   if (gx > 64) gx = 64;
-  hipLaunchKernelGGL(unpad_kernel, dim3(gx, R, batch), dim3(256), 0, st, src, src_stride, ld, dst, R,
-                     C);
+  hipLaunchKernelGGL(unpad_kernel, dim3(gx, R < 65535 ? R : 65535, batch), dim3(256), 0, st, src,
+                     src_stride, ld, dst, R, C);
   return hipGetLastError();
 }
 

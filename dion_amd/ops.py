@@ -185,12 +185,15 @@ def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: f
     carr = (_lib.ctypes.c_float * max(1, len(flat)))(*flat)
     flags = (DION_NS_GRAM if gram else 0) | (DION_NS_CARRY_XT if carry_xt else 0)
     lib = _lib.load()
-    nbytes = lib.dion_ns_workspace_bytes(batch, rows, cols, flags)
-    ws = _workspace(G.device, nbytes)
-    check(lib.dion_ns_orthogonalize(G3.data_ptr(), _dtype_code(G3, "G"), out.data_ptr(), batch, rows, cols,
-                                    carr, n_iters, float(norm_scale), float(epsilon), flags,
-                                    int(gram_reset), ws.data_ptr(), ws.numel(), _stream_handle(G.device)),
-          "ns_orthogonalize")
+    chunk = 32768  # one library call takes at most 65535 matrices
+    for b0 in range(0, batch, chunk):
+        nb = min(chunk, batch - b0)
+        nbytes = lib.dion_ns_workspace_bytes(nb, rows, cols, flags)
+        ws = _workspace(G.device, nbytes)
+        check(lib.dion_ns_orthogonalize(G3[b0:].data_ptr(), _dtype_code(G3, "G"), out[b0:].data_ptr(), nb, rows,
+                                        cols, carr, n_iters, float(norm_scale), float(epsilon), flags,
+                                        int(gram_reset), ws.data_ptr(), ws.numel(), _stream_handle(G.device)),
+              "ns_orthogonalize")
     return out.reshape(shape)
 
 

@@ -305,3 +305,17 @@ def test_kj_newton_schulz_vs_oracle(shape):
     assert _np_rel(out_np, ref) <= 2e-2 + e_ref
     sv = np.linalg.svd(out.float().cpu().numpy().astype(np.float64), compute_uv=False)
     assert 0.6 < sv.min() and sv.max() < 1.2  # KJ band [0.68, 1.16] with bf16 slack
+
+
+def test_batches_beyond_one_library_call():
+    """More matrices than one library call takes: the host splits the batch, every matrix gets the
+    result it gets on its own (per-head regime, 40000 matrices of 8x16)."""
+    from dion_amd import zeropower_via_newtonschulz5
+
+    torch.manual_seed(21)
+    G = torch.randn(40000, 8, 16, device=DEV).to(torch.bfloat16)
+    out = zeropower_via_newtonschulz5(G)
+    assert out.shape == G.shape
+    for lo in (0, 32760, 39990):
+        assert torch.equal(out[lo:lo + 10], zeropower_via_newtonschulz5(G[lo:lo + 10].contiguous()))
+    assert bool(torch.isfinite(out.float()).all())
