@@ -33,6 +33,10 @@ WORKLOADS = {
     # 1.3B: 24 layers, d 2048, MLP 8192
     "gpt_1p3b": [("qkv", 6144, 2048, 24), ("out", 2048, 2048, 24), ("fc", 8192, 2048, 24),
                  ("proj", 2048, 8192, 24)],
+    # what one GPU of an 8-GPU node would run for llama3_8b: ceil(N/8) whole matrices of every shape
+    # group through orthogonalization, and the same element count through momentum / update
+    "llama3_8b_share8": [("q_o", 4096, 4096, 8), ("k_v", 1024, 4096, 8), ("gate_up", 14336, 4096, 8),
+                         ("down", 4096, 14336, 4)],
     # the headline shape group on its own
     "ns_4096x14336": [("down", 4096, 14336, 32)],
     # GPT-small with per-head Newton-Schulz on the fused qkv weight (36 heads of 64x768 per layer)
