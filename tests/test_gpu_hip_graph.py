@@ -23,13 +23,18 @@ def _build(cls_name, kwargs, seed):
     emb = [torch.nn.Parameter(torch.randn(64, 48, device=DEV))]
     groups = [dict(params=mats), dict(params=heads, num_heads=4),
               dict(params=vec, algorithm="adamw", lr=0.003), dict(params=emb, algorithm="lion", lr=0.001)]
+    assembled = kwargs.pop("_assembled", False)
     opt = getattr(dion, cls_name)(groups, lr=0.02, **kwargs)
+    if assembled:  # the whole-matrix selection sequence (accumulate, select inside, masked update)
+        opt.assembled_selection = True
     return mats + heads + vec + emb, opt
 
 
 CASES = [("Muon", dict(nesterov=True)), ("Muon", dict(use_polar_express=False, cautious_wd=True)),
          ("NorMuon", {}), ("Dion2", dict(fraction=0.25)), ("NorDion2", dict(fraction=0.5)),
-         ("Muon", dict(weight_decay=torch.tensor(0.02)))]
+         ("Muon", dict(weight_decay=torch.tensor(0.02))),
+         ("Dion2", dict(fraction=0.25, selection_scope="global", _assembled=True)),
+         ("NorDion2", dict(fraction=0.5, selection_scope="global", _assembled=True))]
 
 
 @pytest.mark.parametrize("cls_name,kwargs", CASES)
