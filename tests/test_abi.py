@@ -56,3 +56,39 @@ def test_cpu_tensors_are_rejected():
 
     with pytest.raises(RuntimeError, match="no CPU path"):
         polar_express(torch.randn(8, 8))
+
+
+def test_argument_validation_happens_before_any_device_work():
+    """Bad arguments are refused on the host with DION_E_INVALID (-1) and a message, without a GPU."""
+    import ctypes
+
+    from dion_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libdion_hip.so not built in this checkout")
+    lib = _lib.load()
+    f = ctypes.c_float
+
+    def refused(rc, needle):
+        assert rc == -1
+        assert needle in lib.dion_last_error().decode()
+
+    refused(lib.dion_slice_l1(None, 0, 1, 8, 8, 0, 0, None, None), "select_dim")
+    refused(lib.dion_slice_l1(None, 7, 1, 8, 8, -2, 0, None, None), "dtype")
+    refused(lib.dion_slice_l1(None, 0, 70000, 8, 8, -2, 0, None, None), "65535")
+    refused(lib.dion_gather_slices(None, 0, 1, 8, 8, -2, None, 9, None, None), "k outside")
+    refused(lib.dion_scatter_slices(None, 0, 1, 8, 8, -1, None, -1, None, None), "k outside")
+    refused(lib.dion_mask_index(None, -1, 4, None, None), "bad size")
+    refused(lib.dion_dion2_index_map(None, 1, 9, 8, None, None), "bad size")
+    refused(lib.dion_dion2_post(None, 1, 1, 8, 8, -2, None, 5, 2, None, None, None, None, f(1.0), None, f(0.0), None),
+            "u_dtype")
+    refused(lib.dion_dion2_post(None, 1, 1, 8, 8, 1, None, 0, 2, None, None, None, None, f(1.0), None, f(0.0), None),
+            "select_dim")
+    refused(lib.dion_dion2_post_masked(None, None, 1, 0, 8, 8, -2, None, None, None, None, None, f(1.0), None,
+                                       f(0.0), f(0.9), None), "bad size")
+    refused(lib.dion_ns_orthogonalize(None, 9, None, 1, 8, 8, None, 0, f(1.0), f(0.0), 0, 0, None, 0, None),
+            "in_dtype")
+    # empty problems are accepted and do nothing
+    assert lib.dion_slice_l1(None, 0, 0, 8, 8, -2, 0, None, None) == 0
+    assert lib.dion_gather_slices(None, 0, 1, 8, 8, -2, None, 0, None, None) == 0
+    assert lib.dion_dion2_index_map(None, 0, 0, 8, None, None) == 0
