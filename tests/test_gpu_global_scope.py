@@ -354,3 +354,48 @@ def test_dion2_assembled_step_vs_oracle():
         assert _rel(p.data, x) <= 1e-3
         x = p.data.cpu().clone()
         M = opt.state[p]["momentum"].cpu().clone()
+
+
+@pytest.mark.parametrize("shape,select_dim", [((24, 2048, 8192), -2), ((24, 8192, 2048), -1)])
+def test_full_size_selection_and_masked_update_properties(shape, select_dim):
+    """GPT-1.3B shape groups (fraction 0.25), checked through properties that do not need a CPU pass over
+    400 M elements: exactly k slices survive, they carry the input, everything else is exactly zero, no
+    selected slice has a smaller (bf16-rounded) norm than an unselected one; the masked update leaves
+    unselected entries at exactly a*x, decays exactly the selected slices of M and moves the selected
+    entries of X by -lr*adj*u to fp32 rounding."""
+    from dion_amd import ops
+    from dion_amd.global_scope import dion2_post_orthogonalize_masked
+
+    torch.manual_seed(20)
+    n, rows, cols = shape
+    dim = shape[select_dim]
+    k = math.ceil(0.25 * dim)
+    U = (torch.randn(shape, device=DEV) * 0.02).to(torch.bfloat16)
+    sub, idx, imap = ops.select_slices(U, k, select_dim)
+    out = ops.scatter_slices(sub, imap, U.shape, select_dim)
+    norm_dim = -1 if select_dim == -2 else -2
+    sel = out.float().abs().sum(dim=norm_dim) > 0            # [n, dim]
+    assert bool((sel.sum(dim=-1) == k).all())
+    assert torch.equal(sel, imap >= 0)
+    mask = sel.unsqueeze(norm_dim)                           # broadcast over the slices
+    assert torch.equal(out, torch.where(mask, U, torch.zeros_like(U)))
+    norms = U.float().abs().sum(dim=norm_dim).to(torch.bfloat16).float()
+    lo_sel = torch.where(sel, norms, torch.full_like(norms, float("inf"))).min(dim=-1).values
+    hi_uns = torch.where(sel, torch.full_like(norms, -1.0), norms).max(dim=-1).values
+    assert bool((lo_sel >= hi_uns * (1 - 2.0 ** -7)).all())
+    del sub, norms
+
+    X = [torch.randn(rows, cols, device=DEV) * 0.02 for _ in range(n)]
+    M = [torch.randn(rows, cols, device=DEV) * 0.01 for _ in range(n)]
+    x0 = torch.stack(X)
+    m0 = torch.stack(M)
+    lr = torch.tensor(0.02, device=DEV)
+    dion2_post_orthogonalize_masked(X, M, out, lr, 1.5, 0.1, 0.9, select_dim)
+    x1 = torch.stack(X)
+    m1 = torch.stack(M)
+    a = 1 - lr * torch.tensor(0.1, device=DEV)
+    assert torch.equal(torch.where(mask, x0 * a, x1), x0 * a)              # unselected: exactly a*x
+    assert torch.equal(m1, torch.where(mask, m0 * torch.tensor(0.9, device=DEV), m0))
+    ref = x0.double() * a.double() - (lr.double() * 1.5) * out.double()
+    err = (x1.double() - ref).abs().max()
+    assert float(err) <= 1e-8
