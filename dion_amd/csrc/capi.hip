@@ -573,8 +573,6 @@ extern "C" int dion_dion2_topk(const float* norms, int n_mat, int dim, int k, in
                                int32_t* map, void* stream) {
   if (n_mat < 0 || dim < 0 || k < 0 || k > dim) return fail(DION_E_INVALID, "dion_dion2_topk: bad size");
   if (n_mat == 0 || dim == 0) return DION_OK;
-  if ((size_t)dim * 4 + 128 > 160 * 1024 - 256)
-    return fail(DION_E_INVALID, "dion_dion2_topk: dim %d exceeds the LDS-resident limit", dim);
   if (!norms || !idx || !map) return fail(DION_E_INVALID, "dion_dion2_topk: null argument");
   HIP_TRY(launch_dion2_topk(norms, n_mat, dim, k, idx, map, (hipStream_t)stream), "dion_dion2_topk");
   return DION_OK;

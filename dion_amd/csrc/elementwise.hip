@@ -711,43 +711,55 @@ hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M
 
 // Top-k by rank counting.  Stage 1 (block = 256 candidates of one matrix): the rank of a candidate is
 // the number of entries that beat it (larger value, or equal value at a lower index); it is selected
-// iff rank < k, and the flag goes to map (0 / -1).  NaN counts as +inf.  The whole row sits in LDS and
-// is compared four entries per LDS read; entries before / after the block's own range need one
+// iff rank < k, and the flag goes to map (0 / -1).  NaN counts as +inf.  The row passes through LDS in
+// chunks of kRankChunk entries (one chunk for every dimension a weight matrix has in practice) and is
+// compared four entries per LDS read; entries before / after the block's own range need one
 // comparison each (>= / >).  Stage 2 (one block per matrix) turns the flags into ascending positions.
+constexpr int kRankChunk = 32768;  // floats per LDS chunk (128 KB); a multiple of the 256 candidates
+
 __global__ __launch_bounds__(256) void dion2_rank_kernel(const float* __restrict__ norms, int dim,
                                                          int k, int32_t* __restrict__ map) {
-  extern __shared__ float4 vals4[];  // dim rounded up to 4 floats; padding -1 (never beats anything)
+  extern __shared__ float4 vals4[];  // chunk rounded up to 4 floats; padding -1 (never beats anything)
   float* vals = (float*)vals4;
   const int mat = blockIdx.y;
   const float* v = norms + (int64_t)mat * dim;
-  const int dim4 = (dim + 3) / 4;
-  for (int i = threadIdx.x; i < dim4 * 4; i += 256) {
-    float x = i < dim ? v[i] : -1.0f;
-    if (x != x) x = INFINITY;
-    vals[i] = x;
-  }
-  __syncthreads();
   const int b0 = blockIdx.x * 256;  // multiple of 4
-  const int b1 = (b0 + 256) < dim4 * 4 ? (b0 + 256) : dim4 * 4;
   const int i = b0 + threadIdx.x;
-  if (i >= dim) return;
-  const float x = vals[i];
+  float x = i < dim ? v[i] : 0.f;
+  if (x != x) x = INFINITY;
   int rank = 0;
-  for (int j4 = 0; j4 < b0 / 4; ++j4) {
-    const float4 y = vals4[j4];
-    rank += (y.x >= x) + (y.y >= x) + (y.z >= x) + (y.w >= x);
+  for (int c0 = 0; c0 < dim; c0 += kRankChunk) {
+    const int cn = (dim - c0) < kRankChunk ? (dim - c0) : kRankChunk;
+    const int cn4 = (cn + 3) / 4;
+    __syncthreads();  // the previous chunk has been consumed
+    for (int t = threadIdx.x; t < cn4 * 4; t += 256) {
+      float y = t < cn ? v[c0 + t] : -1.0f;
+      if (y != y) y = INFINITY;
+      vals[t] = y;
+    }
+    __syncthreads();
+    if (i < dim) {
+      // the block's own candidates occupy [lo4, hi4) of this chunk (in float4 units), if at all
+      int lo4 = (b0 > c0 ? b0 - c0 : 0) / 4, hi4 = (b0 + 256 > c0 ? b0 + 256 - c0 : 0) / 4;
+      lo4 = lo4 < cn4 ? lo4 : cn4;
+      hi4 = hi4 < cn4 ? hi4 : cn4;
+      for (int j4 = 0; j4 < lo4; ++j4) {
+        const float4 y = vals4[j4];
+        rank += (y.x >= x) + (y.y >= x) + (y.z >= x) + (y.w >= x);
+      }
+      for (int j4 = lo4; j4 < hi4; ++j4) {
+        const float4 y = vals4[j4];
+        const int j = c0 + j4 * 4;
+        rank += ((y.x > x) || (y.x == x && j < i)) + ((y.y > x) || (y.y == x && j + 1 < i)) +
+                ((y.z > x) || (y.z == x && j + 2 < i)) + ((y.w > x) || (y.w == x && j + 3 < i));
+      }
+      for (int j4 = hi4; j4 < cn4; ++j4) {
+        const float4 y = vals4[j4];
+        rank += (y.x > x) + (y.y > x) + (y.z > x) + (y.w > x);
+      }
+    }
   }
-  for (int j4 = b0 / 4; j4 < b1 / 4; ++j4) {
-    const float4 y = vals4[j4];
-    const int j = j4 * 4;
-    rank += ((y.x > x) || (y.x == x && j < i)) + ((y.y > x) || (y.y == x && j + 1 < i)) +
-            ((y.z > x) || (y.z == x && j + 2 < i)) + ((y.w > x) || (y.w == x && j + 3 < i));
-  }
-  for (int j4 = b1 / 4; j4 < dim4; ++j4) {
-    const float4 y = vals4[j4];
-    rank += (y.x > x) + (y.y > x) + (y.z > x) + (y.w > x);
-  }
-  map[(int64_t)mat * dim + i] = rank < k ? 0 : -1;
+  if (i < dim) map[(int64_t)mat * dim + i] = rank < k ? 0 : -1;
 }
 
 __global__ __launch_bounds__(1024) void dion2_compact_kernel(int dim, int k, int32_t* __restrict__ idx,
@@ -781,7 +793,8 @@ __global__ __launch_bounds__(1024) void dion2_compact_kernel(int dim, int k, int
 
 hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
                              int32_t* map, hipStream_t st) {
-  const size_t shmem = (size_t)((dim + 3) / 4) * 16;
+  const int chunk = dim < kRankChunk ? dim : kRankChunk;
+  const size_t shmem = (size_t)((chunk + 3) / 4) * 16;
   static std::atomic<uint64_t> attr_done{0};
   if (hipError_t e = set_max_dynamic_lds_once((const void*)dion2_rank_kernel, 160 * 1024 - 256, attr_done))
     return e;

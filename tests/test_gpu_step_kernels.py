@@ -291,3 +291,29 @@ def test_scalar_groups_inside_an_optimizer():
         xb, mb, vb = b.data.double().cpu(), opt.state[b]["momentum"].double().cpu(), opt.state[b]["variance"].double().cpu()
         xe, me = e.data.double().cpu(), opt.state[e]["momentum"].double().cpu()
     assert float(opt.state[b]["step_dev"]) == 3.0
+
+
+@pytest.mark.parametrize("dim,k", [(70001, 17501), (32768, 100), (32769, 1), (40000, 40000)])
+def test_topk_past_one_lds_chunk(dim, k):
+    """Rank-counting top-k on rows longer than one LDS chunk (32 768 entries), with heavy ties and a NaN:
+    the selected set is the k first entries of a stable descending sort (ties to the lower index, NaN
+    first), idx ascending, map its inverse."""
+    from dion_amd import _lib
+
+    lib = _lib.load()
+    torch.manual_seed(40)
+    norms = torch.randint(0, 2000, (2, dim)).float()  # many equal values
+    norms[1, dim // 2] = float("nan")
+    nd = norms.to(DEV)
+    idx = torch.empty(2, k, dtype=torch.int32, device=DEV)
+    imap = torch.empty(2, dim, dtype=torch.int32, device=DEV)
+    _lib.check(lib.dion_dion2_topk(nd.data_ptr(), 2, dim, k, idx.data_ptr(), imap.data_ptr(),
+                                   torch.cuda.current_stream().cuda_stream), "topk")
+    key = torch.nan_to_num(norms, nan=float("inf"))
+    for b in range(2):
+        order = torch.sort(key[b], descending=True, stable=True).indices[:k]
+        ref = order.sort().values.to(torch.int32)
+        assert torch.equal(idx[b].cpu(), ref)
+        inv = torch.full((dim,), -1, dtype=torch.int32)
+        inv[ref.long()] = torch.arange(k, dtype=torch.int32)
+        assert torch.equal(imap[b].cpu(), inv)
