@@ -51,6 +51,7 @@ extern "C" int dion_ns_line_1(const void* X, void* A, int batch, int m, int k, v
   if (int rc = check_gemm_dims("dion_ns_line_1", batch, m, k)) return rc;
   if (batch == 0 || m == 0) return DION_OK;
   if (k == 0) return fail(DION_E_INVALID, "dion_ns_line_1: k == 0");
+  if (!X || !A) return fail(DION_E_INVALID, "dion_ns_line_1: null argument");
   GemmParams p;
   memset(&p, 0, sizeof(p));
   p.P = p.Q = (const bf16_t*)X;
@@ -72,6 +73,7 @@ extern "C" int dion_ns_line_2(const void* A, void* B, int batch, int m, float al
                               void* stream) {
   if (int rc = check_gemm_dims("dion_ns_line_2", batch, m, m)) return rc;
   if (batch == 0 || m == 0) return DION_OK;
+  if (!A || !B) return fail(DION_E_INVALID, "dion_ns_line_2: null argument");
   if (A == B) return fail(DION_E_INVALID, "dion_ns_line_2: in-place not supported");
   GemmParams p;
   memset(&p, 0, sizeof(p));
@@ -93,6 +95,7 @@ extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void
   if (int rc = check_gemm_dims("dion_ns_line_3", batch, m, n)) return rc;
   if (batch == 0 || m == 0 || n == 0) return DION_OK;
   if (!C && !Ct) return fail(DION_E_INVALID, "dion_ns_line_3: no output");
+  if (!B || (!X && !Xt)) return fail(DION_E_INVALID, "dion_ns_line_3: null argument");
   GemmParams p;
   memset(&p, 0, sizeof(p));
   p.P = (const bf16_t*)B;

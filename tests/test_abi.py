@@ -88,6 +88,10 @@ def test_argument_validation_happens_before_any_device_work():
                                        f(0.0), f(0.9), None), "bad size")
     refused(lib.dion_ns_orthogonalize(None, 9, None, 1, 8, 8, None, 0, f(1.0), f(0.0), 0, 0, None, 0, None),
             "in_dtype")
+    refused(lib.dion_ns_line_1(None, None, 1, 128, 128, None), "null argument")
+    refused(lib.dion_ns_line_2(None, None, 1, 128, f(1.0), f(1.0), None), "null argument")
+    refused(lib.dion_ns_line_3(None, None, None, None, None, 1, 128, 128, f(0.0), None), "no output")
+    refused(lib.dion_ns_line_1(None, None, 1, 100, 128, None), "multiples of 128")
     # empty problems are accepted and do nothing
     assert lib.dion_slice_l1(None, 0, 0, 8, 8, -2, 0, None, None) == 0
     assert lib.dion_gather_slices(None, 0, 1, 8, 8, -2, None, 0, None, None) == 0
