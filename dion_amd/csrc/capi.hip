@@ -252,7 +252,9 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
           "frobenius norm");
   // Default: X' = B X reads X itself (reduction index along rows) and no X^T is carried.
   // DION_NS_CARRY_XT keeps X and X^T side by side instead.
-  const bool nn = (flags & DION_NS_CARRY_XT) == 0;
+  // (With no iteration at all the result is the prepared input: keep both layouts then, the output
+  // copy reads X^T for a tall input.)
+  const bool nn = (flags & DION_NS_CARRY_XT) == 0 && n_iters > 0;
   if (pl.tall)
     HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, nn ? nullptr : Xt[0], np, mp, ldxt, sXt,
                               X[0], ldx, sX, st),

@@ -319,3 +319,17 @@ def test_batches_beyond_one_library_call():
     for lo in (0, 32760, 39990):
         assert torch.equal(out[lo:lo + 10], zeropower_via_newtonschulz5(G[lo:lo + 10].contiguous()))
     assert bool(torch.isfinite(out.float()).all())
+
+
+@pytest.mark.parametrize("shape", [(2, 256, 512), (2, 512, 256), (100, 36), (36, 100)])
+def test_zero_iterations_return_the_normalised_input(shape):
+    """steps = 0: the output is bf16(G) / (||bf16(G)||_F + eps), wide or tall, padded or not."""
+    from dion_amd import zeropower_kj
+
+    torch.manual_seed(22)
+    G = torch.randn(shape, device=DEV)
+    out = zeropower_kj(G, steps=0)
+    g = G.to(torch.bfloat16).float()
+    ref = g / (g.flatten(-2).norm(dim=-1).view(*shape[:-2], 1, 1) + 1e-7)
+    assert out.shape == G.shape
+    assert float((out.float() - ref).abs().max()) <= 2.0 ** -8 * float(ref.abs().max())
