@@ -35,7 +35,7 @@ SIGNATURES = {
     "dion_muon_post": (c_int, [_u64p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p, c_void_p,
                                c_float, c_void_p, c_float, c_int, c_void_p]),
     "dion_normuon_stats": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_float, c_void_p,
-                                   c_void_p, c_void_p]),
+                                   c_void_p]),
     "dion_normuon_stats_selected": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_void_p, c_int,
                                             c_float, c_void_p, c_void_p]),
     "dion_dion2_accumulate_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),

@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 5; }
+extern "C" int dion_abi_version(void) { return 6; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -439,6 +439,13 @@ static bool table_aligned(const uint64_t* t, int n) {
   return true;
 }
 
+// Pointers per launch when every pointer covers mats_per_ptr matrices and the launch puts one
+// matrix on each gridDim.y slot (at most 65535); 0 if even one pointer is too many.
+static int ptr_chunk(int mats_per_ptr) {
+  const int c = 65535 / mats_per_ptr;
+  return c < kMaxPtrs ? c : kMaxPtrs;
+}
+
 static void fill_tab(PtrTab& tab, const uint64_t* src, int n) {
   memset(&tab, 0, sizeof(tab));
   memcpy(tab.p, src, (size_t)n * sizeof(uint64_t));
@@ -497,8 +504,10 @@ static int normuon_stats_impl(const char* who, const void* U, const uint64_t* V_
   if (n == 0 || rows == 0 || cols == 0) return DION_OK;
   if (!U || !V_ptrs || !row_scale) return fail(DION_E_INVALID, "%s: null argument", who);
   const float w = 1.0f - beta2;
-  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
-    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+  const int cmax = ptr_chunk(mats_per_ptr);  // matrices of one launch sit on gridDim.y
+  if (cmax == 0) return fail(DION_E_INVALID, "more than 65535 matrices behind one pointer");
+  for (int i0 = 0; i0 < n; i0 += cmax) {
+    const int c = (n - i0) < cmax ? (n - i0) : cmax;
     PtrTab v;
     fill_tab(v, V_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
@@ -511,9 +520,7 @@ static int normuon_stats_impl(const char* who, const void* U, const uint64_t* V_
 }
 
 extern "C" int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr,
-                                  int rows, int cols, float beta2, float* row_scale, float* scratch,
-                                  void* stream) {
-  (void)scratch;
+                                  int rows, int cols, float beta2, float* row_scale, void* stream) {
   return normuon_stats_impl("dion_normuon_stats", U, V_ptrs, n, mats_per_ptr, rows, cols, nullptr, rows,
                             beta2, row_scale, stream);
 }
@@ -560,8 +567,10 @@ extern "C" int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const 
     slabs = dion2_acc_slabs((int)n_mat, rows, cols);
     if ((size_t)slabs * n_mat * cols * sizeof(float) > scratch_bytes) slabs = 1;
   }
-  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
-    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+  const int cmax = ptr_chunk(mats_per_ptr);  // matrices of one launch sit on gridDim.y
+  if (cmax == 0) return fail(DION_E_INVALID, "more than 65535 matrices behind one pointer");
+  for (int i0 = 0; i0 < n; i0 += cmax) {
+    const int c = (n - i0) < cmax ? (n - i0) : cmax;
     PtrTab g, m;
     fill_tab(g, G_ptrs + i0, c);
     fill_tab(m, M_ptrs + i0, c);
@@ -579,7 +588,12 @@ extern "C" int dion_dion2_topk(const float* norms, int n_mat, int dim, int k, in
   if (n_mat < 0 || dim < 0 || k < 0 || k > dim) return fail(DION_E_INVALID, "dion_dion2_topk: bad size");
   if (n_mat == 0 || dim == 0) return DION_OK;
   if (!norms || !idx || !map) return fail(DION_E_INVALID, "dion_dion2_topk: null argument");
-  HIP_TRY(launch_dion2_topk(norms, n_mat, dim, k, idx, map, (hipStream_t)stream), "dion_dion2_topk");
+  for (int m0 = 0; m0 < n_mat; m0 += 65535) {  // one matrix per gridDim.y slot
+    const int c = (n_mat - m0) < 65535 ? (n_mat - m0) : 65535;
+    HIP_TRY(launch_dion2_topk(norms + (int64_t)m0 * dim, c, dim, k, idx + (int64_t)m0 * k,
+                              map + (int64_t)m0 * dim, (hipStream_t)stream),
+            "dion_dion2_topk");
+  }
   return DION_OK;
 }
 
@@ -593,8 +607,10 @@ extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr
   if (!M_ptrs || !idx || !U_sel) return fail(DION_E_INVALID, "dion_dion2_gather: null argument");
   const int64_t sel_numel = select_dim == -2 ? (int64_t)k * cols : (int64_t)rows * k;
   const bool vec4 = (cols % 4 == 0) && table_aligned(M_ptrs, n) && aligned16((uint64_t)U_sel);
-  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
-    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+  const int cmax = ptr_chunk(mats_per_ptr);  // matrices of one launch sit on gridDim.y
+  if (cmax == 0) return fail(DION_E_INVALID, "more than 65535 matrices behind one pointer");
+  for (int i0 = 0; i0 < n; i0 += cmax) {
+    const int c = (n - i0) < cmax ? (n - i0) : cmax;
     PtrTab m;
     fill_tab(m, M_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
@@ -624,8 +640,10 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
   const int es = u_dtype == DION_BF16 ? 2 : 4;
   const bool vec4 = (cols % 4 == 0) && table_aligned(X_ptrs, n) && aligned16((uint64_t)U_sel) &&
                     aligned16((uint64_t)map);
-  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
-    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+  const int cmax = ptr_chunk(mats_per_ptr);  // matrices of one launch sit on gridDim.y
+  if (cmax == 0) return fail(DION_E_INVALID, "more than 65535 matrices behind one pointer");
+  for (int i0 = 0; i0 < n; i0 += cmax) {
+    const int c = (n - i0) < cmax ? (n - i0) : cmax;
     PtrTab x;
     fill_tab(x, X_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
@@ -726,8 +744,10 @@ extern "C" int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_
   const int dim = select_dim == -2 ? rows : cols;
   const bool vec4 = (cols % 4 == 0) && table_aligned(X_ptrs, n) && table_aligned(M_ptrs, n) &&
                     aligned16((uint64_t)U) && aligned16((uint64_t)norms);
-  for (int i0 = 0; i0 < n; i0 += kMaxPtrs) {
-    const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
+  const int cmax = ptr_chunk(mats_per_ptr);  // matrices of one launch sit on gridDim.y
+  if (cmax == 0) return fail(DION_E_INVALID, "more than 65535 matrices behind one pointer");
+  for (int i0 = 0; i0 < n; i0 += cmax) {
+    const int c = (n - i0) < cmax ? (n - i0) : cmax;
     PtrTab x, m;
     fill_tab(x, X_ptrs + i0, c);
     fill_tab(m, M_ptrs + i0, c);

@@ -277,7 +277,7 @@ def normuon_stats(U: Tensor, V: List[Tensor], beta2: float) -> Tensor:
     scale = torch.empty(n_mat, rows, dtype=torch.float32, device=U.device)
     lib = _lib.load()
     check(lib.dion_normuon_stats(U.data_ptr(), vp, n, mats_per_ptr, rows, cols, float(beta2),
-                                 scale.data_ptr(), None, _stream_handle(U.device)), "normuon_stats")
+                                 scale.data_ptr(), _stream_handle(U.device)), "normuon_stats")
     return scale
 
 

@@ -115,15 +115,17 @@ int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype, int n, in
  *   r = mean(U^2, dim=-1); V = lerp(V, r, 1-beta2); d = sqrt(V)+1e-8;
  *   row_scale[i][r] = (1/d) * ||U_i||_F / max(||U_i / d||_F, 1e-8)
  * U [n_mat, rows, cols] bf16 (orthogonalized); V_ptrs: host ptr table of n device pointers, each
- * to mats_per_ptr*rows fp32 (n*mats_per_ptr == n_mat); row_scale out [n_mat, rows] fp32; scratch:
- * device fp32 [2*n_mat].  The scaled update is applied by dion_muon_post(row_scale=...).
+ * to mats_per_ptr*rows fp32 (n*mats_per_ptr == n_mat); row_scale out [n_mat, rows] fp32.  The
+ * scaled update is applied by dion_muon_post(row_scale=...).
  * Replaces normuon_normalization_stacked (dion/normuon.py:345-399) and the V write-back of
  * dion/normuon.py:320. */
 int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr, int rows,
-                       int cols, float beta2, float* row_scale, float* scratch, void* stream);
+                       int cols, float beta2, float* row_scale, void* stream);
 
 /* NorMuon statistics for an update made of k selected rows per matrix (NorDion2): U [n_mat, k,
- * cols] bf16, row_idx [n_mat, k] int32 gives the row of the parameter each update row belongs to;
+ * cols] bf16, row_idx [n_mat, k] int32 gives the row of the parameter each update row belongs to
+ * (a negative entry: that update row is not part of the update, its second moment stays and its
+ * scale is 0);
  * V_ptrs entries each point to mats_per_ptr * v_rows fp32 (the full per-row buffers); only the
  * selected entries of V are read and written.  row_scale out [n_mat, k].
  * Replaces nordion2_normalize_selected_stacked (dion/nordion2.py:430-447). */

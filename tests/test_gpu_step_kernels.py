@@ -317,3 +317,39 @@ def test_topk_past_one_lds_chunk(dim, k):
         inv = torch.full((dim,), -1, dtype=torch.int32)
         inv[ref.long()] = torch.arange(k, dtype=torch.int32)
         assert torch.equal(imap[b].cpu(), inv)
+
+
+def test_many_matrices_per_launch_are_chunked():
+    """Three 3-D parameters of 30000 matrices each: more matrices than one launch addresses (65535), so
+    the pointer table is cut into launches of two parameters and one; through the Dion2 select / post and
+    the NorMuon statistics kernels.  More than 65535 matrices behind a single pointer are refused."""
+    from dion_amd import ops
+
+    torch.manual_seed(41)
+    n, L, rows, cols = 3, 30000, 4, 8
+    G = [torch.randn(L, rows, cols, device=DEV).to(torch.bfloat16) for _ in range(n)]
+    M = [torch.zeros(L, rows, cols, device=DEV) for _ in range(n)]
+    U, idx, imap = ops.dion2_select(G, M, 2, -2, 0.5)
+    assert U.shape == (n, L, 2, cols) and idx.shape == (n * L, 2)
+    g_all = torch.stack(G).view(n * L, rows, cols)
+    norms = g_all.float().abs().sum(-1)
+    srt = norms.sort(-1, descending=True).values
+    tie_free = srt[:, 1] > srt[:, 2]
+    ref = norms.topk(2, dim=-1).indices.sort(-1).values.to(torch.int32)
+    assert torch.equal(idx[tie_free], ref[tie_free])
+    X = [torch.randn(L, rows, cols, device=DEV) for _ in range(n)]
+    x0 = torch.stack(X).view(n * L, rows, cols).clone()
+    lr = torch.tensor(0.1, device=DEV)
+    ops.dion2_post(X, U, imap, lr, 1.0, 0.0, -2)
+    full = torch.zeros(n * L, rows, cols, device=DEV)
+    full.scatter_(1, idx.long().unsqueeze(-1).expand(n * L, 2, cols), U.view(n * L, 2, cols).float())
+    assert torch.allclose(torch.stack(X).view(n * L, rows, cols), x0 - 0.1 * full, rtol=1e-6, atol=1e-7)
+    V = [torch.zeros(L, rows, 1, device=DEV) for _ in range(n)]
+    O = torch.randn(n, L, rows, cols, device=DEV).to(torch.bfloat16)
+    scale = ops.normuon_stats(O, V, 0.9)
+    assert scale.shape == (n * L, rows)
+    assert torch.allclose(torch.stack(V).view(n * L, rows), 0.1 * (O.view(n * L, rows, cols).float() ** 2).mean(-1),
+                          rtol=1e-5)
+    with pytest.raises(ValueError, match="65535"):
+        ops.dion2_select([torch.zeros(70000, 2, 4, device=DEV, dtype=torch.bfloat16)],
+                         [torch.zeros(70000, 2, 4, device=DEV)], 1, -2, 0.5)
