@@ -1,4 +1,4 @@
-"""Shared host logic of the Muon / NorMuon / Dion2 optimizers on one MI355X.
+"""Shared host logic of the Muon / NorMuon / Dion2 / NorDion2 optimizers on one MI355X.
 
 Mirrors the single-GPU behaviour of the reference's ``DistributedOrthoBase``
 (dion/megabatch_base.py:22-632): same constructor contract, param-group keys, eager state
@@ -20,7 +20,7 @@ from . import scalar_opts
 
 class OrthoOptimizer(Optimizer):
     """Base class: orchestration, state and validation.  Subclasses implement
-    ``_update_shape_group``."""
+    ``_shape_group_phases`` (a generator: work before / during / after the orthogonalization)."""
 
     def __init__(self, params, distributed_mesh, algo_name: str, defaults: dict,
                  use_gram_newton_schulz: bool = False, use_triton: bool = False,
