@@ -10,6 +10,7 @@ from typing import List, Optional, Sequence, Tuple
 
 import torch
 from torch import Tensor
+from torch.utils._python_dispatch import is_traceable_wrapper_subclass
 
 from . import _lib
 from ._lib import DION_BF16, DION_F32, DION_NS_GRAM, DION_NS_CARRY_XT, check, ptr_table
@@ -20,6 +21,13 @@ def _stream_handle(device: torch.device) -> int:
 
 
 def _require_gpu(t: Tensor, name: str) -> None:
+    # The kernels write through raw device pointers.  A wrapper subclass (DTensor, quantised-weight
+    # wrappers) keeps its data in inner tensors and exposes no dense buffer at data_ptr()
+    # (the case dion/dion2_triton.py:171-190 routes around): refuse it instead of writing somewhere.
+    if is_traceable_wrapper_subclass(t):
+        raise TypeError(
+            f"{name}: {type(t).__name__} is a tensor wrapper subclass; pass its plain local tensor"
+        )
     if not t.is_cuda:
         raise RuntimeError(
             f"{name} must be a GPU tensor (got device {t.device}); the dion_amd kernels have no CPU path"

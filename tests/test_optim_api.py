@@ -202,3 +202,44 @@ def test_graph_wrapper_host_contract():
     steps = [g["step"] for g in inner.param_groups]
     inner._advance_host_step_counters()
     assert [g["step"] for g in inner.param_groups] == [s + 1 for s in steps]
+
+
+def test_wrapper_subclass_tensors_are_refused():
+    """A tensor wrapper subclass has no dense buffer behind data_ptr() (the case the reference routes
+    around, dion/dion2_triton.py:171-190, tests/test_dion2_post_ortho_triton.py:95-159): the raw-pointer
+    entry points refuse it with TypeError rather than write through a meaningless pointer."""
+    import torch
+    from torch.utils._pytree import tree_map
+
+    from dion_amd import ops
+
+    class Wrapper(torch.Tensor):
+        @staticmethod
+        def __new__(cls, inner):
+            return torch.Tensor._make_wrapper_subclass(cls, inner.shape, dtype=inner.dtype, device=inner.device,
+                                                       layout=inner.layout, strides=inner.stride(),
+                                                       requires_grad=False)
+
+        def __init__(self, inner):
+            self._inner = inner
+
+        def __tensor_flatten__(self):
+            return ["_inner"], None
+
+        @staticmethod
+        def __tensor_unflatten__(inner_tensors, meta, outer_size, outer_stride):
+            return Wrapper(inner_tensors["_inner"])
+
+        @classmethod
+        def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
+            unwrap = lambda t: t._inner if isinstance(t, Wrapper) else t
+            return func(*tree_map(unwrap, args), **tree_map(unwrap, kwargs or {}))
+
+    w = Wrapper(torch.zeros(8, 16))
+    with pytest.raises(TypeError, match="wrapper subclass"):
+        ops.muon_pre([w], [torch.zeros(8, 16)], 0.9, False)
+    with pytest.raises(TypeError, match="wrapper subclass"):
+        ops.ns_orthogonalize(w, [(1.0, 0.0, 0.0)], 1.0, 1e-7)
+    # a plain dense subclass is not a wrapper
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.ns_orthogonalize(torch.nn.Parameter(torch.zeros(8, 16)), [(1.0, 0.0, 0.0)], 1.0, 1e-7)
