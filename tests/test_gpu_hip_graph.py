@@ -111,3 +111,151 @@ def test_capture_refuses_params_without_grad():
     opt.step()  # warm-up step is eager and simply skips the param without a gradient
     with pytest.raises(RuntimeError, match="grad=None at graph capture"):
         opt.step()
+
+
+def _zero_grads(params):
+    for p in params:
+        p.grad = torch.zeros_like(p)
+
+
+def test_frozen_parameter_is_allowed_and_release_rewarms():
+    """A parameter frozen on purpose (requires_grad=False, no gradient) does not block the capture;
+    release() drops the graph and restarts the warm-up, twice in a row is a no-op, and before any
+    capture it still resets the warm-up count (dion/cuda_graph.py:183-200, the contract of the reference's
+    tests/test_cuda_graph.py:765-815)."""
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    params, inner = _build("Dion2", dict(fraction=0.25), 8)
+    wrap = CudaGraphOptimizer(inner, warmup_steps=1)
+    _zero_grads(params)
+    wrap.step()
+    params[0].grad = None
+    params[0].requires_grad_(False)
+    wrap.step()
+    assert wrap._graph is not None
+    wrap.release()
+    assert wrap._graph is None and wrap._step_count == 0
+    wrap.release()
+    wrap.step()
+    assert wrap._graph is None
+    wrap.step()
+    assert wrap._graph is not None
+
+    params, inner = _build("Dion2", dict(fraction=0.25), 8)
+    wrap = CudaGraphOptimizer(inner, warmup_steps=3)
+    _zero_grads(params)
+    wrap.step()
+    wrap.step()
+    assert wrap._graph is None and wrap._step_count == 2
+    wrap.release()
+    assert wrap._step_count == 0
+
+
+def test_failed_capture_leaves_no_graph_and_lr_sync_under_capture_is_an_error():
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    params, inner = _build("Muon", {}, 9)
+    wrap = CudaGraphOptimizer(inner, warmup_steps=1)
+    _zero_grads(params)
+    wrap.step()
+    real_step = inner.step
+
+    def boom(*a, **k):
+        raise RuntimeError("capture blew up")
+
+    inner.step = boom
+    with pytest.raises(RuntimeError, match="capture blew up"):
+        wrap.step()
+    assert wrap._graph is None
+    inner.step = real_step
+    torch.cuda.synchronize()
+    wrap.step()  # captures now
+    assert wrap._graph is not None
+
+    # writing the lr tensor inside a capture would bake the capture-time value into every replay
+    params, opt = _build("Dion2", dict(fraction=0.25), 9)
+    _zero_grads(params)
+    opt.step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, capture_error_mode="thread_local"):
+        torch.zeros(4, device=DEV).add_(1)  # keep the capture non-empty
+        for g in opt.param_groups:
+            g["lr"] = 0.5
+        with pytest.raises(RuntimeError, match="capture"):
+            opt._sync_hyperparam_tensors()
+    del graph
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("cls_name,kwargs", [("Muon", {}), ("NorMuon", {}), ("Dion2", dict(fraction=0.25)),
+                                             ("NorDion2", dict(fraction=0.5))])
+def test_scheduled_lr_tracks_after_resume_and_closure(cls_name, kwargs):
+    """An optimizer restored from a checkpoint (state_dict through torch.save / load with
+    map_location="cpu", loaded by keyword) and then wrapped follows a scheduled learning rate under replay
+    exactly like the eager one; step(closure) returns the closure's value."""
+    import io
+
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    p_src, o_src = _build(cls_name, dict(kwargs), 11)
+    gen = torch.Generator(device=DEV).manual_seed(12)
+    for p in p_src:
+        p.grad = torch.randn(p.shape, device=DEV, generator=gen)
+    o_src.step()
+    o_src.step()
+    buf = io.BytesIO()
+    torch.save(o_src.state_dict(), buf)
+    weights = [p.detach().clone() for p in p_src]
+
+    def resumed():
+        params, opt = _build(cls_name, dict(kwargs), 11)
+        for p, w in zip(params, weights):
+            p.data.copy_(w)
+        buf.seek(0)
+        sd = torch.load(buf, map_location="cpu", weights_only=True)
+        return params, opt, sd
+
+    p_e, o_e, sd = resumed()
+    o_e.load_state_dict(sd)
+    p_g, inner, sd = resumed()
+    o_g = CudaGraphOptimizer(inner, warmup_steps=2)
+    o_g.load_state_dict(state_dict=sd)
+    assert inner.param_groups[0]["step"] == o_src.param_groups[0]["step"] == 2
+    assert all(isinstance(g["lr"], torch.Tensor) and g["lr"].is_cuda for g in inner.param_groups)
+    _zero_grads(p_e + p_g)
+    for step in range(7):
+        for a, b in zip(p_e, p_g):
+            g = torch.randn(a.shape, device=DEV, generator=gen)
+            a.grad.copy_(g)
+            b.grad.copy_(g)
+        for grp_e, grp_g in zip(o_e.param_groups, inner.param_groups):
+            lr = 0.02 * (0.25 + 1.5 * (step + 1) / 7)
+            grp_e["lr"] = lr
+            grp_g["lr"] = lr
+        o_e.step()
+        assert o_g.step(lambda: torch.tensor(3.0)) == 3.0
+        for a, b in zip(p_e, p_g):
+            assert torch.equal(a.data, b.data), (cls_name, step)
+    assert o_g._graph is not None
+
+
+def test_add_param_group_rewarms_before_recapturing():
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    params, inner = _build("Muon", {}, 13)
+    wrap = CudaGraphOptimizer(inner, warmup_steps=2)
+    _zero_grads(params)
+    for _ in range(3):
+        wrap.step()
+    assert wrap._graph is not None
+    extra = torch.nn.Parameter(torch.randn(128, 256, device=DEV) * 0.02)
+    extra.grad = torch.zeros_like(extra)
+    wrap.add_param_group(dict(params=[extra]))
+    assert wrap._graph is None and wrap._step_count == 0
+    wrap.step()
+    wrap.step()
+    assert wrap._graph is None       # two eager steps for the new group first
+    wrap.step()
+    assert wrap._graph is not None
+    assert isinstance(inner.param_groups[-1]["lr"], torch.Tensor)

@@ -243,3 +243,22 @@ def test_wrapper_subclass_tensors_are_refused():
     # a plain dense subclass is not a wrapper
     with pytest.raises(RuntimeError, match="no CPU path"):
         ops.ns_orthogonalize(torch.nn.Parameter(torch.zeros(8, 16)), [(1.0, 0.0, 0.0)], 1.0, 1e-7)
+
+
+def test_graph_wrapper_signatures_match_torch_optimizer():
+    """The wrapper stands in for a torch.optim.Optimizer: every method it overrides keeps the base class's
+    parameter names and kinds (callers such as distributed checkpointing pass ``state_dict=`` by keyword;
+    the contract of the reference's tests/test_cuda_graph.py:818-870).  Defaults are not pinned:
+    zero_grad's set_to_none defaults to False here because replay needs stable .grad buffers."""
+    import inspect
+
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    overridden = sorted(name for name, attr in vars(CudaGraphOptimizer).items()
+                        if callable(attr) and not name.startswith("_") and hasattr(torch.optim.Optimizer, name))
+    assert "load_state_dict" in overridden and "step" in overridden and "zero_grad" in overridden
+    for name in overridden:
+        base = inspect.signature(getattr(torch.optim.Optimizer, name))
+        mine = inspect.signature(getattr(CudaGraphOptimizer, name))
+        assert [(p.name, p.kind) for p in mine.parameters.values()] == \
+               [(p.name, p.kind) for p in base.parameters.values()], name
