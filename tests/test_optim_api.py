@@ -262,3 +262,34 @@ def test_graph_wrapper_signatures_match_torch_optimizer():
         mine = inspect.signature(getattr(CudaGraphOptimizer, name))
         assert [(p.name, p.kind) for p in mine.parameters.values()] == \
                [(p.name, p.kind) for p in base.parameters.values()], name
+
+
+@pytest.mark.parametrize("cls,extra", [(Muon, set()), (Dion2, set()), (NorMuon, {"variance_neuron"}),
+                                       (NorDion2, {"variance_neuron"})])
+def test_add_param_group_prepopulates_and_state_dict_is_complete(cls, extra):
+    """State for a group added later exists at once, and a state_dict taken before any step carries
+    every parameter's state and loads into a fresh optimizer (the contract of the reference's
+    tests/test_state_prepopulation.py:55-86)."""
+    p = _params([(16, 32)])
+    opt = cls(p, lr=0.01)
+    late = _params([(8, 24), (8, 24)])
+    opt.add_param_group({"params": late})
+    for q in late:
+        assert set(opt.state[q].keys()) == {"momentum"} | extra
+    assert isinstance(opt.param_groups[1]["lr"], torch.Tensor)
+    sd = opt.state_dict()
+    assert len(sd["state"]) == 3 and all({"momentum"} | extra <= set(s) for s in sd["state"].values())
+    assert all(isinstance(g["lr"], float) for g in sd["param_groups"])
+    fresh = cls([{"params": _params([(16, 32)])}, {"params": _params([(8, 24), (8, 24)])}], lr=0.5)
+    fresh.load_state_dict(sd)
+    assert float(fresh.param_groups[0]["lr"]) == pytest.approx(0.01)
+    assert len(fresh.state) == 3
+
+
+def test_empty_lists_are_accepted_by_the_list_functions():
+    """The reference's foreach functions return at once on an empty list
+    (tests/test_adamw_foreach.py:218-222); so do these, before any device work."""
+    from dion.scalar_opts import adamw_update_foreach, lion_update_foreach
+
+    adamw_update_foreach([], [], [], [], 0.01, 0.9, 0.95, 0.1, 1, 1e-8)
+    lion_update_foreach([], [], [], 0.01, 0.9, 0.99, 0.1)
