@@ -15,6 +15,7 @@ DION_BF16 = 0
 DION_F32 = 1
 DION_NS_GRAM = 1
 DION_NS_CARRY_XT = 2
+ABI_VERSION = 7  # dion_abi_version() of the library these signatures describe
 
 _u64p = ctypes.POINTER(ctypes.c_uint64)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -31,20 +32,20 @@ SIGNATURES = {
     "dion_ns_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "dion_ns_orthogonalize": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, _f32p, c_int,
                                       c_float, c_float, c_int, c_int, c_void_p, c_size_t, c_void_p]),
-    "dion_muon_pre": (c_int, [_u64p, c_int, _u64p, c_void_p, c_int, c_int64, c_float, c_int, c_void_p]),
-    "dion_muon_post": (c_int, [_u64p, c_void_p, c_int, c_int, c_int64, c_int, c_void_p, c_void_p,
+    "dion_muon_pre": (c_int, [_u64p, c_int, _u64p, c_int, c_void_p, c_int, c_int64, c_float, c_int, c_void_p]),
+    "dion_muon_post": (c_int, [_u64p, c_int, c_void_p, c_int, c_int, c_int64, c_int, c_void_p, c_void_p,
                                c_float, c_void_p, c_float, c_int, c_void_p]),
-    "dion_normuon_stats": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_float, c_void_p,
+    "dion_normuon_stats": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p,
                                    c_void_p]),
-    "dion_normuon_stats_selected": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_void_p, c_int,
+    "dion_normuon_stats_selected": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,
                                             c_float, c_void_p, c_void_p]),
     "dion_dion2_accumulate_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
-    "dion_dion2_accumulate": (c_int, [_u64p, c_int, _u64p, c_int, c_int, c_int, c_int, c_int,
+    "dion_dion2_accumulate": (c_int, [_u64p, c_int, _u64p, c_int, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_void_p, c_size_t, c_void_p]),
     "dion_dion2_topk": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
-    "dion_dion2_gather": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
+    "dion_dion2_gather": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
                                   c_void_p, c_void_p]),
-    "dion_dion2_post": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p,
+    "dion_dion2_post": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float, c_void_p]),
     "dion_dion2_index_map": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "dion_slice_l1": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
@@ -53,12 +54,12 @@ SIGNATURES = {
     "dion_scatter_slices": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
                                     c_void_p]),
     "dion_mask_index": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
-    "dion_dion2_post_masked": (c_int, [_u64p, _u64p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+    "dion_dion2_post_masked": (c_int, [_u64p, _u64p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float, c_float,
                                        c_void_p]),
-    "dion_adamw_step": (c_int, [_u64p, _u64p, c_int, _u64p, _u64p, _u64p, _i64p, c_int, c_void_p, c_float,
+    "dion_adamw_step": (c_int, [_u64p, _u64p, c_int, _u64p, _u64p, c_int, _u64p, _i64p, c_int, c_void_p, c_float,
                                 c_float, c_float, c_void_p, c_float, c_int, c_void_p]),
-    "dion_lion_step": (c_int, [_u64p, _u64p, c_int, _u64p, _i64p, c_int, c_void_p, c_float, c_float,
+    "dion_lion_step": (c_int, [_u64p, _u64p, c_int, _u64p, c_int, _i64p, c_int, c_void_p, c_float, c_float,
                                c_void_p, c_float, c_int, c_void_p]),
 }
 
@@ -84,6 +85,12 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
+    built = lib.dion_abi_version()
+    if built != ABI_VERSION:
+        raise ImportError(
+            f"{LIB_PATH} was built with ABI version {built}, this binding describes version {ABI_VERSION}: "
+            "rebuild it with `python -m dion_amd._build`."
+        )
     _lib = lib
     return lib
 

@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 6; }
+extern "C" int dion_abi_version(void) { return 7; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -446,14 +446,22 @@ static int ptr_chunk(int mats_per_ptr) {
   return c < kMaxPtrs ? c : kMaxPtrs;
 }
 
+static int check_state_dtype(const char* who, const char* arg, int dtype) {
+  if (dtype != DION_BF16 && dtype != DION_F32)
+    return fail(DION_E_INVALID, "%s: %s %d (DION_BF16 or DION_F32)", who, arg, dtype);
+  return DION_OK;
+}
+static inline int dt(int dtype) { return dtype == DION_BF16 ? 0 : 1; }
+
 static void fill_tab(PtrTab& tab, const uint64_t* src, int n) {
   memset(&tab, 0, sizeof(tab));
   memcpy(tab.p, src, (size_t)n * sizeof(uint64_t));
 }
 
-extern "C" int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, void* U,
-                             int n, int64_t numel, float mu, int nesterov, void* stream) {
+extern "C" int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int m_dtype,
+                             void* U, int n, int64_t numel, float mu, int nesterov, void* stream) {
   if (n < 0 || numel < 0) return fail(DION_E_INVALID, "dion_muon_pre: negative size");
+  if (int rc = check_state_dtype("dion_muon_pre", "m_dtype", m_dtype)) return rc;
   if (g_dtype != DION_BF16 && g_dtype != DION_F32) return fail(DION_E_INVALID, "dion_muon_pre: g_dtype");
   if (n == 0 || numel == 0) return DION_OK;
   if (!G_ptrs || !M_ptrs || !U) return fail(DION_E_INVALID, "dion_muon_pre: null argument");
@@ -464,18 +472,19 @@ extern "C" int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t
     PtrTab g, m;
     fill_tab(g, G_ptrs + i0, c);
     fill_tab(m, M_ptrs + i0, c);
-    HIP_TRY(launch_muon_pre(g, g_dtype, m, (bf16_t*)U + (int64_t)i0 * numel, c, numel, mu, nesterov,
-                            vec, (hipStream_t)stream),
+    HIP_TRY(launch_muon_pre(g, dt(g_dtype), m, dt(m_dtype), (bf16_t*)U + (int64_t)i0 * numel, c, numel, mu,
+                            nesterov, vec, (hipStream_t)stream),
             "dion_muon_pre");
   }
   return DION_OK;
 }
 
-extern "C" int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype, int n,
+extern "C" int dion_muon_post(const uint64_t* X_ptrs, int x_dtype, const void* U, int u_dtype, int n,
                               int64_t numel, int cols, const float* row_scale, const float* lr_dev,
                               float adj_ratio, const float* wd_dev, float wd_host, int cautious,
                               void* stream) {
   if (n < 0 || numel < 0 || cols <= 0) return fail(DION_E_INVALID, "dion_muon_post: bad size");
+  if (int rc = check_state_dtype("dion_muon_post", "x_dtype", x_dtype)) return rc;
   if (u_dtype != DION_BF16 && u_dtype != DION_F32) return fail(DION_E_INVALID, "dion_muon_post: u_dtype");
   if (n == 0 || numel == 0) return DION_OK;
   if (numel % cols) return fail(DION_E_INVALID, "dion_muon_post: numel %% cols != 0");
@@ -488,7 +497,8 @@ extern "C" int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype
     const int c = (n - i0) < kMaxPtrs ? (n - i0) : kMaxPtrs;
     PtrTab x;
     fill_tab(x, X_ptrs + i0, c);
-    HIP_TRY(launch_muon_post(x, (const char*)U + (size_t)i0 * numel * usz, u_dtype, c, numel, cols,
+    HIP_TRY(launch_muon_post(x, dt(x_dtype), (const char*)U + (size_t)i0 * numel * usz, dt(u_dtype), c, numel,
+                             cols,
                              row_scale ? row_scale + (int64_t)i0 * rows : nullptr, lr_dev, adj_ratio,
                              wd_dev, wd_host, cautious, vec, (hipStream_t)stream),
             "dion_muon_post");
@@ -496,9 +506,10 @@ extern "C" int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype
   return DION_OK;
 }
 
-static int normuon_stats_impl(const char* who, const void* U, const uint64_t* V_ptrs, int n,
+static int normuon_stats_impl(const char* who, const void* U, const uint64_t* V_ptrs, int v_dtype, int n,
                               int mats_per_ptr, int rows, int cols, const int32_t* row_idx, int v_rows,
                               float beta2, float* row_scale, void* stream) {
+  if (int rc = check_state_dtype(who, "v_dtype", v_dtype)) return rc;
   if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || v_rows < rows)
     return fail(DION_E_INVALID, "%s: bad size", who);
   if (n == 0 || rows == 0 || cols == 0) return DION_OK;
@@ -511,7 +522,7 @@ static int normuon_stats_impl(const char* who, const void* U, const uint64_t* V_
     PtrTab v;
     fill_tab(v, V_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
-    HIP_TRY(launch_normuon_stats((const bf16_t*)U + mat0 * rows * cols, v, c * mats_per_ptr, 0,
+    HIP_TRY(launch_normuon_stats((const bf16_t*)U + mat0 * rows * cols, v, dt(v_dtype), c * mats_per_ptr,
                                  mats_per_ptr, rows, cols, row_idx ? row_idx + mat0 * rows : nullptr,
                                  v_rows, w, row_scale + mat0 * rows, (hipStream_t)stream),
             who);
@@ -519,17 +530,18 @@ static int normuon_stats_impl(const char* who, const void* U, const uint64_t* V_
   return DION_OK;
 }
 
-extern "C" int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr,
-                                  int rows, int cols, float beta2, float* row_scale, void* stream) {
-  return normuon_stats_impl("dion_normuon_stats", U, V_ptrs, n, mats_per_ptr, rows, cols, nullptr, rows,
+extern "C" int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int v_dtype, int n,
+                                  int mats_per_ptr, int rows, int cols, float beta2, float* row_scale,
+                                  void* stream) {
+  return normuon_stats_impl("dion_normuon_stats", U, V_ptrs, v_dtype, n, mats_per_ptr, rows, cols, nullptr, rows,
                             beta2, row_scale, stream);
 }
 
-extern "C" int dion_normuon_stats_selected(const void* U, const uint64_t* V_ptrs, int n,
+extern "C" int dion_normuon_stats_selected(const void* U, const uint64_t* V_ptrs, int v_dtype, int n,
                                            int mats_per_ptr, int k, int cols, const int32_t* row_idx,
                                            int v_rows, float beta2, float* row_scale, void* stream) {
   if (!row_idx) return fail(DION_E_INVALID, "dion_normuon_stats_selected: null row_idx");
-  return normuon_stats_impl("dion_normuon_stats_selected", U, V_ptrs, n, mats_per_ptr, k, cols, row_idx,
+  return normuon_stats_impl("dion_normuon_stats_selected", U, V_ptrs, v_dtype, n, mats_per_ptr, k, cols, row_idx,
                             v_rows, beta2, row_scale, stream);
 }
 
@@ -546,10 +558,11 @@ extern "C" size_t dion_dion2_accumulate_scratch_bytes(int n_mat, int rows, int c
 }
 
 extern "C" int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs,
-                                     int n, int mats_per_ptr, int rows, int cols, int select_dim,
+                                     int m_dtype, int n, int mats_per_ptr, int rows, int cols, int select_dim,
                                      float* norms, void* scratch, size_t scratch_bytes,
                                      void* stream) {
   if (int rc = check_select_dim("dion_dion2_accumulate", select_dim)) return rc;
+  if (int rc = check_state_dtype("dion_dion2_accumulate", "m_dtype", m_dtype)) return rc;
   if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0)
     return fail(DION_E_INVALID, "dion_dion2_accumulate: bad size");
   if (g_dtype != DION_BF16 && g_dtype != DION_F32)
@@ -574,7 +587,7 @@ extern "C" int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const 
     PtrTab g, m;
     fill_tab(g, G_ptrs + i0, c);
     fill_tab(m, M_ptrs + i0, c);
-    HIP_TRY(launch_dion2_accumulate(g, g_dtype, m, c * mats_per_ptr, mats_per_ptr, rows, cols,
+    HIP_TRY(launch_dion2_accumulate(g, dt(g_dtype), m, dt(m_dtype), c * mats_per_ptr, mats_per_ptr, rows, cols,
                                     select_dim == -2, norms + (int64_t)i0 * mats_per_ptr * dim, vec4,
                                     slabs > 1 ? (float*)scratch : nullptr, slabs,
                                     (hipStream_t)stream),
@@ -597,10 +610,11 @@ extern "C" int dion_dion2_topk(const float* norms, int n_mat, int dim, int k, in
   return DION_OK;
 }
 
-extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr, int rows, int cols,
+extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int m_dtype, int n, int mats_per_ptr, int rows, int cols,
                                  int select_dim, const int32_t* idx, int k, float ef_decay,
                                  void* U_sel, void* stream) {
   if (int rc = check_select_dim("dion_dion2_gather", select_dim)) return rc;
+  if (int rc = check_state_dtype("dion_dion2_gather", "m_dtype", m_dtype)) return rc;
   if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || k < 0)
     return fail(DION_E_INVALID, "dion_dion2_gather: bad size");
   if (n == 0 || rows == 0 || cols == 0 || k == 0) return DION_OK;
@@ -614,7 +628,7 @@ extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr
     PtrTab m;
     fill_tab(m, M_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
-    HIP_TRY(launch_dion2_gather(m, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
+    HIP_TRY(launch_dion2_gather(m, dt(m_dtype), c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
                                 idx + mat0 * k, k, ef_decay, (bf16_t*)U_sel + mat0 * sel_numel, vec4,
                                 (hipStream_t)stream),
             "dion_dion2_gather");
@@ -622,11 +636,12 @@ extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr
   return DION_OK;
 }
 
-extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, int cols,
+extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int x_dtype, int n, int mats_per_ptr, int rows, int cols,
                                int select_dim, const void* U_sel, int u_dtype, int k, const int32_t* map,
                                const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
                                float adj_ratio, const float* wd_dev, float wd_host, void* stream) {
   if (int rc = check_select_dim("dion_dion2_post", select_dim)) return rc;
+  if (int rc = check_state_dtype("dion_dion2_post", "x_dtype", x_dtype)) return rc;
   if (u_dtype != DION_BF16 && u_dtype != DION_F32) return fail(DION_E_INVALID, "dion_dion2_post: u_dtype");
   if (row_scale && select_dim != -2)
     return fail(DION_E_INVALID, "dion_dion2_post: row_scale needs select_dim == -2");
@@ -647,7 +662,7 @@ extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, 
     PtrTab x;
     fill_tab(x, X_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
-    HIP_TRY(launch_dion2_post(x, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
+    HIP_TRY(launch_dion2_post(x, dt(x_dtype), c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
                               (const char*)U_sel + mat0 * sel_numel * es, u_dtype == DION_BF16 ? 0 : 1, k,
                               map + mat0 * dim, row_scale ? row_scale + mat0 * k : nullptr, lr_dev,
                               adj_lr_dev, adj_ratio, wd_dev, wd_host, vec4, (hipStream_t)stream),
@@ -725,12 +740,13 @@ extern "C" int dion_mask_index(const float* norms, int n_mat, int dim, int32_t* 
   return DION_OK;
 }
 
-extern "C" int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int n,
+extern "C" int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int s_dtype, int n,
                                       int mats_per_ptr, int rows, int cols, int select_dim,
                                       const void* U, const float* norms, const float* row_scale,
                                       const float* lr_dev, const float* adj_lr_dev, float adj_ratio,
                                       const float* wd_dev, float wd_host, float ef_decay, void* stream) {
   if (int rc = check_select_dim("dion_dion2_post_masked", select_dim)) return rc;
+  if (int rc = check_state_dtype("dion_dion2_post_masked", "s_dtype", s_dtype)) return rc;
   if (row_scale && select_dim != -2)
     return fail(DION_E_INVALID, "dion_dion2_post_masked: row_scale needs select_dim == -2");
   if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0)
@@ -752,7 +768,8 @@ extern "C" int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_
     fill_tab(x, X_ptrs + i0, c);
     fill_tab(m, M_ptrs + i0, c);
     const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
-    HIP_TRY(launch_dion2_post_masked(x, m, c * mats_per_ptr, mats_per_ptr, rows, cols, select_dim == -2,
+    HIP_TRY(launch_dion2_post_masked(x, m, dt(s_dtype), c * mats_per_ptr, mats_per_ptr, rows, cols,
+                                     select_dim == -2,
                                      (const bf16_t*)U + mat0 * rows * cols, norms + mat0 * dim,
                                      row_scale ? row_scale + mat0 * rows : nullptr, lr_dev, adj_lr_dev,
                                      adj_ratio, wd_dev, wd_host, ef_decay, vec4, (hipStream_t)stream),
@@ -777,10 +794,11 @@ static int check_mta(const char* who, const uint64_t* X, const uint64_t* G, int 
 }
 
 extern "C" int dion_adamw_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype,
-                               const uint64_t* M_ptrs, const uint64_t* V_ptrs,
+                               const uint64_t* M_ptrs, const uint64_t* V_ptrs, int s_dtype,
                                const uint64_t* step_ptrs, const int64_t* numels, int n,
                                const float* lr_dev, float beta1, float beta2, float eps,
                                const float* wd_dev, float wd_host, int cautious, void* stream) {
+  if (int rc = check_state_dtype("dion_adamw_step", "s_dtype", s_dtype)) return rc;
   if (int rc = check_mta("dion_adamw_step", X_ptrs, G_ptrs, g_dtype, M_ptrs, numels, n, lr_dev)) return rc;
   if (n == 0) return DION_OK;
   if (!V_ptrs || !step_ptrs) return fail(DION_E_INVALID, "dion_adamw_step: null argument");
@@ -798,7 +816,8 @@ extern "C" int dion_adamw_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, i
                       "dion_adamw_step: step counter of tensor %d is shared with tensor %d of an earlier "
                       "chunk of %d tensors",
                       i, j, kMtaTensors);
-    HIP_TRY(launch_adamw_mt(X_ptrs + i0, G_ptrs + i0, g_dtype, M_ptrs + i0, V_ptrs + i0, step_ptrs + i0,
+    HIP_TRY(launch_adamw_mt(X_ptrs + i0, G_ptrs + i0, dt(g_dtype), M_ptrs + i0, V_ptrs + i0, dt(s_dtype),
+                            step_ptrs + i0,
                             numels + i0, c, lr_dev, beta1, beta2, eps, wd_dev, wd_host, cautious,
                             (hipStream_t)stream),
             "dion_adamw_step");
@@ -807,13 +826,16 @@ extern "C" int dion_adamw_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, i
 }
 
 extern "C" int dion_lion_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype,
-                              const uint64_t* M_ptrs, const int64_t* numels, int n, const float* lr_dev,
+                              const uint64_t* M_ptrs, int s_dtype, const int64_t* numels, int n,
+                              const float* lr_dev,
                               float beta1, float beta2, const float* wd_dev, float wd_host, int cautious,
                               void* stream) {
+  if (int rc = check_state_dtype("dion_lion_step", "s_dtype", s_dtype)) return rc;
   if (int rc = check_mta("dion_lion_step", X_ptrs, G_ptrs, g_dtype, M_ptrs, numels, n, lr_dev)) return rc;
   for (int i0 = 0; i0 < n; i0 += kMtaTensors) {
     const int c = (n - i0) < kMtaTensors ? (n - i0) : kMtaTensors;
-    HIP_TRY(launch_lion_mt(X_ptrs + i0, G_ptrs + i0, g_dtype, M_ptrs + i0, numels + i0, c, lr_dev, beta1,
+    HIP_TRY(launch_lion_mt(X_ptrs + i0, G_ptrs + i0, dt(g_dtype), M_ptrs + i0, dt(s_dtype), numels + i0, c,
+                           lr_dev, beta1,
                            beta2, wd_dev, wd_host, cautious, (hipStream_t)stream),
             "dion_lion_step");
   }

@@ -32,6 +32,79 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
+// Optimizer state (parameters, momentum, second moments) lives in memory as fp32 or bf16.  All
+// arithmetic on it is fp32; a bf16 value is rounded once, when it is stored.  i4 / i8 index groups
+// of 4 / 8 consecutive elements (8- / 16-byte accesses for bf16, 16-byte pairs for fp32).
+template <typename T>
+__device__ __forceinline__ float st_load(const T* p, int64_t i) {
+  if constexpr (sizeof(T) == 2) return bf16_to_f32(p[i]);
+  else return p[i];
+}
+template <typename T>
+__device__ __forceinline__ void st_store(T* p, int64_t i, float v) {
+  if constexpr (sizeof(T) == 2) p[i] = f32_to_bf16(v);
+  else p[i] = v;
+}
+// The value a later load of the stored element returns.
+template <typename T>
+__device__ __forceinline__ float st_round(float v) {
+  if constexpr (sizeof(T) == 2) return bf16_to_f32(f32_to_bf16(v));
+  else return v;
+}
+template <typename T>
+__device__ __forceinline__ void st_load4(const T* p, int64_t i4, float v[4]) {
+  if constexpr (sizeof(T) == 2) {
+    const uint2 raw = ((const uint2*)p)[i4];
+    v[0] = __uint_as_float(raw.x << 16);
+    v[1] = __uint_as_float(raw.x & 0xffff0000u);
+    v[2] = __uint_as_float(raw.y << 16);
+    v[3] = __uint_as_float(raw.y & 0xffff0000u);
+  } else {
+    const float4 q = ((const float4*)p)[i4];
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  }
+}
+template <typename T>
+__device__ __forceinline__ void st_store4(T* p, int64_t i4, const float v[4]) {
+  if constexpr (sizeof(T) == 2) {
+    uint2 o;
+    o.x = pack_bf16x2(v[0], v[1]);
+    o.y = pack_bf16x2(v[2], v[3]);
+    ((uint2*)p)[i4] = o;
+  } else {
+    ((float4*)p)[i4] = make_float4(v[0], v[1], v[2], v[3]);
+  }
+}
+template <typename T>
+__device__ __forceinline__ void st_load8(const T* p, int64_t i8, float v[8]) {
+  if constexpr (sizeof(T) == 2) {
+    const uint4 raw = ((const uint4*)p)[i8];
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[2 * e] = __uint_as_float(w[e] << 16);
+      v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+    }
+  } else {
+    st_load4<T>(p, 2 * i8, v);
+    st_load4<T>(p, 2 * i8 + 1, v + 4);
+  }
+}
+template <typename T>
+__device__ __forceinline__ void st_store8(T* p, int64_t i8, const float v[8]) {
+  if constexpr (sizeof(T) == 2) {
+    uint4 o;
+    o.x = pack_bf16x2(v[0], v[1]);
+    o.y = pack_bf16x2(v[2], v[3]);
+    o.z = pack_bf16x2(v[4], v[5]);
+    o.w = pack_bf16x2(v[6], v[7]);
+    ((uint4*)p)[i8] = o;
+  } else {
+    st_store4<T>(p, 2 * i8, v);
+    st_store4<T>(p, 2 * i8 + 1, v + 4);
+  }
+}
+
 // Raises a kernel's dynamic-LDS limit once per device: the attribute belongs to the device that is
 // current when it is set, so `done` keeps one bit per device ordinal.
 static inline hipError_t set_max_dynamic_lds_once(const void* fn, int bytes, std::atomic<uint64_t>& done) {

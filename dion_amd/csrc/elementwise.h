@@ -32,16 +32,18 @@ hipError_t launch_ns_prepare(const void* in, int in_dtype, int batch, int R, int
                              hipStream_t st);
 hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* dst, int batch, int R,
                         int C, hipStream_t st);
-hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, bf16_t* U, int n,
+// State tensors (parameters X, momentum M, second moments V) are fp32 or bf16: *_dtype 0 = bf16,
+// 1 = fp32, like the gradient / update dtypes.
+hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, bf16_t* U, int n,
                            int64_t numel, float mu, int nesterov, bool vec, hipStream_t st);
-hipError_t launch_muon_post(const PtrTab& X, const void* U, int u_dtype, int n, int64_t numel,
+hipError_t launch_muon_post(const PtrTab& X, int x_dtype, const void* U, int u_dtype, int n, int64_t numel,
                             int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
                             const float* wd_dev, float wd_host, int cautious, bool vec,
                             hipStream_t st);
-hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int n_mat, int mat0,
-                                int mats_per_ptr, int rows, int cols, const int32_t* row_idx,
-                                int v_rows, float w, float* row_scale, hipStream_t st);
-hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int n_mat,
+hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int v_dtype, int n_mat, int mats_per_ptr,
+                                int rows, int cols, const int32_t* row_idx, int v_rows, float w,
+                                float* row_scale, hipStream_t st);
+hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, int n_mat,
                                    int mats_per_ptr, int rows, int cols, int select_rows,
                                    float* norms, bool vec4, float* slab_scratch, int slabs,
                                    hipStream_t st);
@@ -49,10 +51,10 @@ hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M
 int dion2_acc_slabs(int n_mat, int rows, int cols);
 hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
                              int32_t* map, hipStream_t st);
-hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int rows, int cols,
+hipError_t launch_dion2_gather(const PtrTab& M, int m_dtype, int n_mat, int mats_per_ptr, int rows, int cols,
                                int select_rows, const int32_t* idx, int k, float ef_decay, bf16_t* U,
                                bool vec4, hipStream_t st);
-hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
+hipError_t launch_dion2_post(const PtrTab& X, int x_dtype, int n_mat, int mats_per_ptr, int rows, int cols,
                              int select_rows, const void* U, int u_dtype, int k, const int32_t* map,
                              const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
                              float adj_ratio, const float* wd_dev, float wd_host, bool vec4,
@@ -70,7 +72,7 @@ hipError_t launch_gather_slices(const void* U, int dtype, int n_mat, int rows, i
 hipError_t launch_scatter_slices(const void* sub, int dtype, int n_mat, int rows, int cols,
                                  int select_rows, const int32_t* map, int k, void* out, hipStream_t st);
 hipError_t launch_mask_index(const float* norms, int n_mat, int dim, int32_t* gate, hipStream_t st);
-hipError_t launch_dion2_post_masked(const PtrTab& X, const PtrTab& M, int n_mat, int mats_per_ptr,
+hipError_t launch_dion2_post_masked(const PtrTab& X, const PtrTab& M, int s_dtype, int n_mat, int mats_per_ptr,
                                     int rows, int cols, int select_rows, const bf16_t* U,
                                     const float* norms, const float* row_scale, const float* lr_dev,
                                     const float* adj_lr_dev, float adj_ratio, const float* wd_dev,
@@ -80,10 +82,10 @@ hipError_t launch_dion2_post_masked(const PtrTab& X, const PtrTab& M, int n_mat,
 // device pointers and element counts.
 constexpr int kMtaTensors = 48;
 hipError_t launch_adamw_mt(const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M,
-                           const uint64_t* V, const uint64_t* steps, const int64_t* numel, int n,
+                           const uint64_t* V, int s_dtype, const uint64_t* steps, const int64_t* numel, int n,
                            const float* lr_dev, float beta1, float beta2, float eps, const float* wd_dev,
                            float wd_host, int cautious, hipStream_t st);
-hipError_t launch_lion_mt(const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M,
+hipError_t launch_lion_mt(const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M, int s_dtype,
                           const int64_t* numel, int n, const float* lr_dev, float beta1, float beta2,
                           const float* wd_dev, float wd_host, int cautious, hipStream_t st);
 

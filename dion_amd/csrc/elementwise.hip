@@ -247,79 +247,45 @@ hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* d
 // ------------------------------------------------------------------------------------------
 // Muon pre: momentum + Nesterov + bf16 cast, list-of-parameters in, one arena out.
 // ------------------------------------------------------------------------------------------
-template <typename GT, bool VEC>
+template <typename GT, typename MT, bool VEC>
 __global__ __launch_bounds__(256) void muon_pre_kernel(PtrTab G, PtrTab M, bf16_t* __restrict__ U,
                                                        int64_t numel, float mu, int nesterov) {
   const int p = blockIdx.y;
   const GT* __restrict__ g = (const GT*)G.p[p];
-  float* __restrict__ m = (float*)M.p[p];
+  MT* __restrict__ m = (MT*)M.p[p];
   bf16_t* __restrict__ u = U + (int64_t)p * numel;
   const int64_t stride = (int64_t)gridDim.x * 256;
   if (VEC) {
-    // Two 8-element chunks per thread per trip, all loads issued before the arithmetic: 96 bytes
-    // of reads in flight per lane.
+    // Two 8-element chunks per thread per trip, all loads issued before the arithmetic: up to 96
+    // bytes of reads in flight per lane.
     const int64_t nv = numel >> 3;
     for (int64_t i0 = (int64_t)blockIdx.x * 256 + threadIdx.x; i0 < nv; i0 += 2 * stride) {
       const int64_t i1 = i0 + stride;
       const bool has1 = i1 < nv;
-      uint4 graw[2];
-      float4 gf[2][2], mf[2][2];
-      if (sizeof(GT) == 2) {
-        graw[0] = ((const uint4*)g)[i0];
-        if (has1) graw[1] = ((const uint4*)g)[i1];
-      } else {
-        gf[0][0] = ((const float4*)g)[2 * i0];
-        gf[0][1] = ((const float4*)g)[2 * i0 + 1];
-        if (has1) {
-          gf[1][0] = ((const float4*)g)[2 * i1];
-          gf[1][1] = ((const float4*)g)[2 * i1 + 1];
-        }
-      }
-      mf[0][0] = ((const float4*)m)[2 * i0];
-      mf[0][1] = ((const float4*)m)[2 * i0 + 1];
-      if (has1) {
-        mf[1][0] = ((const float4*)m)[2 * i1];
-        mf[1][1] = ((const float4*)m)[2 * i1 + 1];
-      }
+      float gv[2][8], mv[2][8];
+      st_load8<GT>(g, i0, gv[0]);
+      if (has1) st_load8<GT>(g, i1, gv[1]);
+      st_load8<MT>(m, i0, mv[0]);
+      if (has1) st_load8<MT>(m, i1, mv[1]);
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         if (c == 1 && !has1) break;
         const int64_t i = c == 0 ? i0 : i1;
-        float gv[8];
-        if (sizeof(GT) == 2) {
-          const uint32_t w[4] = {graw[c].x, graw[c].y, graw[c].z, graw[c].w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            gv[2 * e] = __uint_as_float(w[e] << 16);
-            gv[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
-          }
-        } else {
-          gv[0] = gf[c][0].x; gv[1] = gf[c][0].y; gv[2] = gf[c][0].z; gv[3] = gf[c][0].w;
-          gv[4] = gf[c][1].x; gv[5] = gf[c][1].y; gv[6] = gf[c][1].z; gv[7] = gf[c][1].w;
-        }
-        float mv[8] = {mf[c][0].x, mf[c][0].y, mf[c][0].z, mf[c][0].w,
-                       mf[c][1].x, mf[c][1].y, mf[c][1].z, mf[c][1].w};
         float uv[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          mv[e] = __fadd_rn(__fmul_rn(mv[e], mu), gv[e]);
-          uv[e] = nesterov ? __fadd_rn(__fmul_rn(mv[e], mu), gv[e]) : mv[e];
+          mv[c][e] = __fadd_rn(__fmul_rn(mv[c][e], mu), gv[c][e]);
+          uv[e] = nesterov ? __fadd_rn(__fmul_rn(mv[c][e], mu), gv[c][e]) : mv[c][e];
         }
-        ((float4*)m)[2 * i] = make_float4(mv[0], mv[1], mv[2], mv[3]);
-        ((float4*)m)[2 * i + 1] = make_float4(mv[4], mv[5], mv[6], mv[7]);
-        uint4 o;
-        o.x = pack_bf16x2(uv[0], uv[1]);
-        o.y = pack_bf16x2(uv[2], uv[3]);
-        o.z = pack_bf16x2(uv[4], uv[5]);
-        o.w = pack_bf16x2(uv[6], uv[7]);
-        ((uint4*)u)[i] = o;
+        st_store8<MT>(m, i, mv[c]);
+        st_store8<bf16_t>(u, i, uv);
       }
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
-      const float gv = sizeof(GT) == 2 ? bf16_to_f32(((const bf16_t*)g)[i]) : ((const float*)g)[i];
-      const float mv = __fadd_rn(__fmul_rn(m[i], mu), gv);
-      m[i] = mv;
+      const float gv = st_load<GT>(g, i);
+      const float mv = __fadd_rn(__fmul_rn(st_load<MT>(m, i), mu), gv);
+      st_store<MT>(m, i, mv);
       u[i] = f32_to_bf16(nesterov ? __fadd_rn(__fmul_rn(mv, mu), gv) : mv);
     }
   }
@@ -332,25 +298,20 @@ static int ew_blocks(int64_t work_items) {
   return (int)b;
 }
 
-hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, bf16_t* U, int n,
+hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, bf16_t* U, int n,
                            int64_t numel, float mu, int nesterov, bool vec, hipStream_t st) {
-  if (vec) {
-    dim3 grid(ew_blocks(numel >> 3), n);
-    if (g_dtype == 0)
-      hipLaunchKernelGGL((muon_pre_kernel<bf16_t, true>), grid, dim3(256), 0, st, G, M, U, numel, mu,
-                         nesterov);
-    else
-      hipLaunchKernelGGL((muon_pre_kernel<float, true>), grid, dim3(256), 0, st, G, M, U, numel, mu,
-                         nesterov);
+  dim3 grid(ew_blocks(vec ? (numel >> 3) : numel), n);
+#define PRE_LAUNCH(GT, MT, V) \
+  hipLaunchKernelGGL((muon_pre_kernel<GT, MT, V>), grid, dim3(256), 0, st, G, M, U, numel, mu, nesterov)
+#define PRE_LAUNCH_M(GT, V) \
+  do { if (m_dtype == 0) PRE_LAUNCH(GT, bf16_t, V); else PRE_LAUNCH(GT, float, V); } while (0)
+  if (g_dtype == 0) {
+    if (vec) PRE_LAUNCH_M(bf16_t, true); else PRE_LAUNCH_M(bf16_t, false);
   } else {
-    dim3 grid(ew_blocks(numel), n);
-    if (g_dtype == 0)
-      hipLaunchKernelGGL((muon_pre_kernel<bf16_t, false>), grid, dim3(256), 0, st, G, M, U, numel, mu,
-                         nesterov);
-    else
-      hipLaunchKernelGGL((muon_pre_kernel<float, false>), grid, dim3(256), 0, st, G, M, U, numel, mu,
-                         nesterov);
+    if (vec) PRE_LAUNCH_M(float, true); else PRE_LAUNCH_M(float, false);
   }
+#undef PRE_LAUNCH_M
+#undef PRE_LAUNCH
   return hipGetLastError();
 }
 
@@ -369,7 +330,7 @@ static __device__ __forceinline__ float post_one(float x, float u, float a, floa
   return __fsub_rn(x, __fmul_rn(u, b));
 }
 
-template <typename UT, bool VEC>
+template <typename UT, typename XT, bool VEC>
 __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __restrict__ U,
                                                         int64_t numel, int cols,
                                                         const float* __restrict__ row_scale,
@@ -378,7 +339,7 @@ __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __re
                                                         const float* __restrict__ wd_dev,
                                                         float wd_host, int cautious) {
   const int p = blockIdx.y;
-  float* __restrict__ x = (float*)X.p[p];
+  XT* __restrict__ x = (XT*)X.p[p];
   const UT* __restrict__ u = U + (int64_t)p * numel;
   const float lr = *lr_dev;
   const float wd = wd_dev ? *wd_dev : wd_host;
@@ -391,54 +352,43 @@ __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __re
   if (VEC) {
     const int64_t nv = numel >> 3;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nv; i += stride) {
-      float uv[8];
-      if (sizeof(UT) == 2) {
-        const uint4 raw = ((const uint4*)u)[i];
-        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          uv[2 * e] = __uint_as_float(w[e] << 16);
-          uv[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
-        }
-      } else {
-        const float4 q0 = ((const float4*)u)[2 * i], q1 = ((const float4*)u)[2 * i + 1];
-        uv[0] = q0.x; uv[1] = q0.y; uv[2] = q0.z; uv[3] = q0.w;
-        uv[4] = q1.x; uv[5] = q1.y; uv[6] = q1.z; uv[7] = q1.w;
-      }
+      float uv[8], xv[8];
+      st_load8<UT>(u, i, uv);
       if (rs) {  // cols % 8 == 0 on this path, so the 8 elements share a row
         const float s = rs[(i << 3) / cols];
 #pragma unroll
         for (int e = 0; e < 8; ++e) uv[e] = __fmul_rn(uv[e], s);
       }
-      float4 x0 = ((float4*)x)[2 * i], x1 = ((float4*)x)[2 * i + 1];
-      float xv[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+      st_load8<XT>(x, i, xv);
 #pragma unroll
       for (int e = 0; e < 8; ++e) xv[e] = post_one(xv[e], uv[e], a, coeff, b, cautious);
-      ((float4*)x)[2 * i] = make_float4(xv[0], xv[1], xv[2], xv[3]);
-      ((float4*)x)[2 * i + 1] = make_float4(xv[4], xv[5], xv[6], xv[7]);
+      st_store8<XT>(x, i, xv);
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
-      float uv = sizeof(UT) == 2 ? bf16_to_f32(((const bf16_t*)u)[i]) : ((const float*)u)[i];
+      float uv = st_load<UT>(u, i);
       if (rs) uv = __fmul_rn(uv, rs[i / cols]);
-      x[i] = post_one(x[i], uv, a, coeff, b, cautious);
+      st_store<XT>(x, i, post_one(st_load<XT>(x, i), uv, a, coeff, b, cautious));
     }
   }
 }
 
-hipError_t launch_muon_post(const PtrTab& X, const void* U, int u_dtype, int n, int64_t numel,
+hipError_t launch_muon_post(const PtrTab& X, int x_dtype, const void* U, int u_dtype, int n, int64_t numel,
                             int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
                             const float* wd_dev, float wd_host, int cautious, bool vec,
                             hipStream_t st) {
   dim3 grid(ew_blocks(vec ? (numel >> 3) : numel), n);
-#define POST_LAUNCH(UT, V)                                                                        \
-  hipLaunchKernelGGL((muon_post_kernel<UT, V>), grid, dim3(256), 0, st, X, (const UT*)U, numel,   \
+#define POST_LAUNCH(UT, XT, V)                                                                      \
+  hipLaunchKernelGGL((muon_post_kernel<UT, XT, V>), grid, dim3(256), 0, st, X, (const UT*)U, numel, \
                      cols, row_scale, lr_dev, adj_ratio, wd_dev, wd_host, cautious)
+#define POST_LAUNCH_X(UT, V) \
+  do { if (x_dtype == 0) POST_LAUNCH(UT, bf16_t, V); else POST_LAUNCH(UT, float, V); } while (0)
   if (u_dtype == 0) {
-    if (vec) POST_LAUNCH(bf16_t, true); else POST_LAUNCH(bf16_t, false);
+    if (vec) POST_LAUNCH_X(bf16_t, true); else POST_LAUNCH_X(bf16_t, false);
   } else {
-    if (vec) POST_LAUNCH(float, true); else POST_LAUNCH(float, false);
+    if (vec) POST_LAUNCH_X(float, true); else POST_LAUNCH_X(float, false);
   }
+#undef POST_LAUNCH_X
 #undef POST_LAUNCH
   return hipGetLastError();
 }
@@ -452,6 +402,7 @@ hipError_t launch_muon_post(const PtrTab& X, const void* U, int u_dtype, int n, 
 // that is not part of the update (an all-zero row of a masked full-size tensor,
 // dion/nordion2.py:485-497): its second moment is left alone and its scale is 0.
 // Pass 1: one wavefront per row.  V <- lerp(V, mean(u^2), w);  tmp[row] = sum(u^2).
+template <typename VT>
 __global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restrict__ U, PtrTab V,
                                                            int mats_per_ptr, int rows, int cols,
                                                            const int32_t* __restrict__ row_idx,
@@ -484,10 +435,10 @@ __global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restr
   if (lane == 0) {
     const int vr = row_idx ? row_idx[(int64_t)mat * rows + row] : row;
     if (vr >= 0) {
-      float* v = (float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * v_rows + vr;
+      VT* v = (VT*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * v_rows + vr;
       const float mean = s / (float)cols;
-      const float vo = *v;
-      *v = vo + w * (mean - vo);  // torch.lerp for weight < 0.5
+      const float vo = st_load<VT>(v, 0);
+      st_store<VT>(v, 0, vo + w * (mean - vo));  // torch.lerp for weight < 0.5
     }
     rowsq[(int64_t)mat * rows + row] = vr >= 0 ? s : 0.f;
   }
@@ -495,19 +446,20 @@ __global__ __launch_bounds__(256) void normuon_rows_kernel(const bf16_t* __restr
 
 // Pass 2: one block per matrix.  scale[row] = (1/d) * sqrt(S1) / max(sqrt(S2), 1e-8) with
 // d = sqrt(V)+1e-8, S1 = sum rowsq, S2 = sum rowsq/d^2.  In place over rowsq.
+template <typename VT>
 __global__ __launch_bounds__(1024) void normuon_scale_kernel(PtrTab V, int mats_per_ptr, int rows,
                                                              const int32_t* __restrict__ row_idx,
                                                              int v_rows, float* __restrict__ scale) {
   __shared__ float red[16];
   const int mat = blockIdx.x;
-  const float* v = (const float*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * v_rows;
+  const VT* v = (const VT*)V.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * v_rows;
   const int32_t* ri = row_idx ? row_idx + (int64_t)mat * rows : nullptr;
   float* sc = scale + (int64_t)mat * rows;
   float s1 = 0.f, s2 = 0.f;
   for (int r = threadIdx.x; r < rows; r += 1024) {
     const float q = sc[r];
     const int vr = ri ? ri[r] : r;
-    const float inv = vr >= 0 ? 1.0f / (sqrtf(v[vr]) + 1e-8f) : 0.f;
+    const float inv = vr >= 0 ? 1.0f / (sqrtf(st_load<VT>(v, vr)) + 1e-8f) : 0.f;
     s1 += q;
     s2 += q * inv * inv;
   }
@@ -517,20 +469,26 @@ __global__ __launch_bounds__(1024) void normuon_scale_kernel(PtrTab V, int mats_
   __syncthreads();
   for (int r = threadIdx.x; r < rows; r += 1024) {
     const int vr = ri ? ri[r] : r;
-    sc[r] = vr >= 0 ? (1.0f / (sqrtf(v[vr]) + 1e-8f)) * ratio : 0.f;
+    sc[r] = vr >= 0 ? (1.0f / (sqrtf(st_load<VT>(v, vr)) + 1e-8f)) * ratio : 0.f;
   }
 }
 
-hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int n_mat, int mat0,
-                                int mats_per_ptr, int rows, int cols, const int32_t* row_idx,
-                                int v_rows, float w, float* row_scale, hipStream_t st) {
-  // U / row_scale / row_idx are offset to matrix mat0 by the caller; V is the table chunk covering
-  // them.
-  (void)mat0;
-  hipLaunchKernelGGL(normuon_rows_kernel, dim3((rows + 3) / 4, n_mat), dim3(256), 0, st, U, V,
-                     mats_per_ptr, rows, cols, row_idx, v_rows, w, row_scale);
-  hipLaunchKernelGGL(normuon_scale_kernel, dim3(n_mat), dim3(1024), 0, st, V, mats_per_ptr, rows,
-                     row_idx, v_rows, row_scale);
+hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int v_dtype, int n_mat, int mats_per_ptr,
+                                int rows, int cols, const int32_t* row_idx, int v_rows, float w,
+                                float* row_scale, hipStream_t st) {
+  // U / row_scale / row_idx are offset to the first matrix by the caller; V is the table chunk
+  // covering them.
+  if (v_dtype == 0) {
+    hipLaunchKernelGGL(normuon_rows_kernel<bf16_t>, dim3((rows + 3) / 4, n_mat), dim3(256), 0, st, U, V,
+                       mats_per_ptr, rows, cols, row_idx, v_rows, w, row_scale);
+    hipLaunchKernelGGL(normuon_scale_kernel<bf16_t>, dim3(n_mat), dim3(1024), 0, st, V, mats_per_ptr, rows,
+                       row_idx, v_rows, row_scale);
+  } else {
+    hipLaunchKernelGGL(normuon_rows_kernel<float>, dim3((rows + 3) / 4, n_mat), dim3(256), 0, st, U, V,
+                       mats_per_ptr, rows, cols, row_idx, v_rows, w, row_scale);
+    hipLaunchKernelGGL(normuon_scale_kernel<float>, dim3(n_mat), dim3(1024), 0, st, V, mats_per_ptr, rows,
+                       row_idx, v_rows, row_scale);
+  }
   return hipGetLastError();
 }
 
@@ -542,8 +500,8 @@ static __device__ __forceinline__ float g_load(const GT* g, int64_t i) {
   return sizeof(GT) == 2 ? bf16_to_f32(((const bf16_t*)g)[i]) : ((const float*)g)[i];
 }
 
-// select rows: one wavefront per row, norms[mat][row] = sum_j |M+G|.
-template <typename GT>
+// select rows: one wavefront per row, norms[mat][row] = sum_j |M+G| (of the values as stored).
+template <typename GT, typename MT>
 __global__ __launch_bounds__(256) void dion2_acc_rows_kernel(PtrTab G, PtrTab M, int mats_per_ptr,
                                                              int rows, int cols,
                                                              float* __restrict__ norms) {
@@ -553,11 +511,11 @@ __global__ __launch_bounds__(256) void dion2_acc_rows_kernel(PtrTab G, PtrTab M,
   const int lane = threadIdx.x & 63;
   const int64_t base = ((int64_t)(mat % mats_per_ptr) * rows + row) * cols;
   const GT* g = (const GT*)G.p[mat / mats_per_ptr] + base;
-  float* m = (float*)M.p[mat / mats_per_ptr] + base;
+  MT* m = (MT*)M.p[mat / mats_per_ptr] + base;
   float s = 0.f;
   for (int c = lane; c < cols; c += 64) {
-    const float v = __fadd_rn(m[c], g_load<GT>(g, c));
-    m[c] = v;
+    const float v = st_round<MT>(__fadd_rn(st_load<MT>(m, c), g_load<GT>(g, c)));
+    st_store<MT>(m, c, v);
     s += fabsf(v);
   }
   s = wave_sum(s);
@@ -565,7 +523,7 @@ __global__ __launch_bounds__(256) void dion2_acc_rows_kernel(PtrTab G, PtrTab M,
 }
 
 // select columns: each block owns 64 columns of one matrix and walks all rows (4 rows at a time).
-template <typename GT>
+template <typename GT, typename MT>
 __global__ __launch_bounds__(256) void dion2_acc_cols_kernel(PtrTab G, PtrTab M, int mats_per_ptr,
                                                              int rows, int cols,
                                                              float* __restrict__ norms) {
@@ -575,13 +533,13 @@ __global__ __launch_bounds__(256) void dion2_acc_cols_kernel(PtrTab G, PtrTab M,
   const int ry = threadIdx.x >> 6;
   const int64_t base = (int64_t)(mat % mats_per_ptr) * rows * cols;
   const GT* g = (const GT*)G.p[mat / mats_per_ptr] + base;
-  float* m = (float*)M.p[mat / mats_per_ptr] + base;
+  MT* m = (MT*)M.p[mat / mats_per_ptr] + base;
   float s = 0.f;
   if (c < cols) {
     for (int r = ry; r < rows; r += 4) {
       const int64_t i = (int64_t)r * cols + c;
-      const float v = __fadd_rn(m[i], g_load<GT>(g, i));
-      m[i] = v;
+      const float v = st_round<MT>(__fadd_rn(st_load<MT>(m, i), g_load<GT>(g, i)));
+      st_store<MT>(m, i, v);
       s += fabsf(v);
     }
   }
@@ -592,10 +550,10 @@ __global__ __launch_bounds__(256) void dion2_acc_cols_kernel(PtrTab G, PtrTab M,
                                      (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
-// 4 columns per thread (16-byte accesses): each block owns 256 columns, four row lanes.
+// 4 columns per thread (8- / 16-byte accesses): each block owns 256 columns, four row lanes.
 // With gridDim.z row slabs the block writes its slab's partial sums to out[(slab*n_mat + mat)*cols]
 // (n_mat = gridDim.y); dion2_sum_slabs_kernel adds the slabs in a fixed order.
-template <typename GT>
+template <typename GT, typename MT>
 __global__ __launch_bounds__(256) void dion2_acc_cols_vec_kernel(PtrTab G, PtrTab M, int mats_per_ptr,
                                                                  int rows, int cols, int slab_rows,
                                                                  float* __restrict__ norms) {
@@ -608,32 +566,22 @@ __global__ __launch_bounds__(256) void dion2_acc_cols_vec_kernel(PtrTab G, PtrTa
   const int ry = threadIdx.x >> 6;
   const int64_t base = (int64_t)(mat % mats_per_ptr) * rows * cols;
   const GT* g = (const GT*)G.p[mat / mats_per_ptr] + base;
-  float* m = (float*)M.p[mat / mats_per_ptr] + base;
+  MT* m = (MT*)M.p[mat / mats_per_ptr] + base;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
   if (c < cols) {
 #pragma unroll 4
     for (int r = r0 + ry; r < r1; r += 4) {
-      const int64_t i = (int64_t)r * cols + c;
-      float4 gv;
-      if (sizeof(GT) == 2) {
-        const uint2 raw = *(const uint2*)((const bf16_t*)g + i);
-        gv.x = __uint_as_float(raw.x << 16);
-        gv.y = __uint_as_float(raw.x & 0xffff0000u);
-        gv.z = __uint_as_float(raw.y << 16);
-        gv.w = __uint_as_float(raw.y & 0xffff0000u);
-      } else {
-        gv = *(const float4*)((const float*)g + i);
-      }
-      float4 mv = *(const float4*)(m + i);
-      mv.x = __fadd_rn(mv.x, gv.x);
-      mv.y = __fadd_rn(mv.y, gv.y);
-      mv.z = __fadd_rn(mv.z, gv.z);
-      mv.w = __fadd_rn(mv.w, gv.w);
-      *(float4*)(m + i) = mv;
-      s.x += fabsf(mv.x);
-      s.y += fabsf(mv.y);
-      s.z += fabsf(mv.z);
-      s.w += fabsf(mv.w);
+      const int64_t i4 = ((int64_t)r * cols + c) >> 2;  // cols % 4 == 0 on this path
+      float gv[4], mv[4];
+      st_load4<GT>(g, i4, gv);
+      st_load4<MT>(m, i4, mv);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) mv[e] = st_round<MT>(__fadd_rn(mv[e], gv[e]));
+      st_store4<MT>(m, i4, mv);
+      s.x += fabsf(mv[0]);
+      s.y += fabsf(mv[1]);
+      s.z += fabsf(mv[2]);
+      s.w += fabsf(mv[3]);
     }
   }
   red[ry][threadIdx.x & 63] = s;
@@ -668,30 +616,32 @@ int dion2_acc_slabs(int n_mat, int rows, int cols) {
   return s < 1 ? 1 : (int)s;
 }
 
-hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int n_mat,
+hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, int n_mat,
                                    int mats_per_ptr, int rows, int cols, int select_rows,
                                    float* norms, bool vec4, float* slab_scratch, int slabs,
                                    hipStream_t st) {
+  // DISPATCH(kernel, grid, args...): the four (gradient, momentum) dtype pairs
+#define ACC_LAUNCH(K, GRID, ...)                                                                        \
+  do {                                                                                                  \
+    if (g_dtype == 0 && m_dtype == 0)                                                                   \
+      hipLaunchKernelGGL((K<bf16_t, bf16_t>), GRID, dim3(256), 0, st, __VA_ARGS__);                      \
+    else if (g_dtype == 0)                                                                              \
+      hipLaunchKernelGGL((K<bf16_t, float>), GRID, dim3(256), 0, st, __VA_ARGS__);                       \
+    else if (m_dtype == 0)                                                                              \
+      hipLaunchKernelGGL((K<float, bf16_t>), GRID, dim3(256), 0, st, __VA_ARGS__);                       \
+    else                                                                                                \
+      hipLaunchKernelGGL((K<float, float>), GRID, dim3(256), 0, st, __VA_ARGS__);                        \
+  } while (0)
   if (select_rows) {
     dim3 grid((rows + 3) / 4, n_mat);
-    if (g_dtype == 0)
-      hipLaunchKernelGGL(dion2_acc_rows_kernel<bf16_t>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
-                         rows, cols, norms);
-    else
-      hipLaunchKernelGGL(dion2_acc_rows_kernel<float>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
-                         rows, cols, norms);
+    ACC_LAUNCH(dion2_acc_rows_kernel, grid, G, M, mats_per_ptr, rows, cols, norms);
   } else if (vec4) {
     if (!slab_scratch) slabs = 1;
     const int slab_rows = ((rows + slabs - 1) / slabs + 3) / 4 * 4;
     slabs = (rows + slab_rows - 1) / slab_rows;
     float* dst = slabs > 1 ? slab_scratch : norms;
     dim3 grid((cols / 4 + 63) / 64, n_mat, slabs);
-    if (g_dtype == 0)
-      hipLaunchKernelGGL(dion2_acc_cols_vec_kernel<bf16_t>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
-                         rows, cols, slab_rows, dst);
-    else
-      hipLaunchKernelGGL(dion2_acc_cols_vec_kernel<float>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
-                         rows, cols, slab_rows, dst);
+    ACC_LAUNCH(dion2_acc_cols_vec_kernel, grid, G, M, mats_per_ptr, rows, cols, slab_rows, dst);
     if (slabs > 1) {
       const int64_t n = (int64_t)n_mat * cols;
       hipLaunchKernelGGL(dion2_sum_slabs_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
@@ -699,13 +649,9 @@ hipError_t launch_dion2_accumulate(const PtrTab& G, int g_dtype, const PtrTab& M
     }
   } else {
     dim3 grid((cols + 63) / 64, n_mat);
-    if (g_dtype == 0)
-      hipLaunchKernelGGL(dion2_acc_cols_kernel<bf16_t>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
-                         rows, cols, norms);
-    else
-      hipLaunchKernelGGL(dion2_acc_cols_kernel<float>, grid, dim3(256), 0, st, G, M, mats_per_ptr,
-                         rows, cols, norms);
+    ACC_LAUNCH(dion2_acc_cols_kernel, grid, G, M, mats_per_ptr, rows, cols, norms);
   }
+#undef ACC_LAUNCH
   return hipGetLastError();
 }
 
@@ -807,61 +753,60 @@ hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int3
 // U_sel = bf16(M[sel]); M[sel] *= ef_decay.
 // rows selected: block (j, mat) copies row idx[j]; columns selected: block (row, mat) gathers the k
 // selected columns (ascending, so the reads walk the row forwards).
-template <bool VEC>
+template <typename MT, bool VEC>
 __global__ __launch_bounds__(256) void dion2_gather_kernel(PtrTab M, int mats_per_ptr, int rows,
                                                            int cols, int select_rows,
                                                            const int32_t* __restrict__ idx, int k,
                                                            float ef_decay, bf16_t* __restrict__ U) {
   const int mat = blockIdx.y;
-  float* m = (float*)M.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
+  MT* m = (MT*)M.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
   const int32_t* id = idx + (int64_t)mat * k;
   if (select_rows) {
     const int j = blockIdx.x;
-    float* src = m + (int64_t)id[j] * cols;
+    MT* src = m + (int64_t)id[j] * cols;
     bf16_t* u = U + ((int64_t)mat * k + j) * cols;
     if (VEC) {
-      for (int c = threadIdx.x * 4; c < cols; c += 1024) {
-        float4 v = *(const float4*)(src + c);
-        uint2 o;
-        o.x = pack_bf16x2(v.x, v.y);
-        o.y = pack_bf16x2(v.z, v.w);
-        *(uint2*)(u + c) = o;
-        v.x = __fmul_rn(v.x, ef_decay);
-        v.y = __fmul_rn(v.y, ef_decay);
-        v.z = __fmul_rn(v.z, ef_decay);
-        v.w = __fmul_rn(v.w, ef_decay);
-        *(float4*)(src + c) = v;
+      for (int c4 = threadIdx.x; c4 < cols / 4; c4 += 256) {
+        float v[4];
+        st_load4<MT>(src, c4, v);
+        st_store4<bf16_t>(u, c4, v);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], ef_decay);
+        st_store4<MT>(src, c4, v);
       }
     } else {
       for (int c = threadIdx.x; c < cols; c += 256) {
-        const float v = src[c];
+        const float v = st_load<MT>(src, c);
         u[c] = f32_to_bf16(v);
-        src[c] = __fmul_rn(v, ef_decay);
+        st_store<MT>(src, c, __fmul_rn(v, ef_decay));
       }
     }
   } else {
     const int r = blockIdx.x;
-    float* src = m + (int64_t)r * cols;
+    MT* src = m + (int64_t)r * cols;
     bf16_t* u = U + ((int64_t)mat * rows + r) * k;
     for (int j = threadIdx.x; j < k; j += 256) {
       const int c = id[j];
-      const float v = src[c];
+      const float v = st_load<MT>(src, c);
       u[j] = f32_to_bf16(v);
-      src[c] = __fmul_rn(v, ef_decay);
+      st_store<MT>(src, c, __fmul_rn(v, ef_decay));
     }
   }
 }
 
-hipError_t launch_dion2_gather(const PtrTab& M, int n_mat, int mats_per_ptr, int rows, int cols,
+hipError_t launch_dion2_gather(const PtrTab& M, int m_dtype, int n_mat, int mats_per_ptr, int rows, int cols,
                                int select_rows, const int32_t* idx, int k, float ef_decay, bf16_t* U,
                                bool vec4, hipStream_t st) {
   dim3 grid(select_rows ? k : rows, n_mat);
-  if (vec4)
-    hipLaunchKernelGGL(dion2_gather_kernel<true>, grid, dim3(256), 0, st, M, mats_per_ptr, rows, cols,
-                       select_rows, idx, k, ef_decay, U);
-  else
-    hipLaunchKernelGGL(dion2_gather_kernel<false>, grid, dim3(256), 0, st, M, mats_per_ptr, rows, cols,
-                       select_rows, idx, k, ef_decay, U);
+#define GATHER_LAUNCH(MT, V)                                                                          \
+  hipLaunchKernelGGL((dion2_gather_kernel<MT, V>), grid, dim3(256), 0, st, M, mats_per_ptr, rows, cols, \
+                     select_rows, idx, k, ef_decay, U)
+  if (m_dtype == 0) {
+    if (vec4) GATHER_LAUNCH(bf16_t, true); else GATHER_LAUNCH(bf16_t, false);
+  } else {
+    if (vec4) GATHER_LAUNCH(float, true); else GATHER_LAUNCH(float, false);
+  }
+#undef GATHER_LAUNCH
   return hipGetLastError();
 }
 
@@ -881,7 +826,7 @@ static __device__ __forceinline__ float4 u_load4(const UT* u, int64_t i) {
   return *(const float4*)((const float*)u + i);
 }
 
-template <bool VEC, typename UT>
+template <bool VEC, typename UT, typename XT>
 __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_ptr, int rows,
                                                          int cols, int select_rows,
                                                          const UT* __restrict__ U, int k,
@@ -893,7 +838,7 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
                                                          const float* __restrict__ wd_dev,
                                                          float wd_host) {
   const int mat = blockIdx.y;
-  float* x = (float*)X.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
+  XT* x = (XT*)X.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
   const float lr = *lr_dev;
   const float wd = wd_dev ? *wd_dev : wd_host;
   const float a = __fsub_rn(1.0f, __fmul_rn(lr, wd));
@@ -904,71 +849,76 @@ __global__ __launch_bounds__(256) void dion2_post_kernel(PtrTab X, int mats_per_
   const UT* u = U + (int64_t)mat * (select_rows ? (int64_t)k * cols : (int64_t)rows * k);
   const int r_end = (blockIdx.x * 8 + 8) < rows ? (blockIdx.x * 8 + 8) : rows;
   for (int r = blockIdx.x * 8; r < r_end; ++r) {
-    float* xr = x + (int64_t)r * cols;
+    XT* xr = x + (int64_t)r * cols;
     if (select_rows) {
       const int j = mp[r];
       const UT* ur = u + (int64_t)(j < 0 ? 0 : j) * cols;
       // per-row scale of the selected slice (rows selected only): u is multiplied by it first
       if (row_scale && j >= 0) b = __fmul_rn(b0, row_scale[(int64_t)mat * k + j]);
       if (VEC) {
-        for (int c = threadIdx.x * 4; c < cols; c += 1024) {
-          float4 v = *(const float4*)(xr + c);
+        for (int c4 = threadIdx.x; c4 < cols / 4; c4 += 256) {
+          float v[4];
+          st_load4<XT>(xr, c4, v);
           float4 uv = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (j >= 0) uv = u_load4<UT>(ur, c);
-          v.x = fmaf(a, v.x, -(b * uv.x));
-          v.y = fmaf(a, v.y, -(b * uv.y));
-          v.z = fmaf(a, v.z, -(b * uv.z));
-          v.w = fmaf(a, v.w, -(b * uv.w));
-          *(float4*)(xr + c) = v;
+          if (j >= 0) uv = u_load4<UT>(ur, c4 * 4);
+          v[0] = fmaf(a, v[0], -(b * uv.x));
+          v[1] = fmaf(a, v[1], -(b * uv.y));
+          v[2] = fmaf(a, v[2], -(b * uv.z));
+          v[3] = fmaf(a, v[3], -(b * uv.w));
+          st_store4<XT>(xr, c4, v);
         }
       } else {
         for (int c = threadIdx.x; c < cols; c += 256) {
           const float uv = j >= 0 ? u_load<UT>(ur, c) : 0.f;
-          xr[c] = fmaf(a, xr[c], -(b * uv));
+          st_store<XT>(xr, c, fmaf(a, st_load<XT>(xr, c), -(b * uv)));
         }
       }
     } else {
       const UT* ur = u + (int64_t)r * k;
       if (VEC) {
-        for (int c = threadIdx.x * 4; c < cols; c += 1024) {
-          float4 v = *(const float4*)(xr + c);
-          const int4 j4 = *(const int4*)(mp + c);
+        for (int c4 = threadIdx.x; c4 < cols / 4; c4 += 256) {
+          float v[4];
+          st_load4<XT>(xr, c4, v);
+          const int4 j4 = *(const int4*)(mp + c4 * 4);
           const float u0 = j4.x >= 0 ? u_load<UT>(ur, j4.x) : 0.f;
           const float u1 = j4.y >= 0 ? u_load<UT>(ur, j4.y) : 0.f;
           const float u2 = j4.z >= 0 ? u_load<UT>(ur, j4.z) : 0.f;
           const float u3 = j4.w >= 0 ? u_load<UT>(ur, j4.w) : 0.f;
-          v.x = fmaf(a, v.x, -(b * u0));
-          v.y = fmaf(a, v.y, -(b * u1));
-          v.z = fmaf(a, v.z, -(b * u2));
-          v.w = fmaf(a, v.w, -(b * u3));
-          *(float4*)(xr + c) = v;
+          v[0] = fmaf(a, v[0], -(b * u0));
+          v[1] = fmaf(a, v[1], -(b * u1));
+          v[2] = fmaf(a, v[2], -(b * u2));
+          v[3] = fmaf(a, v[3], -(b * u3));
+          st_store4<XT>(xr, c4, v);
         }
       } else {
         for (int c = threadIdx.x; c < cols; c += 256) {
           const int j = mp[c];
           const float uv = j >= 0 ? u_load<UT>(ur, j) : 0.f;
-          xr[c] = fmaf(a, xr[c], -(b * uv));
+          st_store<XT>(xr, c, fmaf(a, st_load<XT>(xr, c), -(b * uv)));
         }
       }
     }
   }
 }
 
-hipError_t launch_dion2_post(const PtrTab& X, int n_mat, int mats_per_ptr, int rows, int cols,
+hipError_t launch_dion2_post(const PtrTab& X, int x_dtype, int n_mat, int mats_per_ptr, int rows, int cols,
                              int select_rows, const void* U, int u_dtype, int k, const int32_t* map,
                              const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
                              float adj_ratio, const float* wd_dev, float wd_host, bool vec4,
                              hipStream_t st) {
   dim3 grid((rows + 7) / 8, n_mat);
-#define D2POST_LAUNCH(V, UT)                                                                        \
-  hipLaunchKernelGGL((dion2_post_kernel<V, UT>), grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols, \
-                     select_rows, (const UT*)U, k, map, row_scale, lr_dev, adj_lr_dev, adj_ratio,     \
+#define D2POST_LAUNCH(V, UT, XT)                                                                          \
+  hipLaunchKernelGGL((dion2_post_kernel<V, UT, XT>), grid, dim3(256), 0, st, X, mats_per_ptr, rows, cols, \
+                     select_rows, (const UT*)U, k, map, row_scale, lr_dev, adj_lr_dev, adj_ratio,           \
                      wd_dev, wd_host)
+#define D2POST_LAUNCH_X(V, UT) \
+  do { if (x_dtype == 0) D2POST_LAUNCH(V, UT, bf16_t); else D2POST_LAUNCH(V, UT, float); } while (0)
   if (u_dtype == 0) {
-    if (vec4) D2POST_LAUNCH(true, bf16_t); else D2POST_LAUNCH(false, bf16_t);
+    if (vec4) D2POST_LAUNCH_X(true, bf16_t); else D2POST_LAUNCH_X(false, bf16_t);
   } else {
-    if (vec4) D2POST_LAUNCH(true, float); else D2POST_LAUNCH(false, float);
+    if (vec4) D2POST_LAUNCH_X(true, float); else D2POST_LAUNCH_X(false, float);
   }
+#undef D2POST_LAUNCH_X
 #undef D2POST_LAUNCH
   return hipGetLastError();
 }

@@ -4,7 +4,9 @@
 // One launch updates up to kMtaTensors tensors of different sizes: their pointers and element
 // counts travel by value in the kernel-argument segment, blockIdx.y picks the tensor and the
 // blocks of a row walk it with a grid stride.  All traffic is HBM streaming: AdamW reads X, G, M, V
-// and writes X, M, V (28 B/element with fp32 gradients, 26 with bf16), Lion 20 / 18 B/element.
+// and writes X, M, V (28 B/element with fp32 state and gradients, 26 with bf16 gradients), Lion 20 / 18
+// B/element.  The state tensors X, M, V of one launch share a dtype, fp32 or bf16 (half the bytes);
+// arithmetic is fp32 either way.
 //
 // Arithmetic follows dion/scalar_opts.py:7-65 (adamw_update) and :68-118 (lion_update); the step
 // counters are device scalars advanced on the device, like the capturable form of
@@ -18,11 +20,6 @@ struct MtaTensors {
   uint64_t x[kMtaTensors], g[kMtaTensors], m[kMtaTensors], v[kMtaTensors], step[kMtaTensors];
   int64_t numel[kMtaTensors];
 };
-
-template <typename GT>
-static __device__ __forceinline__ float grad_at(const void* g, int64_t i) {
-  return sizeof(GT) == 2 ? bf16_to_f32(((const bf16_t*)g)[i]) : ((const float*)g)[i];
-}
 
 // step[t] += 1 for every tensor of the launch (before the update kernel reads them).
 __global__ void mta_advance_steps_kernel(MtaTensors a, int n) {
@@ -57,16 +54,16 @@ static __device__ __forceinline__ void adamw_one(float& x, float g, float& m, fl
   x = x - adj_lr * upd;
 }
 
-template <typename GT>
+template <typename GT, typename ST>
 __global__ __launch_bounds__(256) void adamw_mt_kernel(MtaTensors a, const float* __restrict__ lr_dev,
                                                        const float* __restrict__ wd_dev,
                                                        AdamwScalars sc) {
   const int t = blockIdx.y;
   const int64_t numel = a.numel[t];
-  float* __restrict__ x = (float*)a.x[t];
-  const void* __restrict__ g = (const void*)a.g[t];
-  float* __restrict__ m = (float*)a.m[t];
-  float* __restrict__ v = (float*)a.v[t];
+  ST* __restrict__ x = (ST*)a.x[t];
+  const GT* __restrict__ g = (const GT*)a.g[t];
+  ST* __restrict__ m = (ST*)a.m[t];
+  ST* __restrict__ v = (ST*)a.v[t];
   const float step = *(const float*)a.step[t];
   const float lr = *lr_dev;
   const float wd = wd_dev ? *wd_dev : sc.wd_host;
@@ -79,37 +76,31 @@ __global__ __launch_bounds__(256) void adamw_mt_kernel(MtaTensors a, const float
   const float w1 = 1.0f - sc.beta1, w2 = 1.0f - sc.beta2;
   const int64_t stride = (int64_t)gridDim.x * 256;
   const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const bool vec = (((a.x[t] | a.m[t] | a.v[t]) & 15) == 0) &&
+  // groups of 4 elements: 16-byte accesses to fp32 tensors, 8-byte accesses to bf16 ones
+  const bool vec = (((a.x[t] | a.m[t] | a.v[t]) & (sizeof(ST) == 2 ? 7 : 15)) == 0) &&
                    ((a.g[t] & (sizeof(GT) == 2 ? 7 : 15)) == 0);
   const int64_t n4 = vec ? numel / 4 : 0;
   for (int64_t q = tid; q < n4; q += stride) {
-    float4 xv = ((const float4*)x)[q], mv = ((const float4*)m)[q], vv = ((const float4*)v)[q];
-    float gv[4];
-    if (sizeof(GT) == 2) {
-      const uint2 raw = ((const uint2*)g)[q];
-      gv[0] = __uint_as_float(raw.x << 16);
-      gv[1] = __uint_as_float(raw.x & 0xffff0000u);
-      gv[2] = __uint_as_float(raw.y << 16);
-      gv[3] = __uint_as_float(raw.y & 0xffff0000u);
-    } else {
-      const float4 t4 = ((const float4*)g)[q];
-      gv[0] = t4.x; gv[1] = t4.y; gv[2] = t4.z; gv[3] = t4.w;
-    }
-    adamw_one<GT>(xv.x, gv[0], mv.x, vv.x, w1, sc.beta2, w2, inv_bc2_sqrt, sc.eps, adj_lr, aa, coeff, sc.cautious);
-    adamw_one<GT>(xv.y, gv[1], mv.y, vv.y, w1, sc.beta2, w2, inv_bc2_sqrt, sc.eps, adj_lr, aa, coeff, sc.cautious);
-    adamw_one<GT>(xv.z, gv[2], mv.z, vv.z, w1, sc.beta2, w2, inv_bc2_sqrt, sc.eps, adj_lr, aa, coeff, sc.cautious);
-    adamw_one<GT>(xv.w, gv[3], mv.w, vv.w, w1, sc.beta2, w2, inv_bc2_sqrt, sc.eps, adj_lr, aa, coeff, sc.cautious);
-    ((float4*)x)[q] = xv;
-    ((float4*)m)[q] = mv;
-    ((float4*)v)[q] = vv;
+    float xv[4], mv[4], vv[4], gv[4];
+    st_load4<ST>(x, q, xv);
+    st_load4<ST>(m, q, mv);
+    st_load4<ST>(v, q, vv);
+    st_load4<GT>(g, q, gv);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      adamw_one<GT>(xv[e], gv[e], mv[e], vv[e], w1, sc.beta2, w2, inv_bc2_sqrt, sc.eps, adj_lr, aa, coeff,
+                    sc.cautious);
+    st_store4<ST>(x, q, xv);
+    st_store4<ST>(m, q, mv);
+    st_store4<ST>(v, q, vv);
   }
   for (int64_t i = n4 * 4 + tid; i < numel; i += stride) {
-    float xs = x[i], ms = m[i], vs = v[i];
-    adamw_one<GT>(xs, grad_at<GT>(g, i), ms, vs, w1, sc.beta2, w2, inv_bc2_sqrt, sc.eps, adj_lr, aa, coeff,
+    float xs = st_load<ST>(x, i), ms = st_load<ST>(m, i), vs = st_load<ST>(v, i);
+    adamw_one<GT>(xs, st_load<GT>(g, i), ms, vs, w1, sc.beta2, w2, inv_bc2_sqrt, sc.eps, adj_lr, aa, coeff,
                   sc.cautious);
-    x[i] = xs;
-    m[i] = ms;
-    v[i] = vs;
+    st_store<ST>(x, i, xs);
+    st_store<ST>(m, i, ms);
+    st_store<ST>(v, i, vs);
   }
 }
 
@@ -126,15 +117,15 @@ static __device__ __forceinline__ void lion_one(float& x, float g, float& m, flo
   x = x - lr * u;
 }
 
-template <typename GT>
+template <typename GT, typename ST>
 __global__ __launch_bounds__(256) void lion_mt_kernel(MtaTensors a, const float* __restrict__ lr_dev,
                                                       const float* __restrict__ wd_dev, float beta1,
                                                       float beta2, float wd_host, int cautious) {
   const int t = blockIdx.y;
   const int64_t numel = a.numel[t];
-  float* __restrict__ x = (float*)a.x[t];
-  const void* __restrict__ g = (const void*)a.g[t];
-  float* __restrict__ m = (float*)a.m[t];
+  ST* __restrict__ x = (ST*)a.x[t];
+  const GT* __restrict__ g = (const GT*)a.g[t];
+  ST* __restrict__ m = (ST*)a.m[t];
   const float lr = *lr_dev;
   const float wd = wd_dev ? *wd_dev : wd_host;
   const float coeff = lr * wd;
@@ -142,33 +133,24 @@ __global__ __launch_bounds__(256) void lion_mt_kernel(MtaTensors a, const float*
   const float w1 = 1.0f - beta1, w2 = 1.0f - beta2;
   const int64_t stride = (int64_t)gridDim.x * 256;
   const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const bool vec = (((a.x[t] | a.m[t]) & 15) == 0) && ((a.g[t] & (sizeof(GT) == 2 ? 7 : 15)) == 0);
+  const bool vec = (((a.x[t] | a.m[t]) & (sizeof(ST) == 2 ? 7 : 15)) == 0) &&
+                   ((a.g[t] & (sizeof(GT) == 2 ? 7 : 15)) == 0);
   const int64_t n4 = vec ? numel / 4 : 0;
   for (int64_t q = tid; q < n4; q += stride) {
-    float4 xv = ((const float4*)x)[q], mv = ((const float4*)m)[q];
-    float gv[4];
-    if (sizeof(GT) == 2) {
-      const uint2 raw = ((const uint2*)g)[q];
-      gv[0] = __uint_as_float(raw.x << 16);
-      gv[1] = __uint_as_float(raw.x & 0xffff0000u);
-      gv[2] = __uint_as_float(raw.y << 16);
-      gv[3] = __uint_as_float(raw.y & 0xffff0000u);
-    } else {
-      const float4 t4 = ((const float4*)g)[q];
-      gv[0] = t4.x; gv[1] = t4.y; gv[2] = t4.z; gv[3] = t4.w;
-    }
-    lion_one(xv.x, gv[0], mv.x, w1, w2, lr, aa, coeff, cautious);
-    lion_one(xv.y, gv[1], mv.y, w1, w2, lr, aa, coeff, cautious);
-    lion_one(xv.z, gv[2], mv.z, w1, w2, lr, aa, coeff, cautious);
-    lion_one(xv.w, gv[3], mv.w, w1, w2, lr, aa, coeff, cautious);
-    ((float4*)x)[q] = xv;
-    ((float4*)m)[q] = mv;
+    float xv[4], mv[4], gv[4];
+    st_load4<ST>(x, q, xv);
+    st_load4<ST>(m, q, mv);
+    st_load4<GT>(g, q, gv);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) lion_one(xv[e], gv[e], mv[e], w1, w2, lr, aa, coeff, cautious);
+    st_store4<ST>(x, q, xv);
+    st_store4<ST>(m, q, mv);
   }
   for (int64_t i = n4 * 4 + tid; i < numel; i += stride) {
-    float xs = x[i], ms = m[i];
-    lion_one(xs, grad_at<GT>(g, i), ms, w1, w2, lr, aa, coeff, cautious);
-    x[i] = xs;
-    m[i] = ms;
+    float xs = st_load<ST>(x, i), ms = st_load<ST>(m, i);
+    lion_one(xs, st_load<GT>(g, i), ms, w1, w2, lr, aa, coeff, cautious);
+    st_store<ST>(x, i, xs);
+    st_store<ST>(m, i, ms);
   }
 }
 
@@ -197,7 +179,7 @@ static void fill(MtaTensors& a, const uint64_t* X, const uint64_t* G, const uint
 }
 
 hipError_t launch_adamw_mt(const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M,
-                           const uint64_t* V, const uint64_t* steps, const int64_t* numel, int n,
+                           const uint64_t* V, int s_dtype, const uint64_t* steps, const int64_t* numel, int n,
                            const float* lr_dev, float beta1, float beta2, float eps, const float* wd_dev,
                            float wd_host, int cautious, hipStream_t st) {
   MtaTensors a;
@@ -205,25 +187,32 @@ hipError_t launch_adamw_mt(const uint64_t* X, const uint64_t* G, int g_dtype, co
   hipLaunchKernelGGL(mta_advance_steps_kernel, dim3(1), dim3(64), 0, st, a, n);
   AdamwScalars sc{beta1, beta2, eps, wd_host, cautious};
   dim3 grid(mta_blocks(numel, n), n);
-  if (g_dtype == 0)
-    hipLaunchKernelGGL(adamw_mt_kernel<bf16_t>, grid, dim3(256), 0, st, a, lr_dev, wd_dev, sc);
-  else
-    hipLaunchKernelGGL(adamw_mt_kernel<float>, grid, dim3(256), 0, st, a, lr_dev, wd_dev, sc);
+#define ADAMW_LAUNCH(GT, ST) \
+  hipLaunchKernelGGL((adamw_mt_kernel<GT, ST>), grid, dim3(256), 0, st, a, lr_dev, wd_dev, sc)
+  if (g_dtype == 0) {
+    if (s_dtype == 0) ADAMW_LAUNCH(bf16_t, bf16_t); else ADAMW_LAUNCH(bf16_t, float);
+  } else {
+    if (s_dtype == 0) ADAMW_LAUNCH(float, bf16_t); else ADAMW_LAUNCH(float, float);
+  }
+#undef ADAMW_LAUNCH
   return hipGetLastError();
 }
 
-hipError_t launch_lion_mt(const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M,
+hipError_t launch_lion_mt(const uint64_t* X, const uint64_t* G, int g_dtype, const uint64_t* M, int s_dtype,
                           const int64_t* numel, int n, const float* lr_dev, float beta1, float beta2,
                           const float* wd_dev, float wd_host, int cautious, hipStream_t st) {
   MtaTensors a;
   fill(a, X, G, M, nullptr, nullptr, numel, n);
   dim3 grid(mta_blocks(numel, n), n);
-  if (g_dtype == 0)
-    hipLaunchKernelGGL(lion_mt_kernel<bf16_t>, grid, dim3(256), 0, st, a, lr_dev, wd_dev, beta1, beta2,
-                       wd_host, cautious);
-  else
-    hipLaunchKernelGGL(lion_mt_kernel<float>, grid, dim3(256), 0, st, a, lr_dev, wd_dev, beta1, beta2,
-                       wd_host, cautious);
+#define LION_LAUNCH(GT, ST)                                                                             \
+  hipLaunchKernelGGL((lion_mt_kernel<GT, ST>), grid, dim3(256), 0, st, a, lr_dev, wd_dev, beta1, beta2, \
+                     wd_host, cautious)
+  if (g_dtype == 0) {
+    if (s_dtype == 0) LION_LAUNCH(bf16_t, bf16_t); else LION_LAUNCH(bf16_t, float);
+  } else {
+    if (s_dtype == 0) LION_LAUNCH(float, bf16_t); else LION_LAUNCH(float, float);
+  }
+#undef LION_LAUNCH
   return hipGetLastError();
 }
 

@@ -295,8 +295,8 @@ hipError_t launch_mask_index(const float* norms, int n_mat, int dim, int32_t* ga
 
 // x = a*x - b*u (one rounding of the sum; b carries the per-row scale when given) everywhere -- u is
 // zero off the selected slices -- and m *= ef_decay on the selected slices.  Block = 8 rows of one
-// matrix.
-template <bool VEC>
+// matrix.  X and M share their dtype ST (fp32 or bf16).
+template <bool VEC, typename ST>
 __global__ __launch_bounds__(256) void dion2_post_masked_kernel(PtrTab X, PtrTab M, int mats_per_ptr,
                                                                 int rows, int cols, int select_rows,
                                                                 const bf16_t* __restrict__ U,
@@ -309,8 +309,8 @@ __global__ __launch_bounds__(256) void dion2_post_masked_kernel(PtrTab X, PtrTab
                                                                 float wd_host, float ef_decay) {
   const int mat = blockIdx.y;
   const int64_t moff = (int64_t)(mat % mats_per_ptr) * rows * cols;
-  float* x = (float*)X.p[mat / mats_per_ptr] + moff;
-  float* m = (float*)M.p[mat / mats_per_ptr] + moff;
+  ST* x = (ST*)X.p[mat / mats_per_ptr] + moff;
+  ST* m = (ST*)M.p[mat / mats_per_ptr] + moff;
   const bf16_t* u = U + (int64_t)mat * rows * cols;
   const float lr = *lr_dev;
   const float wd = wd_dev ? *wd_dev : wd_host;
@@ -320,80 +320,78 @@ __global__ __launch_bounds__(256) void dion2_post_masked_kernel(PtrTab X, PtrTab
   const float* nm = norms + (int64_t)mat * dim;
   const int r_end = (blockIdx.x * 8 + 8) < rows ? (blockIdx.x * 8 + 8) : rows;
   for (int r = blockIdx.x * 8; r < r_end; ++r) {
-    float* xr = x + (int64_t)r * cols;
-    float* mr = m + (int64_t)r * cols;
+    ST* xr = x + (int64_t)r * cols;
+    ST* mr = m + (int64_t)r * cols;
     const bf16_t* ur = u + (int64_t)r * cols;
     const bool row_sel = select_rows && nm[r] > 0.f;
     const float b = (row_scale && select_rows) ? __fmul_rn(b0, row_scale[(int64_t)mat * rows + r]) : b0;
     if (select_rows && !row_sel) {
       // unselected row: u is zero, m stays
       if (VEC) {
-        for (int c = threadIdx.x * 4; c < cols; c += 1024) {
-          float4 v = *(const float4*)(xr + c);
-          v.x = __fmul_rn(a, v.x);
-          v.y = __fmul_rn(a, v.y);
-          v.z = __fmul_rn(a, v.z);
-          v.w = __fmul_rn(a, v.w);
-          *(float4*)(xr + c) = v;
+        for (int c4 = threadIdx.x; c4 < cols / 4; c4 += 256) {
+          float v[4];
+          st_load4<ST>(xr, c4, v);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(a, v[e]);
+          st_store4<ST>(xr, c4, v);
         }
       } else {
-        for (int c = threadIdx.x; c < cols; c += 256) xr[c] = __fmul_rn(a, xr[c]);
+        for (int c = threadIdx.x; c < cols; c += 256) st_store<ST>(xr, c, __fmul_rn(a, st_load<ST>(xr, c)));
       }
       continue;
     }
     if (VEC) {
-      for (int c = threadIdx.x * 4; c < cols; c += 1024) {
-        float4 v = *(const float4*)(xr + c);
-        const uint2 raw = *(const uint2*)(ur + c);
-        const float u0 = __uint_as_float(raw.x << 16), u1 = __uint_as_float(raw.x & 0xffff0000u);
-        const float u2 = __uint_as_float(raw.y << 16), u3 = __uint_as_float(raw.y & 0xffff0000u);
-        v.x = fmaf(a, v.x, -(b * u0));
-        v.y = fmaf(a, v.y, -(b * u1));
-        v.z = fmaf(a, v.z, -(b * u2));
-        v.w = fmaf(a, v.w, -(b * u3));
-        *(float4*)(xr + c) = v;
+      for (int c4 = threadIdx.x; c4 < cols / 4; c4 += 256) {
+        float v[4], uv[4];
+        st_load4<ST>(xr, c4, v);
+        st_load4<bf16_t>(ur, c4, uv);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = fmaf(a, v[e], -(b * uv[e]));
+        st_store4<ST>(xr, c4, v);
         if (select_rows) {
-          float4 mv = *(const float4*)(mr + c);
-          mv.x = __fmul_rn(mv.x, ef_decay);
-          mv.y = __fmul_rn(mv.y, ef_decay);
-          mv.z = __fmul_rn(mv.z, ef_decay);
-          mv.w = __fmul_rn(mv.w, ef_decay);
-          *(float4*)(mr + c) = mv;
+          float mv[4];
+          st_load4<ST>(mr, c4, mv);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) mv[e] = __fmul_rn(mv[e], ef_decay);
+          st_store4<ST>(mr, c4, mv);
         } else {
-          const float4 n4 = *(const float4*)(nm + c);
+          const float4 n4 = *(const float4*)(nm + c4 * 4);
           if (n4.x > 0.f || n4.y > 0.f || n4.z > 0.f || n4.w > 0.f) {
-            float4 mv = *(const float4*)(mr + c);
-            if (n4.x > 0.f) mv.x = __fmul_rn(mv.x, ef_decay);
-            if (n4.y > 0.f) mv.y = __fmul_rn(mv.y, ef_decay);
-            if (n4.z > 0.f) mv.z = __fmul_rn(mv.z, ef_decay);
-            if (n4.w > 0.f) mv.w = __fmul_rn(mv.w, ef_decay);
-            *(float4*)(mr + c) = mv;
+            float mv[4];
+            st_load4<ST>(mr, c4, mv);
+            if (n4.x > 0.f) mv[0] = __fmul_rn(mv[0], ef_decay);
+            if (n4.y > 0.f) mv[1] = __fmul_rn(mv[1], ef_decay);
+            if (n4.z > 0.f) mv[2] = __fmul_rn(mv[2], ef_decay);
+            if (n4.w > 0.f) mv[3] = __fmul_rn(mv[3], ef_decay);
+            st_store4<ST>(mr, c4, mv);
           }
         }
       }
     } else {
       for (int c = threadIdx.x; c < cols; c += 256) {
-        xr[c] = fmaf(a, xr[c], -(b * bf16_to_f32(ur[c])));
-        if (select_rows || nm[c] > 0.f) mr[c] = __fmul_rn(mr[c], ef_decay);
+        st_store<ST>(xr, c, fmaf(a, st_load<ST>(xr, c), -(b * bf16_to_f32(ur[c]))));
+        if (select_rows || nm[c] > 0.f) st_store<ST>(mr, c, __fmul_rn(st_load<ST>(mr, c), ef_decay));
       }
     }
   }
 }
 
-hipError_t launch_dion2_post_masked(const PtrTab& X, const PtrTab& M, int n_mat, int mats_per_ptr,
+hipError_t launch_dion2_post_masked(const PtrTab& X, const PtrTab& M, int s_dtype, int n_mat, int mats_per_ptr,
                                     int rows, int cols, int select_rows, const bf16_t* U,
                                     const float* norms, const float* row_scale, const float* lr_dev,
                                     const float* adj_lr_dev, float adj_ratio, const float* wd_dev,
                                     float wd_host, float ef_decay, bool vec4, hipStream_t st) {
   dim3 grid((rows + 7) / 8, n_mat);
-  if (vec4)
-    hipLaunchKernelGGL(dion2_post_masked_kernel<true>, grid, dim3(256), 0, st, X, M, mats_per_ptr, rows,
-                       cols, select_rows, U, norms, row_scale, lr_dev, adj_lr_dev, adj_ratio, wd_dev,
-                       wd_host, ef_decay);
-  else
-    hipLaunchKernelGGL(dion2_post_masked_kernel<false>, grid, dim3(256), 0, st, X, M, mats_per_ptr, rows,
-                       cols, select_rows, U, norms, row_scale, lr_dev, adj_lr_dev, adj_ratio, wd_dev,
-                       wd_host, ef_decay);
+#define MASKED_LAUNCH(V, ST)                                                                              \
+  hipLaunchKernelGGL((dion2_post_masked_kernel<V, ST>), grid, dim3(256), 0, st, X, M, mats_per_ptr, rows,  \
+                     cols, select_rows, U, norms, row_scale, lr_dev, adj_lr_dev, adj_ratio, wd_dev,        \
+                     wd_host, ef_decay)
+  if (s_dtype == 0) {
+    if (vec4) MASKED_LAUNCH(true, bf16_t); else MASKED_LAUNCH(false, bf16_t);
+  } else {
+    if (vec4) MASKED_LAUNCH(true, float); else MASKED_LAUNCH(false, float);
+  }
+#undef MASKED_LAUNCH
   return hipGetLastError();
 }
 

@@ -220,6 +220,13 @@ def _list_ptrs(ts: List[Tensor], name: str, dtype=None, numel=None):
     return ptr_table([t.data_ptr() for t in ts])
 
 
+def _state_ptrs(ts: List[Tensor], name: str, numel=None):
+    """(pointer table, dtype code) of a list of optimizer-state tensors (parameters, momentum, second
+    moments): contiguous GPU tensors that share one dtype, float32 or bfloat16."""
+    code = _dtype_code(ts[0], name)
+    return _list_ptrs(ts, name, ts[0].dtype, numel), code
+
+
 def _scalar_args(lr: Tensor, weight_decay, device):
     """lr must already be a 0-d fp32 device tensor; weight decay may be one, or a host number."""
     if not (isinstance(lr, Tensor) and lr.is_cuda and lr.dtype == torch.float32 and lr.numel() == 1):
@@ -239,10 +246,10 @@ def muon_pre(G: List[Tensor], M: List[Tensor], momentum: float, nesterov: bool) 
     assert n == len(M) and n > 0
     numel = M[0].numel()
     gp = _list_ptrs(G, "G", G[0].dtype, numel)
-    mp = _list_ptrs(M, "M", torch.float32, numel)
+    mp, mcode = _state_ptrs(M, "M", numel)
     U = torch.empty((n, *M[0].shape), dtype=torch.bfloat16, device=M[0].device)
     lib = _lib.load()
-    check(lib.dion_muon_pre(gp, _dtype_code(G[0], "G"), mp, U.data_ptr(), n, numel, float(momentum),
+    check(lib.dion_muon_pre(gp, _dtype_code(G[0], "G"), mp, mcode, U.data_ptr(), n, numel, float(momentum),
                             int(bool(nesterov)), _stream_handle(U.device)), "muon_pre")
     return U
 
@@ -256,7 +263,7 @@ def muon_post(X: List[Tensor], U: Tensor, lr: Tensor, adj_ratio: float, weight_d
     assert n > 0 and U.shape[0] == n
     numel = X[0].numel()
     cols = X[0].shape[-1]
-    xp = _list_ptrs(X, "X", torch.float32, numel)
+    xp, xcode = _state_ptrs(X, "X", numel)
     if not U.is_contiguous() or U.numel() != n * numel:
         raise ValueError("U must be a contiguous [N, *shape] arena")
     lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, U.device)
@@ -266,7 +273,7 @@ def muon_post(X: List[Tensor], U: Tensor, lr: Tensor, adj_ratio: float, weight_d
             raise ValueError("row_scale must be float32 [N, rows]")
         rs_p = row_scale.data_ptr()
     lib = _lib.load()
-    check(lib.dion_muon_post(xp, U.data_ptr(), _dtype_code(U, "U"), n, numel, cols, rs_p, lr_p,
+    check(lib.dion_muon_post(xp, xcode, U.data_ptr(), _dtype_code(U, "U"), n, numel, cols, rs_p, lr_p,
                              float(adj_ratio), wd_p, wd_h, int(bool(cautious_wd)),
                              _stream_handle(U.device)), "muon_post")
 
@@ -281,10 +288,10 @@ def normuon_stats(U: Tensor, V: List[Tensor], beta2: float) -> Tensor:
     rows, cols = U.shape[-2], U.shape[-1]
     n_mat = U.numel() // (rows * cols)
     mats_per_ptr = n_mat // n
-    vp = _list_ptrs(V, "V", torch.float32, mats_per_ptr * rows)
+    vp, vcode = _state_ptrs(V, "V", mats_per_ptr * rows)
     scale = torch.empty(n_mat, rows, dtype=torch.float32, device=U.device)
     lib = _lib.load()
-    check(lib.dion_normuon_stats(U.data_ptr(), vp, n, mats_per_ptr, rows, cols, float(beta2),
+    check(lib.dion_normuon_stats(U.data_ptr(), vp, vcode, n, mats_per_ptr, rows, cols, float(beta2),
                                  scale.data_ptr(), _stream_handle(U.device)), "normuon_stats")
     return scale
 
@@ -301,12 +308,12 @@ def normuon_stats_selected(U: Tensor, V: List[Tensor], idx: Tensor, beta2: float
     n_mat = U.numel() // (k * cols)
     mats_per_ptr = n_mat // n
     v_rows = V[0].numel() // mats_per_ptr
-    vp = _list_ptrs(V, "V", torch.float32, mats_per_ptr * v_rows)
+    vp, vcode = _state_ptrs(V, "V", mats_per_ptr * v_rows)
     if idx.dtype != torch.int32 or not idx.is_contiguous() or idx.numel() != n_mat * k:
         raise ValueError("idx must be a contiguous int32 tensor of n_mat * k entries")
     scale = torch.empty(n_mat, k, dtype=torch.float32, device=U.device)
     lib = _lib.load()
-    check(lib.dion_normuon_stats_selected(U.data_ptr(), vp, n, mats_per_ptr, k, cols, idx.data_ptr(), v_rows,
+    check(lib.dion_normuon_stats_selected(U.data_ptr(), vp, vcode, n, mats_per_ptr, k, cols, idx.data_ptr(), v_rows,
                                           float(beta2), scale.data_ptr(), _stream_handle(U.device)),
           "normuon_stats_selected")
     return scale
@@ -326,7 +333,7 @@ def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_d
     mats_per_ptr = numel // (rows * cols)
     n_mat = n * mats_per_ptr
     gp = _list_ptrs(G, "G", G[0].dtype, numel)
-    mp = _list_ptrs(M, "M", torch.float32, numel)
+    mp, mcode = _state_ptrs(M, "M", numel)
     dev = M[0].device
     dim = rows if select_dim == -2 else cols
     norms = torch.empty(n_mat, dim, dtype=torch.float32, device=dev)
@@ -338,12 +345,12 @@ def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_d
     st = _stream_handle(dev)
     sbytes = lib.dion_dion2_accumulate_scratch_bytes(n_mat, rows, cols, select_dim)
     scratch = torch.empty(sbytes, dtype=torch.uint8, device=dev) if sbytes else None
-    check(lib.dion_dion2_accumulate(gp, _dtype_code(G[0], "G"), mp, n, mats_per_ptr, rows, cols, select_dim,
+    check(lib.dion_dion2_accumulate(gp, _dtype_code(G[0], "G"), mp, mcode, n, mats_per_ptr, rows, cols, select_dim,
                                     norms.data_ptr(), scratch.data_ptr() if sbytes else None, sbytes, st),
           "dion2_accumulate")
     check(lib.dion_dion2_topk(norms.data_ptr(), n_mat, dim, k, idx.data_ptr(), imap.data_ptr(), st),
           "dion2_topk")
-    check(lib.dion_dion2_gather(mp, n, mats_per_ptr, rows, cols, select_dim, idx.data_ptr(), k,
+    check(lib.dion_dion2_gather(mp, mcode, n, mats_per_ptr, rows, cols, select_dim, idx.data_ptr(), k,
                                 float(ef_decay), U.data_ptr(), st), "dion2_gather")
     return U, idx, imap
 
@@ -362,7 +369,7 @@ def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: 
     rows, cols = shape[-2], shape[-1]
     numel = X[0].numel()
     mats_per_ptr = numel // (rows * cols)
-    xp = _list_ptrs(X, "X", torch.float32, numel)
+    xp, xcode = _state_ptrs(X, "X", numel)
     _require_gpu(U, "U")
     if not U.is_contiguous():
         raise ValueError("U must be contiguous")
@@ -380,7 +387,7 @@ def dion2_post(X: List[Tensor], U: Tensor, imap: Tensor, lr: Tensor, adj_ratio: 
         if not (adjusted_lr.is_cuda and adjusted_lr.dtype == torch.float32 and adjusted_lr.numel() == 1):
             raise TypeError("adjusted_lr must be a 0-d float32 GPU tensor")
         alr = adjusted_lr.data_ptr()
-    check(lib.dion_dion2_post(xp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(), _dtype_code(U, "U"), k,
+    check(lib.dion_dion2_post(xp, xcode, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(), _dtype_code(U, "U"), k,
                               imap.data_ptr(), rs, lr_p, alr, float(adj_ratio), wd_p, wd_h,
                               _stream_handle(U.device)), "dion2_post")
 
@@ -528,8 +535,10 @@ def dion2_post_masked(X: List[Tensor], M: List[Tensor], U: Tensor, norms: Tensor
     numel = X[0].numel()
     mats_per_ptr = numel // (rows * cols)
     n_mat = n * mats_per_ptr
-    xp = _list_ptrs(X, "X", torch.float32, numel)
-    mp = _list_ptrs(M, "M", torch.float32, numel)
+    xp, xcode = _state_ptrs(X, "X", numel)
+    mp, mcode = _state_ptrs(M, "M", numel)
+    if xcode != mcode:
+        raise TypeError(f"X ({X[0].dtype}) and M ({M[0].dtype}) must share one dtype")
     _check_bf16(U, "U")
     if not U.is_contiguous() or U.numel() != n * numel:
         raise ValueError("U must be a contiguous [N, *shape] arena")
@@ -549,7 +558,7 @@ def dion2_post_masked(X: List[Tensor], M: List[Tensor], U: Tensor, norms: Tensor
             raise TypeError("adjusted_lr must be a 0-d float32 GPU tensor")
         alr = adjusted_lr.data_ptr()
     lib = _lib.load()
-    check(lib.dion_dion2_post_masked(xp, mp, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(),
+    check(lib.dion_dion2_post_masked(xp, mp, xcode, n, mats_per_ptr, rows, cols, select_dim, U.data_ptr(),
                                      norms.data_ptr(), rs, lr_p, alr, float(adj_ratio), wd_p, wd_h,
                                      float(ef_decay), _stream_handle(U.device)), "dion2_post_masked")
 
@@ -561,22 +570,24 @@ def _mta_tables(X: List[Tensor], G: List[Tensor], states: List[List[Tensor]]):
     n = len(X)
     assert n > 0 and len(G) == n and all(len(s) == n for s in states)
     gdt = G[0].dtype
+    sdt = X[0].dtype
     for x, g in zip(X, G):
         _require_gpu(x, "X")
         _require_gpu(g, "G")
-        if x.dtype != torch.float32:
-            raise NotImplementedError(f"X: the gfx950 step kernels keep parameters in float32, got {x.dtype}")
+        if x.dtype != sdt:
+            raise TypeError("X: one parameter dtype per call")
         if g.dtype != gdt:
             raise TypeError("G: one gradient dtype per call")
         if not x.is_contiguous() or not g.is_contiguous() or g.numel() != x.numel():
             raise ValueError("X / G must be contiguous and of equal size")
     for name, st in zip("MV", states):
         for x, s in zip(X, st):
-            if s.dtype != torch.float32 or not s.is_contiguous() or s.numel() != x.numel() or not s.is_cuda:
-                raise ValueError(f"{name}: optimizer state must be contiguous float32 GPU tensors shaped like X")
+            if s.dtype != sdt or not s.is_contiguous() or s.numel() != x.numel() or not s.is_cuda:
+                raise ValueError(f"{name}: optimizer state must be contiguous GPU tensors shaped like X, in the "
+                                 f"dtype of X ({sdt})")
     numels = (_lib.ctypes.c_int64 * n)(*[x.numel() for x in X])
     tabs = [ptr_table([t.data_ptr() for t in ts]) for ts in (X, G, *states)]
-    return tabs, numels, _dtype_code(G[0], "G")
+    return tabs, numels, _dtype_code(G[0], "G"), _dtype_code(X[0], "X")
 
 
 def adamw_step(X: List[Tensor], G: List[Tensor], M: List[Tensor], V: List[Tensor], steps: List[Tensor],
@@ -584,14 +595,14 @@ def adamw_step(X: List[Tensor], G: List[Tensor], M: List[Tensor], V: List[Tensor
                cautious_wd: bool = False) -> None:
     """One fused AdamW step over tensors of any sizes (dion/scalar_opts.py:7-65, :121-268).  ``steps``
     are 0-d float32 device counters (one per tensor; tensors may share one), advanced on the device."""
-    (xp, gp, mp, vp), numels, gcode = _mta_tables(X, G, [M, V])
+    (xp, gp, mp, vp), numels, gcode, scode = _mta_tables(X, G, [M, V])
     for s in steps:
         if not (s.is_cuda and s.dtype == torch.float32 and s.numel() == 1):
             raise TypeError("steps must be 0-d float32 GPU tensors")
     sp = ptr_table([s.data_ptr() for s in steps])
     lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, X[0].device)
     lib = _lib.load()
-    check(lib.dion_adamw_step(xp, gp, gcode, mp, vp, sp, numels, len(X), lr_p, float(beta1), float(beta2),
+    check(lib.dion_adamw_step(xp, gp, gcode, mp, vp, scode, sp, numels, len(X), lr_p, float(beta1), float(beta2),
                               float(epsilon), wd_p, wd_h, int(bool(cautious_wd)), _stream_handle(X[0].device)),
           "adamw_step")
 
@@ -599,8 +610,8 @@ def adamw_step(X: List[Tensor], G: List[Tensor], M: List[Tensor], V: List[Tensor
 def lion_step(X: List[Tensor], G: List[Tensor], M: List[Tensor], lr: Tensor, beta1: float, beta2: float,
               weight_decay, cautious_wd: bool = False) -> None:
     """One fused Lion step over tensors of any sizes (dion/scalar_opts.py:68-118, :271-325)."""
-    (xp, gp, mp), numels, gcode = _mta_tables(X, G, [M])
+    (xp, gp, mp), numels, gcode, scode = _mta_tables(X, G, [M])
     lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, X[0].device)
     lib = _lib.load()
-    check(lib.dion_lion_step(xp, gp, gcode, mp, numels, len(X), lr_p, float(beta1), float(beta2), wd_p, wd_h,
+    check(lib.dion_lion_step(xp, gp, gcode, mp, scode, numels, len(X), lr_p, float(beta1), float(beta2), wd_p, wd_h,
                              int(bool(cautious_wd)), _stream_handle(X[0].device)), "lion_step")

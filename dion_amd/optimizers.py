@@ -39,10 +39,12 @@ def _note_stream(t: Tensor) -> None:
         t.record_stream(torch.cuda.current_stream(t.device))
 
 
-def _require_fp32(params: List[Tensor], who: str) -> None:
-    if params[0].dtype != torch.float32:
+def _require_state_dtype(params: List[Tensor], who: str) -> None:
+    """Parameters (and with them momentum / second moments, dion/megabatch_base.py:198-203) are kept in
+    float32 or bfloat16; the kernels compute in fp32 and round a bf16 value once, on store."""
+    if params[0].dtype not in (torch.float32, torch.bfloat16):
         raise NotImplementedError(
-            f"{who}: the gfx950 step kernels keep parameters and optimizer state in float32; "
+            f"{who}: the gfx950 step kernels keep parameters and optimizer state in float32 or bfloat16; "
             f"got parameter dtype {params[0].dtype}"
         )
 
@@ -69,7 +71,7 @@ class _MomentumOrtho(OrthoOptimizer):
             rows, cols = shape[-2], shape[-1]
             mats = params[0].numel() // (rows * cols)
             ratio_shape = shape
-        _require_fp32(params, type(self).__name__)
+        _require_state_dtype(params, type(self).__name__)
         n = len(params)
         X = [p.data for p in params]
         G = [p.grad.contiguous() for p in params]
@@ -217,7 +219,7 @@ class Dion2(OrthoOptimizer):
             rows, cols = shape[-2], shape[-1]
             mats = params[0].numel() // (rows * cols)
             ratio_shape = shape
-        _require_fp32(params, "Dion2")
+        _require_state_dtype(params, "Dion2")
         n = len(params)
         # unsharded: select along the shorter dimension (dion/dion2.py:270-272)
         select_dim = -2 if rows <= cols else -1
@@ -336,7 +338,7 @@ class NorDion2(OrthoOptimizer):
             rows, cols = shape[-2], shape[-1]
             mats = params[0].numel() // (rows * cols)
             ratio_shape = shape
-        _require_fp32(params, "NorDion2")
+        _require_state_dtype(params, "NorDion2")
         n = len(params)
         select_dim = -2  # whole rows, so the per-neuron normalisation sees complete neurons
         k = min(max(1, int(math.ceil(group["fraction"] * rows))), rows)

@@ -88,16 +88,20 @@ int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, in
 
 /* --------------------------------------------------------------------------------------------
  * Memory-bound fused kernels of the optimizer step.
+ * Optimizer state -- parameters X, momentum M, second moments V -- is fp32 or bf16 in memory, as the
+ * reference keeps it in the parameter's dtype (dion/megabatch_base.py:198-203, dion/normuon.py:122):
+ * every entry point that touches state takes its dtype (x_dtype / m_dtype / v_dtype / s_dtype,
+ * DION_F32 or DION_BF16).  Arithmetic is fp32; a bf16 state value is rounded once, on store.
  * ------------------------------------------------------------------------------------------ */
 
 /* Momentum update + orthogonalization input for one shape group.
  *   M_i = mu M_i + G_i;  U[i] = bf16(nesterov ? mu M_i + G_i : M_i)
  * G_ptrs / M_ptrs: host ptr tables of n device pointers, each to `numel` dense elements
- * (G bf16 or fp32 per g_dtype; M fp32).  U: one dense [n, numel] bf16 arena.
+ * (G bf16 or fp32 per g_dtype; M per m_dtype).  U: one dense [n, numel] bf16 arena.
  * Replaces muon_update_pre_orthogonalize (dion/muon.py:284-311) plus the torch.stack of
  * dion/megabatch_base.py:872. */
-int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, void* U, int n,
-                  int64_t numel, float mu, int nesterov, void* stream);
+int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int m_dtype, void* U,
+                  int n, int64_t numel, float mu, int nesterov, void* stream);
 
 /* Weight decay + update for one shape group.
  *   X_i = (1 - lr wd) X_i - lr adj_ratio U[i]            (cautious == 0)
@@ -105,9 +109,9 @@ int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, v
  * lr_dev: device float (the reference's live 0-d lr tensor); wd_dev: device float or NULL, in
  * which case wd_host is used.  U is the [n, numel] arena, bf16 or fp32 per u_dtype.
  * row_scale (nullable): device [n, rows] fp32; U[i][r][:] is multiplied by row_scale[i][r]
- * first, rows = numel / cols (used by NorMuon).  X fp32.
+ * first, rows = numel / cols (used by NorMuon).  X per x_dtype.
  * Replaces muon_update_post_orthogonalize (dion/muon.py:315-347). */
-int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype, int n, int64_t numel,
+int dion_muon_post(const uint64_t* X_ptrs, int x_dtype, const void* U, int u_dtype, int n, int64_t numel,
                    int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
                    const float* wd_dev, float wd_host, int cautious, void* stream);
 
@@ -115,22 +119,23 @@ int dion_muon_post(const uint64_t* X_ptrs, const void* U, int u_dtype, int n, in
  *   r = mean(U^2, dim=-1); V = lerp(V, r, 1-beta2); d = sqrt(V)+1e-8;
  *   row_scale[i][r] = (1/d) * ||U_i||_F / max(||U_i / d||_F, 1e-8)
  * U [n_mat, rows, cols] bf16 (orthogonalized); V_ptrs: host ptr table of n device pointers, each
- * to mats_per_ptr*rows fp32 (n*mats_per_ptr == n_mat); row_scale out [n_mat, rows] fp32.  The
+ * to mats_per_ptr*rows elements of v_dtype (n*mats_per_ptr == n_mat); row_scale out [n_mat, rows]
+ * fp32.  The
  * scaled update is applied by dion_muon_post(row_scale=...).
  * Replaces normuon_normalization_stacked (dion/normuon.py:345-399) and the V write-back of
  * dion/normuon.py:320. */
-int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr, int rows,
-                       int cols, float beta2, float* row_scale, void* stream);
+int dion_normuon_stats(const void* U, const uint64_t* V_ptrs, int v_dtype, int n, int mats_per_ptr,
+                       int rows, int cols, float beta2, float* row_scale, void* stream);
 
 /* NorMuon statistics for an update made of k selected rows per matrix (NorDion2): U [n_mat, k,
  * cols] bf16, row_idx [n_mat, k] int32 gives the row of the parameter each update row belongs to
  * (a negative entry: that update row is not part of the update, its second moment stays and its
  * scale is 0);
- * V_ptrs entries each point to mats_per_ptr * v_rows fp32 (the full per-row buffers); only the
+ * V_ptrs entries each point to mats_per_ptr * v_rows elements of v_dtype (the full per-row buffers); only the
  * selected entries of V are read and written.  row_scale out [n_mat, k].
  * Replaces nordion2_normalize_selected_stacked (dion/nordion2.py:430-447). */
-int dion_normuon_stats_selected(const void* U, const uint64_t* V_ptrs, int n, int mats_per_ptr, int k,
-                                int cols, const int32_t* row_idx, int v_rows, float beta2,
+int dion_normuon_stats_selected(const void* U, const uint64_t* V_ptrs, int v_dtype, int n, int mats_per_ptr,
+                                int k, int cols, const int32_t* row_idx, int v_rows, float beta2,
                                 float* row_scale, void* stream);
 
 /* Dion2 momentum accumulate + slice L1 norms for one shape group.
@@ -143,7 +148,7 @@ int dion_normuon_stats_selected(const void* U, const uint64_t* V_ptrs, int n, in
  * all rows of its columns.
  * Replaces the first half of dion2_pre_orthogonalize (dion/dion2.py:487-509). */
 size_t dion_dion2_accumulate_scratch_bytes(int n_mat, int rows, int cols, int select_dim);
-int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int n,
+int dion_dion2_accumulate(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int m_dtype, int n,
                           int mats_per_ptr, int rows, int cols, int select_dim, float* norms,
                           void* scratch, size_t scratch_bytes, void* stream);
 
@@ -159,7 +164,7 @@ int dion_dion2_topk(const float* norms, int n_mat, int dim, int k, int32_t* idx,
  *   U_sel[i] = bf16(M_i[selected slices]);  M_i[selected slices] *= ef_decay
  * U_sel [n_mat, k, cols] (select_dim -2) or [n_mat, rows, k] (select_dim -1) bf16.
  * Replaces dion/dion2.py:519-545. */
-int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr, int rows, int cols,
+int dion_dion2_gather(const uint64_t* M_ptrs, int m_dtype, int n, int mats_per_ptr, int rows, int cols,
                       int select_dim, const int32_t* idx, int k, float ef_decay, void* U_sel,
                       void* stream);
 
@@ -172,7 +177,7 @@ int dion_dion2_gather(const uint64_t* M_ptrs, int n, int mats_per_ptr, int rows,
  * multiplied by row_scale[i][j] first (NorDion2's normalised update).
  * Replaces dion2_post_orthogonalize_triton (dion/dion2_triton.py:147-242, kernel :57-144),
  * dion2_post_orthogonalize (dion/dion2.py:666-697) and its use at dion/nordion2.py:403-425. */
-int dion_dion2_post(const uint64_t* X_ptrs, int n, int mats_per_ptr, int rows, int cols,
+int dion_dion2_post(const uint64_t* X_ptrs, int x_dtype, int n, int mats_per_ptr, int rows, int cols,
                     int select_dim, const void* U_sel, int u_dtype, int k, const int32_t* map,
                     const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
                     float adj_ratio, const float* wd_dev, float wd_host, void* stream);
@@ -220,7 +225,7 @@ int dion_mask_index(const float* norms, int n_mat, int dim, int32_t* gate, void*
  * [n_mat, rows] fp32, row r of u is multiplied by row_scale[i][r] first.
  * Replaces dion2_post_orthogonalize_masked (dion/dion2.py:623-659) and, with row_scale, the update
  * half of nordion2_post_orthogonalize_masked (dion/nordion2.py:448-500). */
-int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int n, int mats_per_ptr,
+int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int s_dtype, int n, int mats_per_ptr,
                            int rows, int cols, int select_dim, const void* U, const float* norms,
                            const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
                            float adj_ratio, const float* wd_dev, float wd_host, float ef_decay,
@@ -229,7 +234,7 @@ int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int n
 /* --------------------------------------------------------------------------------------------
  * Multi-tensor AdamW / Lion for the non-matrix parameter groups (algorithm "adamw" / "lion").
  * X_ptrs, G_ptrs, M_ptrs, V_ptrs: host ptr tables of n device pointers; tensor i has numels[i]
- * elements (host array); X, M, V fp32, G bf16 or fp32 per g_dtype (one dtype per call).
+ * elements (host array); X, M, V share s_dtype, G bf16 or fp32 per g_dtype (one dtype each per call).
  * lr_dev / wd_dev as in dion_muon_post.  Any number of tensors per call, any sizes.
  * ------------------------------------------------------------------------------------------ */
 
@@ -241,7 +246,7 @@ int dion_dion2_post_masked(const uint64_t* X_ptrs, const uint64_t* M_ptrs, int n
  * Replaces adamw_update / adamw_update_foreach (dion/scalar_opts.py:7-65, :121-268; capturable
  * form: counters advance on the device, lr is read on the device). */
 int dion_adamw_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs,
-                    const uint64_t* V_ptrs, const uint64_t* step_ptrs, const int64_t* numels, int n,
+                    const uint64_t* V_ptrs, int s_dtype, const uint64_t* step_ptrs, const int64_t* numels, int n,
                     const float* lr_dev, float beta1, float beta2, float eps, const float* wd_dev,
                     float wd_host, int cautious, void* stream);
 
@@ -249,7 +254,7 @@ int dion_adamw_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype,
  *   X = X (1 - lr wd)   [cautious: X -= X [U X >= 0] lr wd];   X -= lr U
  * Replaces lion_update / lion_update_foreach (dion/scalar_opts.py:68-118, :271-325). */
 int dion_lion_step(const uint64_t* X_ptrs, const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs,
-                   const int64_t* numels, int n, const float* lr_dev, float beta1, float beta2,
+                   int s_dtype, const int64_t* numels, int n, const float* lr_dev, float beta1, float beta2,
                    const float* wd_dev, float wd_host, int cautious, void* stream);
 
 #ifdef __cplusplus

@@ -13,6 +13,48 @@ def _declared_symbols():
     return sorted(set(re.findall(r"\b(dion_[a-z0-9_]+)\s*\(", text)))
 
 
+def _declared_prototypes():
+    """name -> list of C parameter declarations, from the header text."""
+    text = open(os.path.join(ROOT, "include", "dion_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for name, args in re.findall(r"\b(dion_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        args = " ".join(args.split())
+        out[name] = [] if args in ("", "void") else [a.strip() for a in args.split(",")]
+    return out
+
+
+def test_ctypes_prototypes_follow_the_header():
+    """Argument count and kind (pointer / float / integer) of every ctypes prototype match the header."""
+    import ctypes
+
+    from dion_amd import _lib
+
+    protos = _declared_prototypes()
+    assert set(protos) == set(_declared_symbols())
+    for name, cargs in protos.items():
+        _res, argtypes = _lib.SIGNATURES[name]
+        assert len(argtypes) == len(cargs), f"{name}: header has {len(cargs)} parameters, ctypes {len(argtypes)}"
+        for decl, ct in zip(cargs, argtypes):
+            if "*" in decl:
+                kind = "ptr"
+            elif decl.startswith("float"):
+                kind = "float"
+            else:
+                kind = "int"
+            if ct is ctypes.c_float:
+                got = "float"
+            elif ct in (ctypes.c_int, ctypes.c_int64, ctypes.c_size_t):
+                got = "int"
+            else:
+                got = "ptr"
+            assert kind == got, f"{name}: `{decl}` bound as {ct}"
+            if kind == "int":
+                want = ctypes.c_int64 if decl.startswith("int64_t") else \
+                    ctypes.c_size_t if decl.startswith("size_t") else ctypes.c_int
+                assert ct is want, f"{name}: `{decl}` bound as {ct}"
+
+
 def test_header_declares_the_expected_surface():
     syms = _declared_symbols()
     for name in ["dion_ns_line_1", "dion_ns_line_2", "dion_ns_line_3", "dion_ns_orthogonalize",
@@ -31,7 +73,7 @@ def test_library_exports_every_declared_symbol():
     for name in _declared_symbols():
         assert hasattr(lib, name), f"{name} declared in dion_hip.h but not exported"
         assert name in _lib.SIGNATURES, f"{name} has no ctypes prototype"
-    assert lib.dion_abi_version() >= 1
+    assert lib.dion_abi_version() == _lib.ABI_VERSION
     # pure host entry points
     assert lib.dion_ns_workspace_bytes(0, 128, 128, 0) == 0
     n = lib.dion_ns_workspace_bytes(2, 768, 3072, 0)
@@ -80,12 +122,17 @@ def test_argument_validation_happens_before_any_device_work():
     refused(lib.dion_scatter_slices(None, 0, 1, 8, 8, -1, None, -1, None, None), "k outside")
     refused(lib.dion_mask_index(None, -1, 4, None, None), "bad size")
     refused(lib.dion_dion2_index_map(None, 1, 9, 8, None, None), "bad size")
-    refused(lib.dion_dion2_post(None, 1, 1, 8, 8, -2, None, 5, 2, None, None, None, None, f(1.0), None, f(0.0), None),
-            "u_dtype")
-    refused(lib.dion_dion2_post(None, 1, 1, 8, 8, 1, None, 0, 2, None, None, None, None, f(1.0), None, f(0.0), None),
-            "select_dim")
-    refused(lib.dion_dion2_post_masked(None, None, 1, 0, 8, 8, -2, None, None, None, None, None, f(1.0), None,
+    refused(lib.dion_dion2_post(None, 1, 1, 1, 8, 8, -2, None, 5, 2, None, None, None, None, f(1.0), None, f(0.0),
+                                None), "u_dtype")
+    refused(lib.dion_dion2_post(None, 1, 1, 1, 8, 8, 1, None, 0, 2, None, None, None, None, f(1.0), None, f(0.0),
+                                None), "select_dim")
+    refused(lib.dion_dion2_post(None, 3, 1, 1, 8, 8, -2, None, 0, 2, None, None, None, None, f(1.0), None, f(0.0),
+                                None), "x_dtype")
+    refused(lib.dion_dion2_post_masked(None, None, 1, 1, 0, 8, 8, -2, None, None, None, None, None, f(1.0), None,
                                        f(0.0), f(0.9), None), "bad size")
+    refused(lib.dion_muon_pre(None, 0, None, 2, None, 1, 8, f(0.9), 0, None), "m_dtype")
+    refused(lib.dion_adamw_step(None, None, 0, None, None, -1, None, None, 1, None, f(0.9), f(0.9), f(1e-8), None,
+                                f(0.0), 0, None), "s_dtype")
     refused(lib.dion_ns_orthogonalize(None, 9, None, 1, 8, 8, None, 0, f(1.0), f(0.0), 0, 0, None, 0, None),
             "in_dtype")
     refused(lib.dion_ns_line_1(None, None, 1, 128, 128, None), "null argument")
