@@ -108,6 +108,8 @@ def main() -> int:
     ap.add_argument("--selection-scope", default="local", choices=["local", "global"],
                     help="dion2 / nordion2: 'global' runs the whole-matrix sequence (accumulate, select inside the "
                          "orthogonalization call, masked update) that a rank runs on assembled matrices")
+    ap.add_argument("--state-dtype", default="fp32", choices=["fp32", "bf16"],
+                    help="dtype of parameters and optimizer state (the headline configuration is fp32)")
     ap.add_argument("--graph", action="store_true",
                     help="capture the step into a hipGraph during warm-up and time replays (needs --warmup >= 2)")
     ap.add_argument("--breakdown", action="store_true",
@@ -135,7 +137,9 @@ def main() -> int:
     torch.cuda.set_device(dev)
     spec = WORKLOADS[args.workload]
 
-    # ---- synthetic model: X ~ N(0, 0.02) fp32, G ~ N(0, 0.02) bf16, momentum fp32 zeros
+    # ---- synthetic model: X ~ N(0, 0.02), G ~ N(0, 0.02) bf16, momentum zeros in the dtype of X (fp32 unless
+    # --state-dtype bf16)
+    sdt = torch.float32 if args.state_dtype == "fp32" else torch.bfloat16
     params = []
     groups = []
     gen = torch.Generator(device=dev).manual_seed(1234)
@@ -145,7 +149,7 @@ def main() -> int:
     for name, rows, cols, count in spec:
         these = []
         for _ in range(count):
-            p = torch.nn.Parameter(torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen))
+            p = torch.nn.Parameter(torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen).to(sdt))
             p.grad_dtype = None
             p.grad = torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen).to(torch.bfloat16)
             these.append(p)
@@ -215,6 +219,7 @@ def main() -> int:
                         + ({"dion2": ", fraction 0.25, ef_decay 0.95", "nordion2": ", fraction 0.25, mu 0.95"}
                            .get(args.optimizer, ", nesterov mu=0.95"))
                         + (", whole-matrix selection" if args.selection_scope == "global" else "")
+                        + (", bf16 parameters and state" if args.state_dtype == "bf16" else "")
                         + (", muon_beta2 0.95" if args.optimizer in ("normuon", "nordion2") else "") + ") over "
                         + ", ".join(f"{c}x({r}x{k})" for _n, r, k, c in spec),
             "matrices": sum(c for *_x, c in spec),
