@@ -110,6 +110,8 @@ def main() -> int:
                          "orthogonalization call, masked update) that a rank runs on assembled matrices")
     ap.add_argument("--state-dtype", default="fp32", choices=["fp32", "bf16"],
                     help="dtype of parameters and optimizer state (the headline configuration is fp32)")
+    ap.add_argument("--two-call-update", action="store_true",
+                    help="Muon: orthogonalize and update as two library calls instead of the fused one")
     ap.add_argument("--graph", action="store_true",
                     help="capture the step into a hipGraph during warm-up and time replays (needs --warmup >= 2)")
     ap.add_argument("--breakdown", action="store_true",
@@ -177,6 +179,8 @@ def main() -> int:
     else:
         opt = Dion2(groups, lr=0.02, fraction=fraction, ef_decay=0.95, weight_decay=0.01,
                     adjust_lr="spectral_norm", selection_scope=args.selection_scope, **ns_kw)
+    if args.two_call_update:
+        opt.fused_update = False
     if args.selection_scope == "global":
         if args.optimizer not in ("dion2", "nordion2"):
             print("bench.py: --selection-scope applies to dion2 / nordion2", file=sys.stderr)
@@ -220,6 +224,7 @@ def main() -> int:
                            .get(args.optimizer, ", nesterov mu=0.95"))
                         + (", whole-matrix selection" if args.selection_scope == "global" else "")
                         + (", bf16 parameters and state" if args.state_dtype == "bf16" else "")
+                        + (", two-call update" if args.two_call_update else "")
                         + (", muon_beta2 0.95" if args.optimizer in ("normuon", "nordion2") else "") + ") over "
                         + ", ".join(f"{c}x({r}x{k})" for _n, r, k, c in spec),
             "matrices": sum(c for *_x, c in spec),

@@ -15,7 +15,7 @@ DION_BF16 = 0
 DION_F32 = 1
 DION_NS_GRAM = 1
 DION_NS_CARRY_XT = 2
-ABI_VERSION = 7  # dion_abi_version() of the library these signatures describe
+ABI_VERSION = 8  # dion_abi_version() of the library these signatures describe
 
 _u64p = ctypes.POINTER(ctypes.c_uint64)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -32,6 +32,10 @@ SIGNATURES = {
     "dion_ns_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "dion_ns_orthogonalize": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, _f32p, c_int,
                                       c_float, c_float, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "dion_ns_update_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "dion_ns_orthogonalize_update": (c_int, [c_void_p, c_int, _u64p, c_int, c_int, c_int, c_int, c_int, _f32p,
+                                             c_int, c_float, c_float, c_int, c_int, c_void_p, c_float, c_void_p,
+                                             c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "dion_muon_pre": (c_int, [_u64p, c_int, _u64p, c_int, c_void_p, c_int, c_int64, c_float, c_int, c_void_p]),
     "dion_muon_post": (c_int, [_u64p, c_int, c_void_p, c_int, c_int, c_int64, c_int, c_void_p, c_void_p,
                                c_float, c_void_p, c_float, c_int, c_void_p]),

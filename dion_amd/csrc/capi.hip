@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 7; }
+extern "C" int dion_abi_version(void) { return 8; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -189,22 +189,57 @@ extern "C" size_t dion_ns_workspace_bytes(int batch, int rows, int cols, int fla
   return make_plan(batch, rows, cols, flags).total;
 }
 
-extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, int rows,
-                                     int cols, const float* coeffs, int n_iters, float norm_scale,
-                                     float eps, int flags, int gram_reset, void* workspace,
-                                     size_t workspace_bytes, void* stream) {
+static bool table_aligned(const uint64_t* t, int n);
+static int check_state_dtype(const char* who, const char* arg, int dtype) {
+  if (dtype != DION_BF16 && dtype != DION_F32)
+    return fail(DION_E_INVALID, "%s: %s %d (DION_BF16 or DION_F32)", who, arg, dtype);
+  return DION_OK;
+}
+static inline int dt(int dtype) { return dtype == DION_BF16 ? 0 : 1; }
+
+namespace {
+// The Muon update that consumes the orthogonalized matrices (dion_ns_orthogonalize_update).
+struct PostSpec {
+  const uint64_t* X_ptrs;
+  int x_dtype, n_ptrs, mats_per_ptr;
+  const float* lr_dev;
+  float adj_ratio;
+  const float* wd_dev;
+  float wd_host;
+  int cautious;
+};
+
+// per-head regime: whole iteration resident in LDS, one workgroup per matrix, no workspace
+bool ns_small_path(int rows, int cols, int flags, int n_iters) {
+  return !(flags & DION_NS_GRAM) && n_iters <= kMaxSmallIters && ns_small_fits(rows, cols) &&
+         !getenv("DION_NO_SMALL_KERNEL");
+}
+
+// The update rides on the last GEMM when that GEMM produces the caller's tensor directly: at least
+// one iteration, the X-only form, no padding between the matrices and the tiles, not the
+// LDS-resident kernel.
+bool ns_update_fuses(int batch, int rows, int cols, int flags, int n_iters) {
+  if (n_iters <= 0 || (flags & DION_NS_CARRY_XT) || ns_small_path(rows, cols, flags, n_iters)) return false;
+  const NsPlan pl = make_plan(batch, rows, cols, flags);
+  return pl.mp == pl.m && pl.np == pl.n;
+}
+}  // namespace
+
+// Orthogonalization proper.  With `post` (only when ns_update_fuses) the last GEMM applies the update
+// to the parameters and `out` is not written.
+static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, int cols, const float* coeffs,
+                  int n_iters, float norm_scale, float eps, int flags, int gram_reset, void* workspace,
+                  size_t workspace_bytes, void* stream, const PostSpec* post) {
   if (batch < 0 || rows < 0 || cols < 0 || n_iters < 0)
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: negative extent");
   if (in_dtype != DION_BF16 && in_dtype != DION_F32)
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: in_dtype %d", in_dtype);
   if (batch == 0 || rows == 0 || cols == 0) return DION_OK;
-  if (!in || !out || (n_iters > 0 && !coeffs))
+  if (!in || (!out && !post) || (n_iters > 0 && !coeffs))
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: null argument");
   if (flags & ~(DION_NS_GRAM | DION_NS_CARRY_XT)) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
   hipStream_t st = (hipStream_t)stream;
-  if (!(flags & DION_NS_GRAM) && n_iters <= kMaxSmallIters && ns_small_fits(rows, cols) &&
-      !getenv("DION_NO_SMALL_KERNEL")) {
-    // per-head regime: whole iteration resident in LDS, one workgroup per matrix, no workspace
+  if (ns_small_path(rows, cols, flags, n_iters)) {
     NsCoeffs co;
     memset(&co, 0, sizeof(co));
     co.n = n_iters;
@@ -334,6 +369,37 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     p.K = mp;
     p.batch = batch;
     p.alpha = 1.0f;
+    if (final_direct && post) {
+      // the product is consumed by the update: one launch per kMaxPtrs parameters
+      const int mpp = post->mats_per_ptr;
+      if (pl.tall) {
+        p.strideCt = (int64_t)mp * np;
+        p.ldct = mp;
+      } else {
+        p.strideC = (int64_t)mp * np;
+        p.ldc = np;
+      }
+      for (int c0 = 0; c0 < post->n_ptrs; c0 += kMaxPtrs) {
+        const int c = (post->n_ptrs - c0) < kMaxPtrs ? (post->n_ptrs - c0) : kMaxPtrs;
+        const int64_t b0 = (int64_t)c0 * mpp;
+        GemmParams q = p;
+        q.P = p.P + b0 * p.strideP;
+        q.Q = p.Q + b0 * p.strideQ;
+        q.batch = c * mpp;
+        FusedPost fp;
+        memset(&fp, 0, sizeof(fp));
+        memcpy(fp.X.p, post->X_ptrs + c0, (size_t)c * sizeof(uint64_t));
+        fp.mats_per_ptr = mpp;
+        fp.vec_ok = table_aligned(post->X_ptrs + c0, c) ? 1 : 0;
+        fp.lr_dev = post->lr_dev;
+        fp.wd_dev = post->wd_dev;
+        fp.wd_host = post->wd_host;
+        fp.adj_ratio = post->adj_ratio;
+        fp.cautious = post->cautious;
+        if (hipError_t e = launch_gemm_nt_post(q, fp, dt(post->x_dtype), pl.tall != 0, st)) return e;
+      }
+      return hipSuccess;
+    }
     if (final_direct) {
       if (pl.tall) {
         p.Ct = (bf16_t*)out;
@@ -422,12 +488,64 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
     }
   }
   if (!wrote_out) {
+    if (post) return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: update not applied (internal)");
     if (pl.tall)
       HIP_TRY(launch_unpad(Xt[cur], sXt, ldxt, (bf16_t*)out, batch, rows, cols, st), "unpad");
     else
       HIP_TRY(launch_unpad(X[cur], sX, ldx, (bf16_t*)out, batch, rows, cols, st), "unpad");
   }
   return DION_OK;
+}
+
+extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, int rows,
+                                     int cols, const float* coeffs, int n_iters, float norm_scale,
+                                     float eps, int flags, int gram_reset, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+  return ns_run(in, in_dtype, out, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
+                workspace, workspace_bytes, stream, nullptr);
+}
+
+extern "C" size_t dion_ns_update_workspace_bytes(int batch, int rows, int cols, int flags, int n_iters) {
+  if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
+  const size_t ns = align256(make_plan(batch, rows, cols, flags).total);
+  if (ns_update_fuses(batch, rows, cols, flags, n_iters)) return ns;
+  return ns + align256((size_t)batch * rows * cols * 2);
+}
+
+extern "C" int dion_ns_orthogonalize_update(const void* in, int in_dtype, const uint64_t* X_ptrs, int x_dtype,
+                                            int n_ptrs, int mats_per_ptr, int rows, int cols,
+                                            const float* coeffs, int n_iters, float norm_scale, float eps,
+                                            int flags, int gram_reset, const float* lr_dev, float adj_ratio,
+                                            const float* wd_dev, float wd_host, int cautious,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = check_state_dtype("dion_ns_orthogonalize_update", "x_dtype", x_dtype)) return rc;
+  if (n_ptrs < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || n_iters < 0)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: bad size");
+  if ((int64_t)n_ptrs * mats_per_ptr > 0x7fffffff)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: too many matrices");
+  const int batch = n_ptrs * mats_per_ptr;
+  if (batch == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!X_ptrs || !lr_dev) return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: null argument");
+  for (int i = 0; i < n_ptrs; ++i)
+    if (!X_ptrs[i]) return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: parameter %d is null", i);
+  if (workspace_bytes < dion_ns_update_workspace_bytes(batch, rows, cols, flags, n_iters))
+    return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize_update: workspace %zu < %zu bytes", workspace_bytes,
+                dion_ns_update_workspace_bytes(batch, rows, cols, flags, n_iters));
+  if (ns_update_fuses(batch, rows, cols, flags, n_iters)) {
+    const PostSpec ps = {X_ptrs, x_dtype, n_ptrs, mats_per_ptr, lr_dev, adj_ratio, wd_dev, wd_host, cautious};
+    return ns_run(in, in_dtype, nullptr, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
+                  workspace, workspace_bytes, stream, &ps);
+  }
+  // padded shapes, the X / X^T form, the LDS-resident kernel: orthogonalize into the tail of the
+  // workspace, then the plain update pass
+  const size_t ns = align256(make_plan(batch, rows, cols, flags).total);
+  if (!workspace) return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize_update: workspace is null");
+  void* tmp = (char*)workspace + ns;
+  if (int rc = ns_run(in, in_dtype, tmp, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
+                      workspace, ns, stream, nullptr))
+    return rc;
+  return dion_muon_post(X_ptrs, x_dtype, tmp, DION_BF16, n_ptrs, (int64_t)mats_per_ptr * rows * cols, cols,
+                        nullptr, lr_dev, adj_ratio, wd_dev, wd_host, cautious, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -446,12 +564,6 @@ static int ptr_chunk(int mats_per_ptr) {
   return c < kMaxPtrs ? c : kMaxPtrs;
 }
 
-static int check_state_dtype(const char* who, const char* arg, int dtype) {
-  if (dtype != DION_BF16 && dtype != DION_F32)
-    return fail(DION_E_INVALID, "%s: %s %d (DION_BF16 or DION_F32)", who, arg, dtype);
-  return DION_OK;
-}
-static inline int dt(int dtype) { return dtype == DION_BF16 ? 0 : 1; }
 
 static void fill_tab(PtrTab& tab, const uint64_t* src, int n) {
   memset(&tab, 0, sizeof(tab));

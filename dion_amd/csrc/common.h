@@ -105,6 +105,57 @@ __device__ __forceinline__ void st_store8(T* p, int64_t i8, const float v[8]) {
   }
 }
 
+// Muon's decoupled weight decay (plain or cautious) + scaled update of one element
+// (dion/muon.py:315-347): a = 1 - lr*wd, coeff = lr*wd, b = lr*adj_ratio.  Every operation is
+// rounded on its own, in the order of the eager reference, in every translation unit that uses it.
+__device__ __forceinline__ float muon_post_one(float x, float u, float a, float coeff, float b, int cautious) {
+  // Plain operators under this pragma: no fused multiply-add, whatever the translation unit's default
+  // (the __fmul_rn / __fsub_rn wrappers carry the default of the header that defines them).
+#pragma clang fp contract(off)
+  if (cautious) {
+    // mask = min(sign(x*u) + 1, 1): 0 only where x*u < 0  (dion/muon.py:333-340)
+    const float mask = (x * u < 0.f) ? 0.f : 1.f;
+    x = x - (x * mask) * coeff;
+  } else {
+    x = x * a;
+  }
+  return x - u * b;
+}
+
+// coeff = lr*wd, a = 1 - coeff, b = lr*adj_ratio, each rounded on its own.
+__device__ __forceinline__ void muon_post_coeffs(float lr, float wd, float adj_ratio, float& a, float& coeff,
+                                                 float& b) {
+#pragma clang fp contract(off)
+  coeff = lr * wd;
+  a = 1.0f - coeff;
+  b = lr * adj_ratio;
+}
+
+// Up to kMaxPtrs device pointers passed by value in the kernel-argument segment: the
+// list-of-parameters of one shape group reaches the GPU without a host->device copy.
+constexpr int kMaxPtrs = 64;
+struct PtrTab {
+  uint64_t p[kMaxPtrs];
+};
+
+// The Muon update applied by the epilogue of the last GEMM of an orthogonalization instead of
+// storing the product: matrix b of the launch updates the parameter matrix
+// X.p[b / mats_per_ptr] + (b % mats_per_ptr) * strideC (strideCt), leading dimension ldc (ldct),
+// with the product element rounded to bf16 first (what a separate update pass would read back).
+struct FusedPost {
+  PtrTab X;
+  int mats_per_ptr;
+  int vec_ok;  // every pointer is 16-byte aligned: the transposed form may use 16-byte accesses
+  const float* lr_dev;
+  const float* wd_dev;  // optional; wd_host otherwise
+  float wd_host;
+  float adj_ratio;
+  int cautious;
+};
+struct NoPost {
+  int unused;
+};
+
 // Raises a kernel's dynamic-LDS limit once per device: the attribute belongs to the device that is
 // current when it is set, so `done` keeps one bit per device ordinal.
 static inline hipError_t set_max_dynamic_lds_once(const void* fn, int bytes, std::atomic<uint64_t>& done) {
@@ -142,6 +193,12 @@ struct GemmParams {
 
 // Returns hipSuccess or the launch error.  variant < 0 picks by shape.
 hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream);
+// C = P * Q with Q K-major (p.q_kmajor, no tri, no D), the product consumed by the fused Muon update
+// instead of being stored: `transposed` false updates X[row][col] (ldc / strideC describe X),
+// true updates X[col][row] (ldct / strideCt).  x_dtype 0 = bf16, 1 = fp32.  p.batch <= kMaxPtrs *
+// post.mats_per_ptr.
+hipError_t launch_gemm_nt_post(const GemmParams& p, const FusedPost& post, int x_dtype, bool transposed,
+                               hipStream_t stream);
 // Tile edge (128 or 256) launch_gemm_nt would use for a problem whose padded short/long
 // dims are given; workspaces are padded to this.
 int gemm_pad_granule(int m, int n, int batch);

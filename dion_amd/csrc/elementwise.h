@@ -5,12 +5,6 @@
 
 namespace dion {
 
-// Up to kMaxPtrs device pointers passed by value in the kernel-argument segment: the
-// list-of-parameters of one shape group reaches the GPU without a host->device copy.
-constexpr int kMaxPtrs = 64;
-struct PtrTab {
-  uint64_t p[kMaxPtrs];
-};
 
 // Coefficient schedule passed by value to the LDS-resident small-matrix kernel.
 constexpr int kMaxSmallIters = 8;

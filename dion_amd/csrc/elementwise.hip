@@ -318,18 +318,6 @@ hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, int m_
 // ------------------------------------------------------------------------------------------
 // Muon / NorMuon post: decoupled weight decay (plain or cautious) + scaled update.
 // ------------------------------------------------------------------------------------------
-static __device__ __forceinline__ float post_one(float x, float u, float a, float coeff, float b,
-                                                 int cautious) {
-  if (cautious) {
-    // mask = min(sign(x*u) + 1, 1): 0 only where x*u < 0  (dion/muon.py:333-340)
-    const float mask = (x * u < 0.f) ? 0.f : 1.f;
-    x = __fsub_rn(x, __fmul_rn(__fmul_rn(x, mask), coeff));
-  } else {
-    x = __fmul_rn(x, a);
-  }
-  return __fsub_rn(x, __fmul_rn(u, b));
-}
-
 template <typename UT, typename XT, bool VEC>
 __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __restrict__ U,
                                                         int64_t numel, int cols,
@@ -361,14 +349,14 @@ __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __re
       }
       st_load8<XT>(x, i, xv);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) xv[e] = post_one(xv[e], uv[e], a, coeff, b, cautious);
+      for (int e = 0; e < 8; ++e) xv[e] = muon_post_one(xv[e], uv[e], a, coeff, b, cautious);
       st_store8<XT>(x, i, xv);
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
       float uv = st_load<UT>(u, i);
       if (rs) uv = __fmul_rn(uv, rs[i / cols]);
-      st_store<XT>(x, i, post_one(st_load<XT>(x, i), uv, a, coeff, b, cautious));
+      st_store<XT>(x, i, muon_post_one(st_load<XT>(x, i), uv, a, coeff, b, cautious));
     }
   }
 }

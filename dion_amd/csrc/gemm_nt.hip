@@ -21,6 +21,8 @@
 // (TileCfg::VG); XOR swizzles keep the LDS writes and the fragment reads bank-conflict free.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace dion {
@@ -128,8 +130,87 @@ __device__ __forceinline__ void pipeline_barrier() {
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
-template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false>
-__global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
+// Parameter accesses of the fused update go through buffer instructions: a descriptor based at the
+// wavefront's tile of X (wave-uniform, scalar registers), a wave-uniform byte offset per instruction
+// (scalar) and one per-lane byte offset shared by all accesses -- no 64-bit address per row in vector
+// registers.  Offsets are 32-bit: the launcher checks that a wavefront tile spans less than 2 GiB.
+typedef __attribute__((ext_vector_type(4))) unsigned bx_u32x4;
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t bx_resource(T* base) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)0xffffffffu, 0x00020000);
+}
+template <typename T>
+__device__ __forceinline__ float bx_load(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int uni_bytes) {
+  if constexpr (sizeof(T) == 2)
+    return bf16_to_f32((bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, lane_bytes, uni_bytes, 0));
+  else return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, lane_bytes, uni_bytes, 0));
+}
+template <typename T>
+__device__ __forceinline__ void bx_store(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int uni_bytes, float v) {
+  if constexpr (sizeof(T) == 2)
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)f32_to_bf16(v), rs, lane_bytes, uni_bytes, 0);
+  else __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rs, lane_bytes, uni_bytes, 0);
+}
+// eight consecutive elements
+template <typename T>
+__device__ __forceinline__ void bx_load8(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int uni_bytes, float v[8]) {
+  if constexpr (sizeof(T) == 2) {
+    const bx_u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_bytes, uni_bytes, 0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[2 * e] = __uint_as_float(w[e] << 16);
+      v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+    }
+  } else {
+    const bx_u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_bytes, uni_bytes, 0);
+    const bx_u32x4 c = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_bytes + 16, uni_bytes, 0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] = __uint_as_float(a[e]);
+      v[4 + e] = __uint_as_float(c[e]);
+    }
+  }
+}
+template <typename T>
+__device__ __forceinline__ void bx_store8(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int uni_bytes,
+                                          const float v[8]) {
+  if constexpr (sizeof(T) == 2) {
+    bx_u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(v[2 * e], v[2 * e + 1]);
+    __builtin_amdgcn_raw_buffer_store_b128(o, rs, lane_bytes, uni_bytes, 0);
+  } else {
+    bx_u32x4 a, c;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      a[e] = __float_as_uint(v[e]);
+      c[e] = __float_as_uint(v[4 + e]);
+    }
+    __builtin_amdgcn_raw_buffer_store_b128(a, rs, lane_bytes, uni_bytes, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(c, rs, lane_bytes + 16, uni_bytes, 0);
+  }
+}
+
+// POST: 0 stores the product; 1 / 2 feed it to the fused Muon update of fp32 / bf16 parameters
+// (HAS_C then means "update X[row][col]", HAS_CT "update X[col][row]"; nothing else is stored).
+template <int POST>
+struct PostSel {
+  typedef NoPost arg;
+  typedef float xt;
+};
+template <>
+struct PostSel<1> {
+  typedef FusedPost arg;
+  typedef float xt;
+};
+template <>
+struct PostSel<2> {
+  typedef FusedPost arg;
+  typedef bf16_t xt;
+};
+
+template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false, int POST = 0>
+__global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, const typename PostSel<POST>::arg post) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, KK = Cfg::KK, NSTAGE = Cfg::NSTAGE;
   constexpr int NM = TM * TN;  // MFMAs per 16-wide k slice
@@ -388,13 +469,74 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
   const bf16_t* Dp = HAS_D ? p.D + (int64_t)b * p.strideD + (int64_t)(row_base + 4 * fhalf) * p.ldd +
                                  col_base + frow
                            : nullptr;
-  bf16_t* Cp = HAS_C ? p.C + (int64_t)b * p.strideC + (int64_t)(row_base + 4 * fhalf) * p.ldc +
-                           col_base + frow
-                     : nullptr;
+  bf16_t* Cp = (HAS_C && POST == 0) ? p.C + (int64_t)b * p.strideC +
+                                           (int64_t)(row_base + 4 * fhalf) * p.ldc + col_base + frow
+                                     : nullptr;
   const int ldd = p.ldd, ldc = p.ldc, ldct = p.ldct;
+  typedef typename PostSel<POST>::xt XT;
+  float pa = 0.f, pcoeff = 0.f, pb = 0.f;
+  int pcautious = 0, pvec = 0;
+  XT* xmat = nullptr;
+  if constexpr (POST != 0) {
+    const float lr = *post.lr_dev;
+    const float wd = post.wd_dev ? *post.wd_dev : post.wd_host;
+    muon_post_coeffs(lr, wd, post.adj_ratio, pa, pcoeff, pb);
+    pcautious = post.cautious;
+    pvec = post.vec_ok;
+    const int pi = b / post.mats_per_ptr;
+    xmat = (XT*)post.X.p[pi] + (int64_t)(b - pi * post.mats_per_ptr) * (HAS_C ? p.strideC : p.strideCt);
+  }
   char* stg = lds + wave * Cfg::STG_BYTES;
   const bool on_diag = p.tri && ti == tj && p.diag != 0.0f;
   if (HAS_CT) __syncthreads();  // every wavefront is done with the operand ring
+
+  if constexpr (POST != 0 && HAS_C) {
+    // Update X[row][col] from registers.  The products are rounded to bf16 first, two per register,
+    // which frees half of the accumulator registers: the parameter values of half a wavefront tile
+    // are then loaded in one go (one round trip to memory per half, not one per 32x32 tile).
+    // 32 lanes x one element: a 128-byte (fp32) or 64-byte (bf16) run of X per row.
+    uint32_t pk[TM][TN][8];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+          pk[i][j][q] = pack_bf16x2(alpha * acc[i][j][2 * q], alpha * acc[i][j][2 * q + 1]);
+    const __amdgpu_buffer_rsrc_t xr = bx_resource(xmat + (int64_t)row_base * ldc + col_base);
+    const int xl = (4 * fhalf * ldc + frow) * (int)sizeof(XT);  // per lane
+    constexpr int HM = TM >= 2 ? TM / 2 : 1;
+    auto run = [&](auto caut) {
+      constexpr int CAUT = decltype(caut)::value;
+#pragma unroll
+      for (int i0 = 0; i0 < TM; i0 += HM) {
+        float xv[HM][TN][16];
+#pragma unroll
+        for (int ii = 0; ii < HM; ++ii)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              xv[ii][j][r] = bx_load<XT>(
+                  xr, xl, (((i0 + ii) * 32 + (r >> 2) * 8 + (r & 3)) * ldc + j * 32) * (int)sizeof(XT));
+#pragma unroll
+        for (int ii = 0; ii < HM; ++ii)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const uint32_t w = pk[i0 + ii][j][r >> 1];
+              const float u = __uint_as_float((r & 1) ? (w & 0xffff0000u) : (w << 16));
+              bx_store<XT>(xr, xl, (((i0 + ii) * 32 + (r >> 2) * 8 + (r & 3)) * ldc + j * 32) * (int)sizeof(XT),
+                           muon_post_one(xv[ii][j][r], u, pa, pcoeff, pb, CAUT));
+            }
+        asm volatile("" ::: "memory");  // the next batch of loads stays behind these stores
+      }
+    };
+    if (pcautious) run(std::integral_constant<int, 1>());
+    else run(std::integral_constant<int, 0>());
+    return;
+  }
 
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -418,7 +560,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
         for (int r = 0; r < 16; ++r)
           if (dcol == (r >> 2) * 8 + (r & 3)) v[r] += p.diag;
       }
-      if (HAS_C) {
+      if (HAS_C && POST == 0) {
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           Cp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldc + j * 32] = f32_to_bf16(v[r]);
@@ -439,12 +581,61 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p) {
       constexpr int CH = Cfg::WTM / 8;  // 16-byte chunks per staged row
       constexpr int RPI = 64 / CH;      // staged rows per store instruction
       const int srow = lane / CH, schunk = lane % CH;
-      bf16_t* Ctp = p.Ct + (int64_t)b * p.strideCt + (int64_t)(col_base + srow) * ldct + row_base + schunk * 8;
       const char* sp = stg + srow * Cfg::STG_PITCH + schunk * 16;
+      if constexpr (POST != 0) {
+        // the staged bf16 tile is the update; 8 consecutive elements of X per lane, the parameter values
+        // of up to eight staged rows loaded in one go
+        const __amdgpu_buffer_rsrc_t xr = bx_resource(xmat + (int64_t)col_base * ldct + row_base);
+        const int xl = (srow * ldct + schunk * 8) * (int)sizeof(XT);  // per lane
+        constexpr int NIT = Cfg::WTN / RPI;
+        constexpr int BI = NIT < 8 ? NIT : 8;
+        static_assert(NIT % BI == 0, "staged rows per wavefront");
+        auto run = [&](auto caut) {
+          constexpr int CAUT = decltype(caut)::value;
+#pragma unroll
+          for (int it0 = 0; it0 < NIT; it0 += BI) {
+            float uv[BI][8], xv[BI][8];
+#pragma unroll
+            for (int k = 0; k < BI; ++k)
+              st_load8<bf16_t>((const bf16_t*)(sp + (it0 + k) * RPI * Cfg::STG_PITCH), 0, uv[k]);
+            if (pvec) {
+#pragma unroll
+              for (int k = 0; k < BI; ++k)
+                bx_load8<XT>(xr, xl, (it0 + k) * RPI * ldct * (int)sizeof(XT), xv[k]);
+            } else {
+#pragma unroll
+              for (int k = 0; k < BI; ++k)
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                  xv[k][e] = bx_load<XT>(xr, xl, ((it0 + k) * RPI * ldct + e) * (int)sizeof(XT));
+            }
+#pragma unroll
+            for (int k = 0; k < BI; ++k)
+#pragma unroll
+              for (int e = 0; e < 8; ++e) xv[k][e] = muon_post_one(xv[k][e], uv[k][e], pa, pcoeff, pb, CAUT);
+            if (pvec) {
+#pragma unroll
+              for (int k = 0; k < BI; ++k)
+                bx_store8<XT>(xr, xl, (it0 + k) * RPI * ldct * (int)sizeof(XT), xv[k]);
+            } else {
+#pragma unroll
+              for (int k = 0; k < BI; ++k)
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                  bx_store<XT>(xr, xl, ((it0 + k) * RPI * ldct + e) * (int)sizeof(XT), xv[k][e]);
+            }
+          }
+        };
+        if (pcautious) run(std::integral_constant<int, 1>());
+        else run(std::integral_constant<int, 0>());
+      } else {
+        bf16_t* Ctp =
+            p.Ct + (int64_t)b * p.strideCt + (int64_t)(col_base + srow) * ldct + row_base + schunk * 8;
 #pragma unroll 8
-      for (int it = 0; it < Cfg::WTN / RPI; ++it) {
-        const uint4 q = *(const uint4*)(sp + it * RPI * Cfg::STG_PITCH);
-        *(uint4*)(Ctp + (int64_t)(it * RPI) * ldct) = q;
+        for (int it = 0; it < Cfg::WTN / RPI; ++it) {
+          const uint4 q = *(const uint4*)(sp + it * RPI * Cfg::STG_PITCH);
+          *(uint4*)(Ctp + (int64_t)(it * RPI) * ldct) = q;
+        }
       }
     }
   }
@@ -458,17 +649,18 @@ typedef TileCfg<256, 256, 32, 2, 4, 4> Cfg256w8k32;  // 8 wavefronts, 4 x 32-dee
 typedef TileCfg<256, 256, 64, 2, 4, 2, true> Cfg256w8vg;  // 8 wavefronts, register-staged operands
 typedef TileCfg<128, 128, 64, 2, 2, 2, true> Cfg128vg;
 
-template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false>
-static hipError_t launch_epi(const GemmParams& p, hipStream_t stream) {
+template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false, int POST = 0>
+static hipError_t launch_epi(const GemmParams& p, hipStream_t stream,
+                             const typename PostSel<POST>::arg& post = typename PostSel<POST>::arg()) {
   static std::atomic<uint64_t> attr_done{0};
-  auto kern = gemm_nt_kernel<Cfg, HAS_D, HAS_C, HAS_CT, QK>;
+  auto kern = gemm_nt_kernel<Cfg, HAS_D, HAS_C, HAS_CT, QK, POST>;
   if (hipError_t e = set_max_dynamic_lds_once((const void*)kern, Cfg::LDS_BYTES, attr_done)) return e;
   const int tilesM = p.M / Cfg::BM, tilesN = p.N / Cfg::BN;
   const int64_t per_mat = p.tri ? (int64_t)tilesM * (tilesM + 1) / 2 : (int64_t)tilesM * tilesN;
   const int64_t total = per_mat * p.batch;
   if (total <= 0) return hipSuccess;
   if (total > 0x7fffffff) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, post);
   return hipGetLastError();
 }
 
@@ -500,17 +692,45 @@ int gemm_pad_granule(int m, int n, int batch) {
   return syrk_tiles >= 256 ? 256 : 128;
 }
 
+// 256-wide tiles only when there are enough of them to keep 256 CUs busy for a few rounds; below that
+// the 128-wide tiles (two workgroups per CU) win.
+static bool wants_256_tiles(const GemmParams& p) {
+  static const long thresh = [] {
+    const char* e = getenv("DION_TILE_THRESH");
+    return e ? atol(e) : 512L;
+  }();
+  const long t256 = (long)(p.M / 256) * (p.tri ? (p.M / 256 + 1) / 2 + 0 : p.N / 256) * p.batch;
+  return p.M % 256 == 0 && p.N % 256 == 0 && t256 >= thresh;
+}
+
+template <class Cfg>
+static hipError_t launch_post_cfg(const GemmParams& p, const FusedPost& post, int x_dtype, bool transposed,
+                                  hipStream_t stream) {
+  if (p.M % Cfg::BM || p.N % Cfg::BN || p.K % (Cfg::BK * Cfg::NSTAGE)) return hipErrorInvalidValue;
+  if (x_dtype == 1) {
+    return transposed ? launch_epi<Cfg, false, false, true, true, 1>(p, stream, post)
+                      : launch_epi<Cfg, false, true, false, true, 1>(p, stream, post);
+  }
+  return transposed ? launch_epi<Cfg, false, false, true, true, 2>(p, stream, post)
+                    : launch_epi<Cfg, false, true, false, true, 2>(p, stream, post);
+}
+
+hipError_t launch_gemm_nt_post(const GemmParams& p, const FusedPost& post, int x_dtype, bool transposed,
+                               hipStream_t stream) {
+  if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.batch <= 0) return hipSuccess;
+  // the epilogue addresses a wavefront tile of X (at most 128 rows) with 32-bit byte offsets
+  if ((int64_t)(transposed ? p.ldct : p.ldc) * 129 * 4 > 0x7fffffffLL) return hipErrorInvalidValue;
+  if (!p.q_kmajor || p.tri || p.D || post.mats_per_ptr <= 0 || !post.lr_dev ||
+      p.batch > (int64_t)kMaxPtrs * post.mats_per_ptr || (x_dtype != 0 && x_dtype != 1))
+    return hipErrorInvalidValue;
+  return wants_256_tiles(p) ? launch_post_cfg<Cfg256w8vg>(p, post, x_dtype, transposed, stream)
+                            : launch_post_cfg<Cfg128vg>(p, post, x_dtype, transposed, stream);
+}
+
 hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.batch <= 0) return hipSuccess;
   if (variant < 0) {
-    // 256-wide tiles only when there are enough of them to keep 256 CUs busy for a few rounds;
-    // below that the 128-wide tiles (two workgroups per CU) win.
-    static const long thresh = [] {
-      const char* e = getenv("DION_TILE_THRESH");
-      return e ? atol(e) : 512L;
-    }();
-    const long t256 = (long)(p.M / 256) * (p.tri ? (p.M / 256 + 1) / 2 + 0 : p.N / 256) * p.batch;
-    variant = (p.M % 256 == 0 && p.N % 256 == 0 && t256 >= thresh) ? 3 : 1;
+    variant = wants_256_tiles(p) ? 3 : 1;
     // Tuning knob: DION_GEMM_VARIANT overrides the 256-wide tile configuration.
     static const int forced = [] {
       const char* e = getenv("DION_GEMM_VARIANT");

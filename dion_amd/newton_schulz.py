@@ -70,6 +70,27 @@ def zeropower_kj(G: Tensor, steps: int = 5, eps: Union[float, Tensor] = 1e-7) ->
     return ops.ns_orthogonalize(G, [KJ_COEFFS] * int(steps), 1.0, _eps(eps, 1e-7))
 
 
+# What each built-in operator runs, as arguments of ``ops.ns_orthogonalize`` /
+# ``ops.ns_orthogonalize_update``: (coeffs, norm_scale, default epsilon, gram, gram_reset).  A fixed
+# epsilon of None means the caller's epsilon is ignored (the Gram form).
+SCHEDULES = {
+    zeropower_via_newtonschulz5: (NS5_COEFFS, 1.0, 1e-7, False, 0),
+    polar_express: (POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 1e-6, False, 0),
+    gram_newton_schulz: (POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, None, True, 2),
+}
+
+
+@torch.no_grad()
+def orthogonalize_update(func, G: Tensor, epsilon, X, lr: Tensor, adj_ratio: float, weight_decay,
+                         cautious_wd: bool = False) -> None:
+    """``ops.muon_post(X, func(G, epsilon), ...)`` for a built-in ``func`` (a key of ``SCHEDULES``), as one
+    fused library call."""
+    coeffs, norm_scale, default_eps, gram, reset = SCHEDULES[func]
+    eps = 0.0 if default_eps is None else _eps(epsilon, default_eps)
+    ops.ns_orthogonalize_update(G, X, coeffs, norm_scale, eps, lr, adj_ratio, weight_decay, cautious_wd,
+                                gram=gram, gram_reset=reset)
+
+
 # The reference exposes Triton-backed twins of the two schedules; here there is one
 # implementation, so the names resolve to it.
 newton_schulz_triton = zeropower_via_newtonschulz5

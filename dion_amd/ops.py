@@ -186,11 +186,7 @@ def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: f
     out = torch.empty(batch, rows, cols, dtype=torch.bfloat16, device=G.device)
     if out.numel() == 0:
         return out.reshape(shape)
-    flat = [float(v) for abc in coeffs for v in abc]
-    if len(flat) % 3:
-        raise ValueError("coeffs must be (a, b, c) triples")
-    n_iters = len(flat) // 3
-    carr = (_lib.ctypes.c_float * max(1, len(flat)))(*flat)
+    carr, n_iters = _flat_coeffs(coeffs)
     flags = (DION_NS_GRAM if gram else 0) | (DION_NS_CARRY_XT if carry_xt else 0)
     lib = _lib.load()
     chunk = 32768  # one library call takes at most 65535 matrices
@@ -203,6 +199,54 @@ def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: f
                                         int(gram_reset), ws.data_ptr(), ws.numel(), _stream_handle(G.device)),
               "ns_orthogonalize")
     return out.reshape(shape)
+
+
+def _flat_coeffs(coeffs):
+    flat = [float(v) for abc in coeffs for v in abc]
+    if len(flat) % 3:
+        raise ValueError("coeffs must be (a, b, c) triples")
+    return (_lib.ctypes.c_float * max(1, len(flat)))(*flat), len(flat) // 3
+
+
+def ns_orthogonalize_update(G: Tensor, X: List[Tensor], coeffs: Sequence[Sequence[float]], norm_scale: float,
+                            epsilon: float, lr: Tensor, adj_ratio: float, weight_decay, cautious_wd: bool = False,
+                            gram: bool = False, gram_reset: int = 0, carry_xt: bool = False) -> None:
+    """``muon_post(X, ns_orthogonalize(G, ...), lr, adj_ratio, weight_decay, cautious_wd)`` in one library
+    call, with the same result bit for bit (dion/muon.py:249-277).  ``G`` is ``[..., rows, cols]`` with
+    ``len(X) * mats`` matrices; every ``X[i]`` is a contiguous fp32 or bf16 parameter of ``mats * rows *
+    cols`` elements laid out as ``[mats, rows, cols]``.  When the matrices fill whole tiles the update runs in
+    the epilogue of the last GEMM and the orthogonalized matrices never reach memory."""
+    _require_gpu(G, "G")
+    if G.ndim < 2:
+        raise ValueError(f"expected a tensor with at least 2 dims, got shape {tuple(G.shape)}")
+    n = len(X)
+    if n == 0:
+        raise ValueError("X is empty")
+    if G.dtype not in (torch.bfloat16, torch.float32):
+        G = G.to(torch.float32)
+    rows, cols = G.shape[-2], G.shape[-1]
+    G3 = G.reshape(-1, rows, cols).contiguous()
+    batch = G3.shape[0]
+    if batch == 0 or rows * cols == 0:
+        return
+    if batch % n:
+        raise ValueError(f"{batch} matrices do not divide over {n} parameters")
+    mats_per_ptr = batch // n
+    xp, xcode = _state_ptrs(X, "X", mats_per_ptr * rows * cols)
+    lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, G.device)
+    if batch > 32768:  # past one library call: the two-pass form, which splits the batch
+        O = ns_orthogonalize(G3, coeffs, norm_scale, epsilon, gram, gram_reset, carry_xt)
+        muon_post(X, O.view(n, -1), lr, adj_ratio, weight_decay, cautious_wd)
+        return
+    carr, n_iters = _flat_coeffs(coeffs)
+    flags = (DION_NS_GRAM if gram else 0) | (DION_NS_CARRY_XT if carry_xt else 0)
+    lib = _lib.load()
+    ws = _workspace(G.device, lib.dion_ns_update_workspace_bytes(batch, rows, cols, flags, n_iters))
+    check(lib.dion_ns_orthogonalize_update(G3.data_ptr(), _dtype_code(G3, "G"), xp, xcode, n, mats_per_ptr, rows,
+                                           cols, carr, n_iters, float(norm_scale), float(epsilon), flags,
+                                           int(gram_reset), lr_p, float(adj_ratio), wd_p, wd_h,
+                                           int(bool(cautious_wd)), ws.data_ptr(), ws.numel(),
+                                           _stream_handle(G.device)), "ns_orthogonalize_update")
 
 
 # ---------------------------------------------------------------------------------------------

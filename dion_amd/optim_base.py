@@ -358,6 +358,15 @@ class OrthoOptimizer(Optimizer):
             out = out.reshape(U.shape).to(torch.bfloat16).contiguous()
         return out
 
+    def _orthogonalize_update(self, U: Tensor, epsilon: float, X: List[Tensor], lr: Tensor, adj_ratio: float,
+                              weight_decay, cautious_wd: bool) -> bool:
+        """Orthogonalize ``U`` and apply the Muon update to ``X`` in one library call; False (nothing done)
+        when a caller-supplied orthogonalization is in use, which has to run on its own."""
+        if self._custom_ns or self._newton_schulz_func not in ns.SCHEDULES:
+            return False
+        ns.orthogonalize_update(self._newton_schulz_func, U, epsilon, X, lr, adj_ratio, weight_decay, cautious_wd)
+        return True
+
     def _orthogonalize_row_blocks(self, U: Tensor, split_sizes, split_scales, epsilon: float) -> Tensor:
         """Row blocks of dim -2 are orthogonalized independently, equal-height blocks batched into
         one call, each rescaled by its ``split_scales`` entry (dion/megabatch_base.py:911-949)."""

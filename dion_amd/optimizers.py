@@ -3,7 +3,7 @@ contract of microsoft/dion (dion/muon.py:20-110, dion/normuon.py:20-133, dion/di
 dion/nordion2.py:26-136), executing on the hand-written gfx950 kernels.
 
 Per shape group (all parameters of one shape and dtype) a step is:
-  Muon     muon_pre -> orthogonalize -> muon_post
+  Muon     muon_pre -> orthogonalize + update (one call; the last GEMM applies the update)
   NorMuon  muon_pre -> orthogonalize -> normuon_stats -> muon_post(row_scale)
   Dion2    dion2_select -> orthogonalize(selected slices) -> dion2_post
   NorDion2 dion2_select(rows) -> orthogonalize -> normuon_stats_selected -> dion2_post(row_scale)
@@ -53,6 +53,8 @@ class _MomentumOrtho(OrthoOptimizer):
     """Shared Muon / NorMuon shape-group update (dion/muon.py:194-280, dion/normuon.py:222-341)."""
 
     _normalize = False
+    # Muon only: run orthogonalization and update as one library call (False: the two-call sequence)
+    fused_update = True
 
     def _shape_group_phases(self, group: dict, params: List[Tensor]):
         """Generator: [momentum / cast] yield [orthogonalization GEMMs] yield [normalise / update]."""
@@ -83,6 +85,15 @@ class _MomentumOrtho(OrthoOptimizer):
         yield
         _note_stream(U)
 
+        ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
+        if not self._normalize and split_sizes is None and self.fused_update:
+            # Muon proper: the update consumes the orthogonalized matrices where the last GEMM
+            # produces them (same result as the two calls below, bit for bit)
+            Uv = U.view(n, shape[0], -1) if flatten and len(shape) >= 3 else U.view(n * mats, rows, cols)
+            if self._orthogonalize_update(Uv, eps, X, group["lr"], ratio, group["weight_decay"],
+                                          group["cautious_wd"]):
+                return
+
         # shape plumbing of muon_update_newton_schulz (dion/megabatch_base.py:884-908)
         if split_sizes is not None:
             O = self._orthogonalize_row_blocks(U, split_sizes, split_scales, eps).contiguous()
@@ -95,7 +106,6 @@ class _MomentumOrtho(OrthoOptimizer):
         yield
         _note_stream(O)
 
-        ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
         row_scale = None
         if self._normalize:
             V = [s["variance_neuron"] for s in states]

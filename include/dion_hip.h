@@ -86,6 +86,23 @@ int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, in
                           const float* coeffs, int n_iters, float norm_scale, float eps, int flags,
                           int gram_reset, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Orthogonalization and Muon update in one call: what dion_ns_orthogonalize followed by dion_muon_post
+ * (bf16 update, no row_scale) does to the parameters, bit for bit, without the pass that writes the
+ * orthogonalized matrices and the pass that reads them back.  Replaces the pair
+ * `muon_update_newton_schulz` + `muon_update_post_orthogonalize`, dion/muon.py:249-277.
+ * in: [n_ptrs * mats_per_ptr, rows, cols] as for dion_ns_orthogonalize; X_ptrs: host array of n_ptrs
+ * device pointers, each to mats_per_ptr contiguous [rows, cols] matrices of x_dtype, updated in place.
+ * When the matrices fill whole tiles (rows, cols multiples of 128; X-only form; more than 64 rows or
+ * columns on the short side) the last GEMM applies the update in its epilogue; otherwise the library
+ * runs the two passes itself, through the tail of the workspace.  Workspace size from
+ * dion_ns_update_workspace_bytes (same flags and n_iters).  lr / weight decay as for dion_muon_post. */
+size_t dion_ns_update_workspace_bytes(int batch, int rows, int cols, int flags, int n_iters);
+int dion_ns_orthogonalize_update(const void* in, int in_dtype, const uint64_t* X_ptrs, int x_dtype, int n_ptrs,
+                                 int mats_per_ptr, int rows, int cols, const float* coeffs, int n_iters,
+                                 float norm_scale, float eps, int flags, int gram_reset, const float* lr_dev,
+                                 float adj_ratio, const float* wd_dev, float wd_host, int cautious,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+
 /* --------------------------------------------------------------------------------------------
  * Memory-bound fused kernels of the optimizer step.
  * Optimizer state -- parameters X, momentum M, second moments V -- is fp32 or bf16 in memory, as the
