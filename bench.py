@@ -39,6 +39,8 @@ WORKLOADS = {
                          ("down", 4096, 14336, 4)],
     # the headline shape group on its own
     "ns_4096x14336": [("down", 4096, 14336, 32)],
+    # a single 768x3072 matrix (the reference's CPU-runnable case): pure launch latency on a GPU
+    "one_768x3072": [("proj", 768, 3072, 1)],
     # GPT-small with per-head Newton-Schulz on the fused qkv weight (36 heads of 64x768 per layer)
     "gpt_small_heads": [("qkv", 2304, 768, 12), ("attn_out", 768, 768, 12), ("fc", 3072, 768, 12),
                         ("proj", 768, 3072, 12)],
@@ -247,6 +249,8 @@ def main() -> int:
         B, m, n = 32, 4096, 14336
         if args.workload in ("gpt_small", "gpt_small_heads"):
             B, m, n = 12, 768, 3072
+        elif args.workload == "one_768x3072":
+            B, m, n = 1, 768, 3072
         elif args.workload == "gpt_1p3b":
             B, m, n = 24, 2048, 8192
         st = torch.cuda.current_stream().cuda_stream
