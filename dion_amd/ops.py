@@ -323,7 +323,7 @@ def muon_post(X: List[Tensor], U: Tensor, lr: Tensor, adj_ratio: float, weight_d
 
 
 def normuon_stats(U: Tensor, V: List[Tensor], beta2: float) -> Tensor:
-    """Updates every ``V[i]`` (``[..., rows, 1]`` fp32) in place from the orthogonalized arena
+    """Updates every ``V[i]`` (``[..., rows, 1]``, fp32 or bf16) in place from the orthogonalized arena
     ``U [N, ..., rows, cols]`` and returns the per-row scales ``[n_mat, rows]`` that turn ``U`` into the
     NorMuon-normalised update.  Mirrors ``normuon_normalization_stacked`` (dion/normuon.py:345-399)."""
     n = len(V)
@@ -342,7 +342,7 @@ def normuon_stats(U: Tensor, V: List[Tensor], beta2: float) -> Tensor:
 
 def normuon_stats_selected(U: Tensor, V: List[Tensor], idx: Tensor, beta2: float) -> Tensor:
     """NorMuon statistics for an update made of ``k`` selected rows per matrix: ``U [N, ..., k, cols]``
-    bf16, ``idx [n_mat, k]`` int32 (rows of the parameter), ``V[i]`` the full ``[..., rows, 1]`` fp32
+    bf16, ``idx [n_mat, k]`` int32 (rows of the parameter), ``V[i]`` the full ``[..., rows, 1]`` fp32 or bf16
     buffers, of which only the selected entries are read and updated.  Returns the per-row scales
     ``[n_mat, k]``.  Mirrors ``nordion2_normalize_selected_stacked`` (dion/nordion2.py:430-447)."""
     n = len(V)
@@ -455,7 +455,7 @@ def dion2_index_map(indices: Tensor, dim: int) -> Tensor:
 def dion2_post_orthogonalize_triton(X: List[Tensor], U: List[Tensor], indices: List[Tensor], base_lr: Tensor,
                                     adjusted_lr: Tensor, weight_decay, select_dim: int) -> None:
     """Same call as the reference's ``dion2_post_orthogonalize_triton`` (dion/dion2_triton.py:147-155):
-    per tensor ``x`` ``[*leading, M, N]`` fp32 contiguous, ``u`` the selected slices (bf16 or fp32),
+    per tensor ``x`` ``[*leading, M, N]`` fp32 or bf16, contiguous, ``u`` the selected slices (bf16 or fp32),
     ``indices [*leading, k]`` int64; ``selected: x = (1 - base_lr*wd)*x - adjusted_lr*u``, unselected:
     ``x = (1 - base_lr*wd)*x``.  ``base_lr`` / ``adjusted_lr`` are 0-d fp32 device tensors read in the
     kernel.  Empty tensors are skipped; non-contiguous ``x`` raises ``ValueError``."""
