@@ -15,7 +15,7 @@ DION_BF16 = 0
 DION_F32 = 1
 DION_NS_GRAM = 1
 DION_NS_CARRY_XT = 2
-ABI_VERSION = 8  # dion_abi_version() of the library these signatures describe
+ABI_VERSION = 9  # dion_abi_version() of the library these signatures describe
 
 _u64p = ctypes.POINTER(ctypes.c_uint64)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -37,7 +37,8 @@ SIGNATURES = {
                                              c_int, c_float, c_float, c_int, c_int, c_void_p, c_float, c_void_p,
                                              c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "dion_muon_pre": (c_int, [_u64p, c_int, _u64p, c_int, c_void_p, c_int, c_int64, c_float, c_int, c_void_p]),
-    "dion_muon_post": (c_int, [_u64p, c_int, c_void_p, c_int, c_int, c_int64, c_int, c_void_p, c_void_p,
+    "dion_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_void_p]),
+    "dion_muon_post": (c_int, [_u64p, c_int, c_void_p, c_int, c_int, c_int64, c_int, c_void_p, c_void_p, c_void_p,
                                c_float, c_void_p, c_float, c_int, c_void_p]),
     "dion_normuon_stats": (c_int, [c_void_p, _u64p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p,
                                    c_void_p]),

@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 8; }
+extern "C" int dion_abi_version(void) { return 9; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -545,7 +545,7 @@ extern "C" int dion_ns_orthogonalize_update(const void* in, int in_dtype, const 
                       workspace, ns, stream, nullptr))
     return rc;
   return dion_muon_post(X_ptrs, x_dtype, tmp, DION_BF16, n_ptrs, (int64_t)mats_per_ptr * rows * cols, cols,
-                        nullptr, lr_dev, adj_ratio, wd_dev, wd_host, cautious, stream);
+                        nullptr, lr_dev, nullptr, adj_ratio, wd_dev, wd_host, cautious, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -593,8 +593,8 @@ extern "C" int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t
 
 extern "C" int dion_muon_post(const uint64_t* X_ptrs, int x_dtype, const void* U, int u_dtype, int n,
                               int64_t numel, int cols, const float* row_scale, const float* lr_dev,
-                              float adj_ratio, const float* wd_dev, float wd_host, int cautious,
-                              void* stream) {
+                              const float* adj_lr_dev, float adj_ratio, const float* wd_dev, float wd_host,
+                              int cautious, void* stream) {
   if (n < 0 || numel < 0 || cols <= 0) return fail(DION_E_INVALID, "dion_muon_post: bad size");
   if (int rc = check_state_dtype("dion_muon_post", "x_dtype", x_dtype)) return rc;
   if (u_dtype != DION_BF16 && u_dtype != DION_F32) return fail(DION_E_INVALID, "dion_muon_post: u_dtype");
@@ -611,10 +611,21 @@ extern "C" int dion_muon_post(const uint64_t* X_ptrs, int x_dtype, const void* U
     fill_tab(x, X_ptrs + i0, c);
     HIP_TRY(launch_muon_post(x, dt(x_dtype), (const char*)U + (size_t)i0 * numel * usz, dt(u_dtype), c, numel,
                              cols,
-                             row_scale ? row_scale + (int64_t)i0 * rows : nullptr, lr_dev, adj_ratio,
-                             wd_dev, wd_host, cautious, vec, (hipStream_t)stream),
+                             row_scale ? row_scale + (int64_t)i0 * rows : nullptr, lr_dev, adj_lr_dev,
+                             adj_ratio, wd_dev, wd_host, cautious, vec, (hipStream_t)stream),
             "dion_muon_post");
   }
+  return DION_OK;
+}
+
+extern "C" int dion_scale_rows(const void* U, const float* scale, void* out, int out_dtype, int64_t n_rows,
+                               int cols, void* stream) {
+  if (int rc = check_state_dtype("dion_scale_rows", "out_dtype", out_dtype)) return rc;
+  if (n_rows < 0 || cols < 0 || n_rows > 0x7fffffff) return fail(DION_E_INVALID, "dion_scale_rows: bad size");
+  if (n_rows == 0 || cols == 0) return DION_OK;
+  if (!U || !scale || !out) return fail(DION_E_INVALID, "dion_scale_rows: null argument");
+  HIP_TRY(launch_scale_rows((const bf16_t*)U, scale, out, dt(out_dtype), n_rows, cols, (hipStream_t)stream),
+          "dion_scale_rows");
   return DION_OK;
 }
 

@@ -31,9 +31,11 @@ hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* d
 hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, bf16_t* U, int n,
                            int64_t numel, float mu, int nesterov, bool vec, hipStream_t st);
 hipError_t launch_muon_post(const PtrTab& X, int x_dtype, const void* U, int u_dtype, int n, int64_t numel,
-                            int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
-                            const float* wd_dev, float wd_host, int cautious, bool vec,
+                            int cols, const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
+                            float adj_ratio, const float* wd_dev, float wd_host, int cautious, bool vec,
                             hipStream_t st);
+hipError_t launch_scale_rows(const bf16_t* U, const float* scale, void* out, int out_dtype, int64_t n_rows,
+                             int cols, hipStream_t st);
 hipError_t launch_normuon_stats(const bf16_t* U, const PtrTab& V, int v_dtype, int n_mat, int mats_per_ptr,
                                 int rows, int cols, const int32_t* row_idx, int v_rows, float w,
                                 float* row_scale, hipStream_t st);

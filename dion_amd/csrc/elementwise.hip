@@ -323,6 +323,7 @@ __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __re
                                                         int64_t numel, int cols,
                                                         const float* __restrict__ row_scale,
                                                         const float* __restrict__ lr_dev,
+                                                        const float* __restrict__ adj_lr_dev,
                                                         float adj_ratio,
                                                         const float* __restrict__ wd_dev,
                                                         float wd_host, int cautious) {
@@ -333,7 +334,7 @@ __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __re
   const float wd = wd_dev ? *wd_dev : wd_host;
   const float coeff = __fmul_rn(lr, wd);
   const float a = __fsub_rn(1.0f, coeff);
-  const float b = __fmul_rn(lr, adj_ratio);
+  const float b = adj_lr_dev ? *adj_lr_dev : __fmul_rn(lr, adj_ratio);
   const int64_t rows = numel / cols;
   const float* rs = row_scale ? row_scale + (int64_t)p * rows : nullptr;
   const int64_t stride = (int64_t)gridDim.x * 256;
@@ -362,13 +363,13 @@ __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __re
 }
 
 hipError_t launch_muon_post(const PtrTab& X, int x_dtype, const void* U, int u_dtype, int n, int64_t numel,
-                            int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
-                            const float* wd_dev, float wd_host, int cautious, bool vec,
+                            int cols, const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
+                            float adj_ratio, const float* wd_dev, float wd_host, int cautious, bool vec,
                             hipStream_t st) {
   dim3 grid(ew_blocks(vec ? (numel >> 3) : numel), n);
 #define POST_LAUNCH(UT, XT, V)                                                                      \
   hipLaunchKernelGGL((muon_post_kernel<UT, XT, V>), grid, dim3(256), 0, st, X, (const UT*)U, numel, \
-                     cols, row_scale, lr_dev, adj_ratio, wd_dev, wd_host, cautious)
+                     cols, row_scale, lr_dev, adj_lr_dev, adj_ratio, wd_dev, wd_host, cautious)
 #define POST_LAUNCH_X(UT, V) \
   do { if (x_dtype == 0) POST_LAUNCH(UT, bf16_t, V); else POST_LAUNCH(UT, float, V); } while (0)
   if (u_dtype == 0) {
@@ -378,6 +379,34 @@ hipError_t launch_muon_post(const PtrTab& X, int x_dtype, const void* U, int u_d
   }
 #undef POST_LAUNCH_X
 #undef POST_LAUNCH
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// out[row][:] = U[row][:] * scale[row]: the normalised update itself, for callers that want it as a
+// tensor (the optimizers fold the scale into the update kernels instead).
+// ------------------------------------------------------------------------------------------
+template <typename OT>
+__global__ __launch_bounds__(256) void scale_rows_kernel(const bf16_t* __restrict__ U,
+                                                         const float* __restrict__ scale,
+                                                         OT* __restrict__ out, int cols) {
+  const int64_t row = blockIdx.x;
+  const float s = scale[row];
+  const bf16_t* u = U + row * cols;
+  OT* o = out + row * cols;
+  for (int c = threadIdx.x; c < cols; c += 256) st_store<OT>(o, c, __fmul_rn(bf16_to_f32(u[c]), s));
+}
+
+hipError_t launch_scale_rows(const bf16_t* U, const float* scale, void* out, int out_dtype, int64_t n_rows,
+                             int cols, hipStream_t st) {
+  if (n_rows <= 0 || cols <= 0) return hipSuccess;
+  if (n_rows > 0x7fffffff) return hipErrorInvalidValue;
+  if (out_dtype == 0)
+    hipLaunchKernelGGL((scale_rows_kernel<bf16_t>), dim3((unsigned)n_rows), dim3(256), 0, st, U, scale,
+                       (bf16_t*)out, cols);
+  else
+    hipLaunchKernelGGL((scale_rows_kernel<float>), dim3((unsigned)n_rows), dim3(256), 0, st, U, scale,
+                       (float*)out, cols);
   return hipGetLastError();
 }
 

@@ -299,10 +299,11 @@ def muon_pre(G: List[Tensor], M: List[Tensor], momentum: float, nesterov: bool) 
 
 
 def muon_post(X: List[Tensor], U: Tensor, lr: Tensor, adj_ratio: float, weight_decay, cautious_wd: bool = False,
-              row_scale: Optional[Tensor] = None) -> None:
+              row_scale: Optional[Tensor] = None, adjusted_lr: Optional[Tensor] = None) -> None:
     """In-place weight decay + update of every ``X[i]`` from the arena ``U[i]``.  Mirrors
     ``muon_update_post_orthogonalize`` (dion/muon.py:315-347); ``row_scale`` folds NorMuon's
-    per-row normalisation into the same pass."""
+    per-row normalisation into the same pass; ``adjusted_lr`` (0-d fp32 device tensor) replaces
+    ``lr * adj_ratio`` in the update term."""
     n = len(X)
     assert n > 0 and U.shape[0] == n
     numel = X[0].numel()
@@ -316,10 +317,32 @@ def muon_post(X: List[Tensor], U: Tensor, lr: Tensor, adj_ratio: float, weight_d
         if row_scale.dtype != torch.float32 or row_scale.numel() != n * (numel // cols):
             raise ValueError("row_scale must be float32 [N, rows]")
         rs_p = row_scale.data_ptr()
+    alr = None
+    if adjusted_lr is not None:
+        if not (adjusted_lr.is_cuda and adjusted_lr.dtype == torch.float32 and adjusted_lr.numel() == 1):
+            raise TypeError("adjusted_lr must be a 0-d float32 GPU tensor")
+        alr = adjusted_lr.data_ptr()
     lib = _lib.load()
-    check(lib.dion_muon_post(xp, xcode, U.data_ptr(), _dtype_code(U, "U"), n, numel, cols, rs_p, lr_p,
+    check(lib.dion_muon_post(xp, xcode, U.data_ptr(), _dtype_code(U, "U"), n, numel, cols, rs_p, lr_p, alr,
                              float(adj_ratio), wd_p, wd_h, int(bool(cautious_wd)),
                              _stream_handle(U.device)), "muon_post")
+
+
+def scale_rows(U: Tensor, scale: Tensor, dtype: torch.dtype) -> Tensor:
+    """``U[..., r, :] * scale[r]`` for a contiguous bf16 ``U [..., rows, cols]`` and fp32 ``scale`` with one
+    entry per row of ``U``; result in ``dtype`` (float32 or bfloat16)."""
+    _check_bf16(U, "U")
+    if not U.is_contiguous():
+        raise ValueError("U must be contiguous")
+    cols = U.shape[-1]
+    n_rows = U.numel() // cols if cols else 0
+    if scale.dtype != torch.float32 or not scale.is_contiguous() or scale.numel() != n_rows or not scale.is_cuda:
+        raise ValueError("scale must be a contiguous float32 GPU tensor with one entry per row of U")
+    out = torch.empty(U.shape, dtype=dtype, device=U.device)
+    lib = _lib.load()
+    check(lib.dion_scale_rows(U.data_ptr(), scale.data_ptr(), out.data_ptr(), _dtype_code(out, "out"), n_rows,
+                              cols, _stream_handle(U.device)), "scale_rows")
+    return out
 
 
 def normuon_stats(U: Tensor, V: List[Tensor], beta2: float) -> Tensor:

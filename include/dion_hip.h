@@ -127,10 +127,19 @@ int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, i
  * which case wd_host is used.  U is the [n, numel] arena, bf16 or fp32 per u_dtype.
  * row_scale (nullable): device [n, rows] fp32; U[i][r][:] is multiplied by row_scale[i][r]
  * first, rows = numel / cols (used by NorMuon).  X per x_dtype.
+ * adj_lr_dev (nullable): device float that replaces lr * adj_ratio in the update term (the
+ * reference's `adjusted_lr` tensor).
  * Replaces muon_update_post_orthogonalize (dion/muon.py:315-347). */
 int dion_muon_post(const uint64_t* X_ptrs, int x_dtype, const void* U, int u_dtype, int n, int64_t numel,
-                   int cols, const float* row_scale, const float* lr_dev, float adj_ratio,
-                   const float* wd_dev, float wd_host, int cautious, void* stream);
+                   int cols, const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
+                   float adj_ratio, const float* wd_dev, float wd_host, int cautious, void* stream);
+
+/* out[r][:] = U[r][:] * scale[r] for n_rows rows of cols bf16 elements; out fp32 or bf16 per out_dtype.
+ * With the scales of dion_normuon_stats this is the `normalized_U` that
+ * normuon_normalization_stacked returns (dion/normuon.py:344-399); the optimizers never materialise
+ * it (the scale is folded into dion_muon_post / dion_dion2_post). */
+int dion_scale_rows(const void* U, const float* scale, void* out, int out_dtype, int64_t n_rows, int cols,
+                    void* stream);
 
 /* NorMuon neuron-wise normalization statistics for one shape group.
  *   r = mean(U^2, dim=-1); V = lerp(V, r, 1-beta2); d = sqrt(V)+1e-8;

@@ -213,20 +213,116 @@ def test_lion_update_foreach():
         assert int(bad.sum()) <= 1  # a blend within rounding of zero may take the other sign
 
 
+@pytest.mark.parametrize("nesterov", [False, True])
+def test_muon_update_pre_and_post_orthogonalize(nesterov):
+    """The list-of-tensors forms of dion/muon.py:284-347 against the oracle."""
+    from dion.muon import muon_update_post_orthogonalize, muon_update_pre_orthogonalize
+
+    torch.manual_seed(21)
+    shape, n = (48, 80), 3
+    G = [(torch.randn(shape) * 0.02).to(torch.bfloat16) for _ in range(n)]
+    M = [torch.randn(shape) * 0.01 for _ in range(n)]
+    X = [torch.randn(shape) * 0.05 for _ in range(n)]
+    Md, Xd = [m.to(DEV) for m in M], [x.to(DEV) for x in X]
+    U = muon_update_pre_orthogonalize([g.to(DEV) for g in G], Md, torch.tensor(0.95), nesterov)
+    assert len(U) == n and all(u.dtype == torch.bfloat16 and u.shape == shape for u in U)
+    for i in range(n):
+        m_ref, u_ref = oracle.muon_pre(G[i], M[i], 0.95, nesterov)
+        assert torch.equal(Md[i].cpu(), m_ref) and torch.equal(U[i].cpu(), u_ref)
+    base_lr, adjusted_lr = torch.tensor(0.02, device=DEV), torch.tensor(0.02 * 0.7746, device=DEV)
+    for cautious, u_list in ((False, U), (True, [u.float().clone() for u in U])):  # arena views, then loose tensors
+        Xc = [x.clone() for x in Xd]
+        muon_update_post_orthogonalize(Xc, u_list, base_lr, adjusted_lr, 0.1, cautious_wd=cautious)
+        for i in range(n):
+            ref = oracle.muon_post(X[i], U[i].cpu(), 0.02, float(adjusted_lr) / 0.02, 0.1, cautious)
+            assert float((Xc[i].cpu() - ref).abs().max()) <= 1e-7
+    muon_update_post_orthogonalize([], [], base_lr, adjusted_lr, 0.1)
+    assert muon_update_pre_orthogonalize([], [], 0.95, nesterov) == []
+
+
+@pytest.mark.parametrize("vdtype", [torch.float32, torch.bfloat16])
+def test_normuon_normalization_stacked(vdtype):
+    """dion/normuon.py:344-399 out of place: normalised update and new second moments against the oracle,
+    the Frobenius norm is preserved, and split_sizes equals separate calls on the blocks."""
+    from dion.normuon import normuon_normalization_stacked
+
+    torch.manual_seed(22)
+    n, rows, cols = 4, 24, 40
+    U = (torch.randn(n, rows, cols) * 0.05).to(torch.bfloat16)
+    V = (torch.rand(n, rows, 1) * 1e-3).to(vdtype)
+    Ud, Vd = U.to(DEV), V.to(DEV)
+    v_before = Vd.clone()
+    nU, nV = normuon_normalization_stacked(Ud, Vd, torch.tensor(0.95))
+    assert torch.equal(Vd, v_before), "the call is out of place"
+    assert nU.dtype == vdtype and nV.dtype == vdtype and nU.shape == U.shape and nV.shape == V.shape
+    tol = 1e-5 if vdtype == torch.float32 else 2.0 ** -7
+    for i in range(n):
+        u_ref, v_ref = oracle.normuon_normalize(U[i], V[i].float(), 0.95)
+        assert _rel(nV[i].float(), v_ref) <= tol and _rel(nU[i].float(), u_ref) <= tol
+        assert abs(float(nU[i].float().norm()) / float(U[i].float().norm()) - 1) <= tol
+    split = (8, 16)
+    sU, sV = normuon_normalization_stacked(Ud, Vd, 0.95, split_sizes=split)
+    off = 0
+    for sz in split:
+        bU, bV = normuon_normalization_stacked(Ud[:, off:off + sz].contiguous(), Vd[:, off:off + sz].contiguous(), 0.95)
+        assert torch.equal(sU[:, off:off + sz], bU) and torch.equal(sV[:, off:off + sz], bV)
+        off += sz
+    with pytest.raises(ValueError):
+        normuon_normalization_stacked(Ud, Vd, 0.95, split_sizes=(8, 8))
+    with pytest.raises(TypeError):
+        normuon_normalization_stacked(Ud.float(), Vd, 0.95)
+
+
+@pytest.mark.parametrize("vdtype", [torch.float32, torch.bfloat16])
+def test_normalize_selected_stacked_matches_unfused(vdtype):
+    """The reference's own check (tests/test_optimizers.py:241-277): the selected-rows helper equals gather ->
+    normuon_normalization_stacked -> scatter."""
+    from dion.nordion2 import nordion2_normalize_selected_stacked
+    from dion.normuon import normuon_normalization_stacked
+
+    torch.manual_seed(3)
+    n, rows, cols, k = 4, 16, 32, 8
+    u = torch.randn(n, k, cols, device=DEV, dtype=torch.bfloat16)
+    v_full = torch.rand(n, rows, 1, device=DEV).to(vdtype)
+    indices = torch.stack([torch.randperm(rows, device=DEV)[:k] for _ in range(n)], dim=0)
+    beta2 = torch.tensor(0.9)
+    u_fused, v_fused = nordion2_normalize_selected_stacked(u.clone(), v_full.clone(), indices, beta2)
+    assert u_fused.dtype == torch.float32 and v_fused.dtype == vdtype
+
+    idx = indices.unsqueeze(-1)
+    v_sel = torch.gather(v_full, dim=-2, index=idx).float()
+    u_ref, v_sel_new = normuon_normalization_stacked(u.clone(), v_sel, beta2)
+    v_ref = v_full.clone()
+    for i in range(n):
+        v_ref[i].scatter_(dim=-2, index=idx[i], src=v_sel_new[i].to(v_ref.dtype))
+    if vdtype == torch.float32:
+        torch.testing.assert_close(u_fused, u_ref, atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(v_fused, v_ref, atol=1e-5, rtol=1e-5)
+    else:  # the scale comes from the stored (rounded) second moments
+        torch.testing.assert_close(u_fused, u_ref, atol=1e-5, rtol=2.0 ** -8)
+        assert torch.equal(v_fused, v_ref)
+    unsel = torch.ones(n, rows, dtype=torch.bool, device=DEV).scatter_(1, indices, False)
+    assert torch.equal(v_fused.squeeze(-1)[unsel], v_full.squeeze(-1)[unsel])
+
+
 def test_submodule_import_paths():
     """The names the reference's tests and callers import from its submodules resolve."""
     import dion
     from dion.cuda_graph import CudaGraphOptimizer
     from dion.dion2 import Dion2, _make_select_and_orthogonalize, dion2_post_orthogonalize_masked, dion2_pre_accumulate
     from dion.dion3 import Dion3
-    from dion.muon import Muon
+    from dion.muon import Muon, muon_update_post_orthogonalize, muon_update_pre_orthogonalize
     from dion.newton_schulz_triton import newton_schulz_triton, ns_line_1, ns_line_2, ns_line_3, zeropower_via_newtonschulz5
-    from dion.nordion2 import NorDion2, nordion2_post_orthogonalize_masked
-    from dion.normuon import NorMuon
+    from dion.nordion2 import NorDion2, nordion2_normalize_selected_stacked, nordion2_post_orthogonalize_masked
+    from dion.normuon import NorMuon, normuon_normalization_stacked
+    from dion.opt_utils import as_scalar_tensor, lm_head_lr_scale
     from dion.polar_express import polar_express, polar_express_triton
 
     assert Dion3 is NorDion2 is dion.NorDion2 and Dion2 is dion.Dion2 and Muon is dion.Muon and NorMuon is dion.NorMuon
     assert all(callable(f) for f in (CudaGraphOptimizer, _make_select_and_orthogonalize, dion2_pre_accumulate,
                                      dion2_post_orthogonalize_masked, nordion2_post_orthogonalize_masked,
                                      newton_schulz_triton, ns_line_1, ns_line_2, ns_line_3,
-                                     zeropower_via_newtonschulz5, polar_express, polar_express_triton))
+                                     zeropower_via_newtonschulz5, polar_express, polar_express_triton,
+                                     muon_update_pre_orthogonalize, muon_update_post_orthogonalize,
+                                     nordion2_normalize_selected_stacked, normuon_normalization_stacked,
+                                     as_scalar_tensor, lm_head_lr_scale))

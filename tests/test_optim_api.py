@@ -293,3 +293,13 @@ def test_empty_lists_are_accepted_by_the_list_functions():
 
     adamw_update_foreach([], [], [], [], 0.01, 0.9, 0.95, 0.1, 1, 1e-8)
     lion_update_foreach([], [], [], 0.01, 0.9, 0.99, 0.1)
+
+
+@pytest.mark.parametrize(("scalar_opt", "expected_scale"), [("adamw", 1.0), ("lion", 1 / 768 ** 0.5)])
+def test_lm_head_lr_scale_by_scalar_opt(scalar_opt, expected_scale):
+    """The reference's own check (tests/test_optimizers.py:42-53)."""
+    from dion.opt_utils import as_scalar_tensor, lm_head_lr_scale
+
+    assert lm_head_lr_scale(scalar_opt, model_dim=768) == pytest.approx(expected_scale)
+    t = torch.tensor(0.5)
+    assert as_scalar_tensor(t) is t and float(as_scalar_tensor(0.25)) == 0.25
