@@ -79,6 +79,14 @@ def test_parameters_that_are_offset_views(shape, xdtype):
     assert all(torch.equal(a, b) for a, b in zip(Xa, Xb))
 
 
+@pytest.mark.parametrize("shape,xdtype", [((4096, 14336), torch.float32), ((14336, 4096), torch.float32),
+                                          ((14336, 4096), BF), ((1024, 4096), BF)])
+def test_llama_sized_parameters(shape, xdtype):
+    """The 256x256-tile kernels at the headline shapes, both orientations."""
+    _X0, _O, Xa, Xb = _run_both(shape, 2, xdtype, False)
+    assert all(torch.equal(a, b) for a, b in zip(Xa, Xb))
+
+
 @pytest.mark.parametrize("shape", [(128, 256), (256, 128)])
 def test_more_parameters_than_one_launch_holds(shape):
     """70 parameters: the last GEMM is launched once per 64 pointers."""
