@@ -288,10 +288,16 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   // One direct-to-LDS load (index j of the LPS that make up a stage) of k-slab kt into ring
   // slot buf.  kt past the end re-fetches the last slab (never read): the refill count per stage
   // stays fixed, which is what the vmcnt bookkeeping in pipeline_barrier relies on.
+  // A diagonal tile of a symmetric product of one matrix with itself (A = X X^T, A A) needs one operand
+  // tile, not two: Q's loads are skipped and its fragments are read from P's half of the slot.  (With a
+  // two-slot ring the barrier waits for every outstanding load, so the load count per slab is free to vary.)
+  const bool one_operand = !QK && !Cfg::VG && NSTAGE == 2 && p.tri && ti == tj && p.P == p.Q &&
+                           p.ldp == p.ldq && p.strideP == p.strideQ;
   auto issue_load = [&](int kt, int buf, int j) {
 #ifdef DION_DBG_NO_LOADS
     if (kt >= NSTAGE) return;
 #endif
+    if (one_operand && j >= Cfg::P_LOADS) return;
     const int k = kt < KT ? kt : KT - 1;
     char* l = lds + buf * Cfg::STAGE_BYTES + wave * (64 * 16);
     if (j < Cfg::P_LOADS) {
@@ -327,7 +333,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   for (int kk = 0; kk < KK; ++kk) {
     const int chunk = ((kk * 2 + fhalf) ^ fswz) * 16;
     aoff[kk] = (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + chunk);
-    boff[kk] = (uint32_t)(Cfg::P_BYTES + (wn * Cfg::WTN + frow) * (BK * 2) + chunk);
+    boff[kk] = (uint32_t)((one_operand ? 0 : Cfg::P_BYTES) + (wn * Cfg::WTN + frow) * (BK * 2) + chunk);
   }
 
   // QK fragments: within a 16-lane group, lane 4r+q addresses row r / 4-element piece q of a 4x16
