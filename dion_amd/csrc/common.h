@@ -187,6 +187,7 @@ struct GemmParams {
   int batch;
   int tri;           // 1: Q == P, only tiles with tile_row <= tile_col are computed, Ct mirrors
   int q_kmajor;      // 1: Q is stored [K][N] (reduction index along rows); not with tri
+  int xcd_interleave;  // set by the launcher: tile list dealt to the XCDs in interleaved 32-tile chunks
   float alpha, beta;
   float diag;        // added to C[i][i] (global diagonal); used with tri to fold a*I into B
 };

@@ -241,9 +241,21 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   int lt;
   {
     const int pid = blockIdx.x;
-    const int xcd = pid & 7, loc = pid >> 3;
-    const int q = total >> 3, r = total & 7;
-    lt = xcd * q + (xcd < r ? xcd : r) + loc;
+    if (p.xcd_interleave && pid < (total & ~255)) {
+      // 256 consecutive workgroups = 32 per XCD: each XCD takes 32 consecutive tiles of the same 256-tile
+      // stretch, so the 8 XCDs work on neighbouring tile groups (same matrix, same operand row panels)
+      // at the same time, and what one of them fetches from memory the others find in the memory-side
+      // cache.  Pays when a matrix's operands are much larger than an XCD's L2.
+      const int j = pid & 255;
+      lt = (pid & ~255) + (j & 7) * 32 + (j >> 3);
+    } else if (p.xcd_interleave) {
+      lt = pid;
+    } else {
+      // one contiguous run of the tile list per XCD: a small matrix stays in one L2
+      const int xcd = pid & 7, loc = pid >> 3;
+      const int q = total >> 3, r = total & 7;
+      lt = xcd * q + (xcd < r ? xcd : r) + loc;
+    }
   }
   const int b = lt / tiles_per_mat;
   const int t = lt - b * tiles_per_mat;
@@ -655,6 +667,16 @@ typedef TileCfg<256, 256, 32, 2, 4, 4> Cfg256w8k32;  // 8 wavefronts, 4 x 32-dee
 typedef TileCfg<256, 256, 64, 2, 4, 2, true> Cfg256w8vg;  // 8 wavefronts, register-staged operands
 typedef TileCfg<128, 128, 64, 2, 2, 2, true> Cfg128vg;
 
+// Tile list dealt to the XCDs in interleaved 32-tile chunks (see the kernel) when the first operand of
+// one matrix is at least 16 MB; below that a contiguous run per XCD keeps whole matrices in one L2.
+static bool xcd_interleave_pays(const GemmParams& p) {
+  static const long thresh = [] {
+    const char* e = getenv("DION_XCD_INTERLEAVE_BYTES");
+    return e ? atol(e) : (16L << 20);
+  }();
+  return (int64_t)p.M * p.K * 2 >= thresh;
+}
+
 template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false, int POST = 0>
 static hipError_t launch_epi(const GemmParams& p, hipStream_t stream,
                              const typename PostSel<POST>::arg& post = typename PostSel<POST>::arg()) {
@@ -666,7 +688,9 @@ static hipError_t launch_epi(const GemmParams& p, hipStream_t stream,
   const int64_t total = per_mat * p.batch;
   if (total <= 0) return hipSuccess;
   if (total > 0x7fffffff) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, post);
+  GemmParams pp = p;
+  pp.xcd_interleave = xcd_interleave_pays(p) ? 1 : 0;
+  hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, pp, post);
   return hipGetLastError();
 }
 
