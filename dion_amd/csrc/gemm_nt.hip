@@ -151,44 +151,33 @@ __device__ __forceinline__ void bx_store(__amdgpu_buffer_rsrc_t rs, int lane_byt
     __builtin_amdgcn_raw_buffer_store_b16((unsigned short)f32_to_bf16(v), rs, lane_bytes, uni_bytes, 0);
   else __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rs, lane_bytes, uni_bytes, 0);
 }
-// eight consecutive elements
+// 16 bytes per lane: eight bf16 or four fp32 elements
 template <typename T>
-__device__ __forceinline__ void bx_load8(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int uni_bytes, float v[8]) {
+__device__ __forceinline__ void bx_load16(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int uni_bytes, float* v) {
+  const bx_u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_bytes, uni_bytes, 0);
   if constexpr (sizeof(T) == 2) {
-    const bx_u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_bytes, uni_bytes, 0);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       v[2 * e] = __uint_as_float(w[e] << 16);
       v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
     }
   } else {
-    const bx_u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_bytes, uni_bytes, 0);
-    const bx_u32x4 c = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_bytes + 16, uni_bytes, 0);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      v[e] = __uint_as_float(a[e]);
-      v[4 + e] = __uint_as_float(c[e]);
-    }
+    for (int e = 0; e < 4; ++e) v[e] = __uint_as_float(w[e]);
   }
 }
 template <typename T>
-__device__ __forceinline__ void bx_store8(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int uni_bytes,
-                                          const float v[8]) {
+__device__ __forceinline__ void bx_store16(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int uni_bytes,
+                                           const float* v) {
+  bx_u32x4 o;
   if constexpr (sizeof(T) == 2) {
-    bx_u32x4 o;
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(v[2 * e], v[2 * e + 1]);
-    __builtin_amdgcn_raw_buffer_store_b128(o, rs, lane_bytes, uni_bytes, 0);
   } else {
-    bx_u32x4 a, c;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      a[e] = __float_as_uint(v[e]);
-      c[e] = __float_as_uint(v[4 + e]);
-    }
-    __builtin_amdgcn_raw_buffer_store_b128(a, rs, lane_bytes, uni_bytes, 0);
-    __builtin_amdgcn_raw_buffer_store_b128(c, rs, lane_bytes + 16, uni_bytes, 0);
+    for (int e = 0; e < 4; ++e) o[e] = __float_as_uint(v[e]);
   }
+  __builtin_amdgcn_raw_buffer_store_b128(o, rs, lane_bytes, uni_bytes, 0);
 }
 
 // POST: 0 stores the product; 1 / 2 feed it to the fused Muon update of fp32 / bf16 parameters
@@ -601,46 +590,54 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
       const int srow = lane / CH, schunk = lane % CH;
       const char* sp = stg + srow * Cfg::STG_PITCH + schunk * 16;
       if constexpr (POST != 0) {
-        // the staged bf16 tile is the update; 8 consecutive elements of X per lane, the parameter values
-        // of up to eight staged rows loaded in one go
+        // The staged bf16 tile is the update.  One 16-byte access of X per lane and step (4 fp32 or 8 bf16
+        // elements), lanes side by side along the row: every instruction covers whole contiguous runs.
+        constexpr int EPL = 16 / (int)sizeof(XT);   // elements per lane
+        constexpr int PCH = Cfg::WTM / EPL;          // lanes per staged row
+        constexpr int PRPI = 64 / PCH;               // staged rows per instruction
+        constexpr int NIT = Cfg::WTN / PRPI;
+        constexpr int BI = NIT < (EPL == 4 ? 16 : 8) ? NIT : (EPL == 4 ? 16 : 8);
+        static_assert(64 % PCH == 0 && Cfg::WTN % PRPI == 0 && NIT % BI == 0, "staged rows per wavefront");
+        const int prow = lane / PCH, pchunk = lane % PCH;
+        const char* pp = stg + prow * Cfg::STG_PITCH + pchunk * (EPL * 2);
         const __amdgpu_buffer_rsrc_t xr = bx_resource(xmat + (int64_t)col_base * ldct + row_base);
-        const int xl = (srow * ldct + schunk * 8) * (int)sizeof(XT);  // per lane
-        constexpr int NIT = Cfg::WTN / RPI;
-        constexpr int BI = NIT < 8 ? NIT : 8;
-        static_assert(NIT % BI == 0, "staged rows per wavefront");
+        const int xl = (prow * ldct + pchunk * EPL) * (int)sizeof(XT);  // per lane
         auto run = [&](auto caut) {
           constexpr int CAUT = decltype(caut)::value;
 #pragma unroll
           for (int it0 = 0; it0 < NIT; it0 += BI) {
-            float uv[BI][8], xv[BI][8];
+            float uv[BI][EPL], xv[BI][EPL];
 #pragma unroll
-            for (int k = 0; k < BI; ++k)
-              st_load8<bf16_t>((const bf16_t*)(sp + (it0 + k) * RPI * Cfg::STG_PITCH), 0, uv[k]);
+            for (int k = 0; k < BI; ++k) {
+              const char* q = pp + (it0 + k) * PRPI * Cfg::STG_PITCH;
+              if constexpr (EPL == 8) st_load8<bf16_t>((const bf16_t*)q, 0, uv[k]);
+              else st_load4<bf16_t>((const bf16_t*)q, 0, uv[k]);
+            }
             if (pvec) {
 #pragma unroll
               for (int k = 0; k < BI; ++k)
-                bx_load8<XT>(xr, xl, (it0 + k) * RPI * ldct * (int)sizeof(XT), xv[k]);
+                bx_load16<XT>(xr, xl, (it0 + k) * PRPI * ldct * (int)sizeof(XT), xv[k]);
             } else {
 #pragma unroll
               for (int k = 0; k < BI; ++k)
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                  xv[k][e] = bx_load<XT>(xr, xl, ((it0 + k) * RPI * ldct + e) * (int)sizeof(XT));
+                for (int e = 0; e < EPL; ++e)
+                  xv[k][e] = bx_load<XT>(xr, xl, ((it0 + k) * PRPI * ldct + e) * (int)sizeof(XT));
             }
 #pragma unroll
             for (int k = 0; k < BI; ++k)
 #pragma unroll
-              for (int e = 0; e < 8; ++e) xv[k][e] = muon_post_one(xv[k][e], uv[k][e], pa, pcoeff, pb, CAUT);
+              for (int e = 0; e < EPL; ++e) xv[k][e] = muon_post_one(xv[k][e], uv[k][e], pa, pcoeff, pb, CAUT);
             if (pvec) {
 #pragma unroll
               for (int k = 0; k < BI; ++k)
-                bx_store8<XT>(xr, xl, (it0 + k) * RPI * ldct * (int)sizeof(XT), xv[k]);
+                bx_store16<XT>(xr, xl, (it0 + k) * PRPI * ldct * (int)sizeof(XT), xv[k]);
             } else {
 #pragma unroll
               for (int k = 0; k < BI; ++k)
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                  bx_store<XT>(xr, xl, ((it0 + k) * RPI * ldct + e) * (int)sizeof(XT), xv[k][e]);
+                for (int e = 0; e < EPL; ++e)
+                  bx_store<XT>(xr, xl, ((it0 + k) * PRPI * ldct + e) * (int)sizeof(XT), xv[k][e]);
             }
           }
         };
