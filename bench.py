@@ -279,7 +279,7 @@ def main() -> int:
         achieved = flop3 / (ms3 * 1e-3) * 1e-12
         result["roofline"] = {
             "bound": "mfma",
-            "kernel": "gemm_nt_kernel<256x256x64, 8 waves, register-staged, K-major second operand> (X' = B X)",
+            "kernel": "gemm_nt_kernel<256x256x64, 8 waves, direct-to-LDS loads, K-major second operand> (X' = B X)",
             "achieved": round(achieved, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",

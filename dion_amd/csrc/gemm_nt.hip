@@ -350,6 +350,12 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
                            (t16 & 3) * 8);
   }
 
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+  // Fragment reads of a slice go out in the order A0, B0..B(TN-1), A1..A(TM-1); LDS returns in order, so once
+  // at most the TM-1 reads issued after the last B fragment are outstanding, every B fragment has arrived.
+  auto qk_wait = [&]() {
+    if (QK && !Cfg::VG) __builtin_amdgcn_s_waitcnt(0xC07F | ((TM - 1) << 8));  // lgkmcnt(TM-1) only
+  };
   bf16x8 fa[2][TM], fb[2][TN];
   // Fragment read r (0..NR-1) of slice kk of ring slot buf into fragment set f, in the order the
   // MFMAs (row-major over the TM x TN accumulators) first need them: A0, B0..B(TN-1), A1..A(TM-1).
@@ -358,6 +364,20 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
     if (r == 0 || r > TN) {
       const int i = r == 0 ? 0 : r - TN;
       fa[f][i] = *(const bf16x8*)(st + aoff[kk] + i * (32 * BK * 2));
+    } else if (QK && !Cfg::VG) {
+      // With the DMA transport the transposing reads are written as assembly: through the builtin the
+      // compiler makes each of them wait for every outstanding direct-to-LDS load (it cannot tell that they
+      // read another ring slot), which exposes the whole load latency once per slab.  The compiler does not
+      // know these reads are in flight: qk_wait() below is the wait their consumers need.
+      const int j = r - 1;
+      const uint32_t a = lds_base + (uint32_t)(buf * Cfg::STAGE_BYTES) + qoff[j] + (uint32_t)(kk * (16 * BN * 2));
+      typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+      u32x2 lo, hi;
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(a));
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(a), "n"(4 * BN * 2));
+      typedef __attribute__((ext_vector_type(4))) unsigned u32x4f;
+      const u32x4f v = {lo[0], lo[1], hi[0], hi[1]};
+      fb[f][j] = __builtin_bit_cast(bf16x8, v);
     } else if (QK) {
       const int j = r - 1;
       const char* q = st + qoff[j] + kk * (16 * BN * 2);
@@ -421,6 +441,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
         const bool last = (kk == KK - 1);
         // slab kt+1 landed (DMA) / written by every wavefront (VG), slab kt fully read
         if (last) pipeline_barrier<Cfg::VG ? 63 : (NSTAGE - 2) * LPS>();
+        qk_wait();
 #pragma unroll
         for (int q = 0; q < NM; ++q) {
 #ifdef DION_DBG_NO_MFMA
@@ -462,6 +483,18 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
     }
   }
   if (!Cfg::VG) wait_vmcnt<0>();  // drain the redundant tail refills before LDS is reused / the wave exits
+  if (QK && !Cfg::VG) {
+    // The read-ahead of the last slice issued transposing reads whose results nobody uses.  The compiler
+    // does not know they are in flight; were their destination registers dead here, it would hand them
+    // to whatever comes next (the lane index, store addresses) and a read landing late would overwrite
+    // that.  So: wait for the LDS queue to drain, and only then let go of the fragment registers -- the
+    // empty asm statements below are their last use and sit behind the wait.
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) asm volatile("" ::"v"(fb[f][j]));
+  }
 
   // ---- epilogue.  Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4,
   // column l%32 of its 32x32 tile.  Whole tiles are stored: destinations are padded to the tile.
@@ -750,8 +783,8 @@ hipError_t launch_gemm_nt_post(const GemmParams& p, const FusedPost& post, int x
   if (!p.q_kmajor || p.tri || p.D || post.mats_per_ptr <= 0 || !post.lr_dev ||
       p.batch > (int64_t)kMaxPtrs * post.mats_per_ptr || (x_dtype != 0 && x_dtype != 1))
     return hipErrorInvalidValue;
-  return wants_256_tiles(p) ? launch_post_cfg<Cfg256w8vg>(p, post, x_dtype, transposed, stream)
-                            : launch_post_cfg<Cfg128vg>(p, post, x_dtype, transposed, stream);
+  return wants_256_tiles(p) ? launch_post_cfg<Cfg256w8>(p, post, x_dtype, transposed, stream)
+                            : launch_post_cfg<Cfg128>(p, post, x_dtype, transposed, stream);
 }
 
 hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) {
@@ -769,10 +802,11 @@ hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) 
       return e ? atoi(e) : -1;
     }();
     if (forced128 >= 0 && variant == 1) variant = forced128;
-    // The K-major second operand loads better through registers than through the DMA.
+    // Tuning knob: DION_QK_VG=1 sends the K-major second operand through registers (global -> VGPR ->
+    // ds_write) instead of the DMA; slower since the transposing reads no longer wait for the DMA.
     static const bool qk_vg = [] {
       const char* e = getenv("DION_QK_VG");
-      return !(e && atoi(e) == 0);
+      return e && atoi(e) != 0;
     }();
     if (p.q_kmajor && qk_vg) variant = variant == 3 ? 6 : (variant == 1 ? 8 : variant);
   }

@@ -92,6 +92,39 @@ def test_line_3_both_operand_forms(batch, m, n, a):
     assert torch.equal(Ct_only, Ct_nt)
 
 
+@pytest.mark.parametrize("batch,m,n", [(24, 512, 8192), (24, 512, 2048), (8, 256, 1024), (3, 128, 384)])
+def test_line_3_short_reduction_many_launches(batch, m, n):
+    """X' = B X with only a few k-slabs per tile, launched back to back: the epilogue starts right behind the
+    last fragment reads of the main loop.  (Those reads are issued from assembly; their destination registers
+    have to stay allocated until the LDS queue has drained, or the epilogue's addresses get overwritten.)
+    Every launch must reproduce the first one bit for bit, and that one must be the product."""
+    lib, check = _lib()
+    torch.manual_seed(batch + m + n)
+    X = torch.randn(batch, m, n, device=DEV).to(torch.bfloat16)
+    Bm = torch.randn(batch, m, m, device=DEV)
+    Bm = ((Bm + Bm.mT) / 2).to(torch.bfloat16)
+    st = _stream()
+    first = torch.empty_like(X)
+    check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), None, first.data_ptr(), None, batch, m, n,
+                             ctypes.c_float(0.0), st), "line_3")
+    ref = torch.bmm(Bm.float(), X.float())
+    assert float((first.float() - ref).norm() / ref.norm()) <= 4e-3
+    outs = [torch.empty_like(X) for _ in range(4)]
+    for rep in range(40):
+        out = outs[rep % 4]
+        check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), None, out.data_ptr(), None, batch, m, n,
+                                 ctypes.c_float(0.0), st), "line_3")
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, first) for o in outs)
+    # the transposed-output form of the same kernel is the last product of a tall orthogonalization
+    from dion_amd import zeropower_via_newtonschulz5
+
+    wide = zeropower_via_newtonschulz5(X)
+    tall_in = X.mT.contiguous()
+    for _ in range(6):
+        assert torch.equal(zeropower_via_newtonschulz5(tall_in), wide.mT)
+
+
 def test_line_3_argument_errors():
     lib, check = _lib()
     from dion_amd._lib import DionHipError
