@@ -125,6 +125,32 @@ def test_line_3_short_reduction_many_launches(batch, m, n):
         assert torch.equal(zeropower_via_newtonschulz5(tall_in), wide.mT)
 
 
+@pytest.mark.parametrize("batch,m,n", [(24, 512, 8192), (5, 1024, 14336), (3, 2304, 10240), (2, 4096, 8192),
+                                       (33, 768, 4096)])
+def test_line_3_thousand_tile_launches(batch, m, n):
+    """X' = B X over a thousand or more 256-wide tiles (tile counts that are and are not multiples of the CU
+    count; both tile orders): the form that reads X as it lies and the form that takes X^T must agree bit for
+    bit, on every launch, and be the product."""
+    lib, check = _lib()
+    torch.manual_seed(batch + m + n)
+    X = torch.randn(batch, m, n, device=DEV).to(torch.bfloat16)
+    Xt = X.mT.contiguous()
+    Bm = torch.randn(batch, m, m, device=DEV)
+    Bm = ((Bm + Bm.mT) / 2).to(torch.bfloat16)
+    st = _stream()
+    C_nt = torch.empty_like(X)
+    check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), Xt.data_ptr(), C_nt.data_ptr(), None, batch, m, n,
+                             ctypes.c_float(0.0), st), "line_3 (X^T given)")
+    ref = torch.bmm(Bm.float(), X.float())
+    assert float((C_nt.float() - ref).norm() / ref.norm()) <= 4e-3
+    del ref
+    for rep in range(3):
+        C_qk = torch.full_like(X, float("nan"))
+        check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), None, C_qk.data_ptr(), None, batch, m, n,
+                                 ctypes.c_float(0.0), st), "line_3 (X as it lies)")
+        assert torch.equal(C_qk, C_nt), rep
+
+
 def test_line_3_argument_errors():
     lib, check = _lib()
     from dion_amd._lib import DionHipError
