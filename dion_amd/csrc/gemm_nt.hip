@@ -16,9 +16,9 @@
 //
 // Kernel structure: one workgroup per BM x BN output tile, WM x WN wavefronts (64 lanes) each
 // owning a (BM/WM) x (BN/WN) sub-tile as 32x32 MFMA accumulators
-// (v_mfma_f32_32x32x16_bf16).  Operand tiles reach a two-slot LDS ring either through the
-// direct-to-LDS loads (global_load_lds_dwordx4, no VGPR staging) or staged through registers
-// (TileCfg::VG); XOR swizzles keep the LDS writes and the fragment reads bank-conflict free.
+// (v_mfma_f32_32x32x16_bf16).  Operand tiles reach a two-slot LDS ring through direct-to-LDS
+// loads (global_load_lds_dwordx4, no VGPR staging); XOR swizzles keep the LDS writes and the
+// fragment reads bank-conflict free.
 #include <stdlib.h>
 
 #include <type_traits>
@@ -30,14 +30,10 @@ namespace dion {
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
-// VG_: operand slabs travel global -> VGPR -> LDS (plain 16-byte loads, ds_write_b128 one slab
-// later) instead of the direct-to-LDS DMA: every load gets a full slab of latency slack and the
-// kernel places the LDS writes itself, between MFMAs.
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int NSTAGE_, bool VG_ = false>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int NSTAGE_>
 struct TileCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, NSTAGE = NSTAGE_;
-  static constexpr bool VG = VG_;
-  static_assert(!VG_ || NSTAGE_ == 2, "register staging is written for a two-slot ring");
+  static_assert(NSTAGE_ == 2, "the pipeline below is written for a two-slot ring");
   static constexpr int NT = WM * WN * 64;
   static constexpr int CPR = BK / 8;            // 16-byte chunks per tile row
   static constexpr int ROWS_PER_LOAD = NT / CPR; // tile rows covered by one load instruction
@@ -208,13 +204,6 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   static_assert(KK % 2 == 0, "fragment double buffer needs an even slice count per stage");
   constexpr int RPM = (NR + NM - 1) / NM;    // fragment reads slotted behind each MFMA
   constexpr int LPM = (LPS + NM - 1) / NM;   // refill loads slotted behind each MFMA
-  // With three or more ring slots the refill of a slot need not be issued in one burst: it is
-  // spread over the KK slices that follow the barrier which frees the slot (the last slice of its
-  // slab and the first KK-1 slices of the next), LPW loads per slice at even MFMA spacing, so the
-  // loads reach the vector memory pipeline at the rate it drains them.
-  constexpr bool SPREAD = NSTAGE >= 3 && LPS % KK == 0 && NM % (LPS / KK) == 0;
-  constexpr int LPW = SPREAD ? LPS / KK : LPS;
-  constexpr int QPL = SPREAD ? NM / LPW : 1;  // MFMAs per load slot
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int tid = threadIdx.x;
@@ -292,12 +281,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   // A diagonal tile of a symmetric product of one matrix with itself (A = X X^T, A A) needs one operand
   // tile, not two: Q's loads are skipped and its fragments are read from P's half of the slot.  (With a
   // two-slot ring the barrier waits for every outstanding load, so the load count per slab is free to vary.)
-  const bool one_operand = !QK && !Cfg::VG && NSTAGE == 2 && p.tri && ti == tj && p.P == p.Q &&
-                           p.ldp == p.ldq && p.strideP == p.strideQ;
+  const bool one_operand = !QK && p.tri && ti == tj && p.P == p.Q && p.ldp == p.ldq && p.strideP == p.strideQ;
   auto issue_load = [&](int kt, int buf, int j) {
-#ifdef DION_DBG_NO_LOADS
-    if (kt >= NSTAGE) return;
-#endif
     if (one_operand && j >= Cfg::P_LOADS) return;
     const int k = kt < KT ? kt : KT - 1;
     char* l = lds + buf * Cfg::STAGE_BYTES + wave * (64 * 16);
@@ -310,19 +295,6 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
       __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + Cfg::P_BYTES + jq * (Cfg::NT * 16)),
                                        16, 0, 0);
     }
-  };
-
-  // Register-staged transport (Cfg::VG): stage_reg[j] holds load j of the slab after next.
-  typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
-  u32x4 stage_reg[Cfg::VG ? LPS : 1];
-  auto stage_fetch = [&](int kt, int j) {
-    const int k = kt < KT ? kt : KT - 1;
-    const char* src = j < Cfg::P_LOADS ? gP + (int64_t)k * (BK * 2) + (offP + j * stepP)
-                                       : gQ + k * slabQ + (offQ + (j - Cfg::P_LOADS) * stepQ);
-    stage_reg[j] = *(const u32x4*)src;
-  };
-  auto stage_store = [&](int buf, int j) {
-    *(u32x4*)(lds + buf * Cfg::STAGE_BYTES + j * (Cfg::NT * 16) + tid * 16) = stage_reg[j];
   };
 
   // ---- LDS -> register fragment addressing (per lane, per 16-wide k slice).
@@ -354,7 +326,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   // Fragment reads of a slice go out in the order A0, B0..B(TN-1), A1..A(TM-1); LDS returns in order, so once
   // at most the TM-1 reads issued after the last B fragment are outstanding, every B fragment has arrived.
   auto qk_wait = [&]() {
-    if (QK && !Cfg::VG) __builtin_amdgcn_s_waitcnt(0xC07F | ((TM - 1) << 8));  // lgkmcnt(TM-1) only
+    if (QK) __builtin_amdgcn_s_waitcnt(0xC07F | ((TM - 1) << 8));  // lgkmcnt(TM-1) only
   };
   bf16x8 fa[2][TM], fb[2][TN];
   // Fragment read r (0..NR-1) of slice kk of ring slot buf into fragment set f, in the order the
@@ -364,8 +336,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
     if (r == 0 || r > TN) {
       const int i = r == 0 ? 0 : r - TN;
       fa[f][i] = *(const bf16x8*)(st + aoff[kk] + i * (32 * BK * 2));
-    } else if (QK && !Cfg::VG) {
-      // With the DMA transport the transposing reads are written as assembly: through the builtin the
+    } else if (QK) {
+      // The transposing reads are written as assembly: through the builtin the
       // compiler makes each of them wait for every outstanding direct-to-LDS load (it cannot tell that they
       // read another ring slot), which exposes the whole load latency once per slab.  The compiler does not
       // know these reads are in flight: qk_wait() below is the wait their consumers need.
@@ -377,16 +349,6 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
       asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(a), "n"(4 * BN * 2));
       typedef __attribute__((ext_vector_type(4))) unsigned u32x4f;
       const u32x4f v = {lo[0], lo[1], hi[0], hi[1]};
-      fb[f][j] = __builtin_bit_cast(bf16x8, v);
-    } else if (QK) {
-      const int j = r - 1;
-      const char* q = st + qoff[j] + kk * (16 * BN * 2);
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) s16x4*)(q));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) s16x4*)(q + 4 * BN * 2));
-      typedef __attribute__((ext_vector_type(8))) short s16x8;
-      const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       fb[f][j] = __builtin_bit_cast(bf16x8, v);
     } else {
       const int j = r - 1;
@@ -404,28 +366,15 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 
   // ---- prologue: fill NSTAGE-1 ring slots, wait for slab 0, read its first fragments, start the
   // last free slot.
-  if (Cfg::VG) {
 #pragma unroll
-    for (int j = 0; j < LPS; ++j) stage_fetch(0, j);
+  for (int s = 0; s < NSTAGE - 1; ++s)
 #pragma unroll
-    for (int j = 0; j < LPS; ++j) {
-      stage_store(0, j);
-      stage_fetch(1, j);
-    }
-    pipeline_barrier<63>();
+    for (int j = 0; j < LPS; ++j) issue_load(s, s, j);
+  pipeline_barrier<(NSTAGE - 2) * LPS>();
 #pragma unroll
-    for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
-  } else {
+  for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
 #pragma unroll
-    for (int s = 0; s < NSTAGE - 1; ++s)
-#pragma unroll
-      for (int j = 0; j < LPS; ++j) issue_load(s, s, j);
-    pipeline_barrier<(NSTAGE - 2) * LPS>();
-#pragma unroll
-    for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
-#pragma unroll
-    for (int j = 0; j < LPW; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
-  }
+  for (int j = 0; j < LPS; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- main loop.  Slices run back to back across slab boundaries: while the MFMAs of one slice
@@ -439,14 +388,11 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
       for (int kk = 0; kk < KK; ++kk) {
         const int cur = kk & 1, nxt = cur ^ 1;
         const bool last = (kk == KK - 1);
-        // slab kt+1 landed (DMA) / written by every wavefront (VG), slab kt fully read
-        if (last) pipeline_barrier<Cfg::VG ? 63 : (NSTAGE - 2) * LPS>();
+        // slab kt+1 landed, slab kt fully read
+        if (last) pipeline_barrier<(NSTAGE - 2) * LPS>();
         qk_wait();
 #pragma unroll
         for (int q = 0; q < NM; ++q) {
-#ifdef DION_DBG_NO_MFMA
-          if (q == 0)
-#endif
           acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
               fa[cur][q / TN], fb[cur][q % TN], acc[q / TN][q % TN], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
@@ -455,24 +401,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
             if (last) read_frag((s + 1) % NSTAGE, 0, nxt, r);
             else read_frag(s, kk + 1, nxt, r);
           }
-          if (Cfg::VG) {
-            // slices 0..KK-2 of slab kt: write slab kt+1 (fetched during slab kt-1) into the other
-            // slot, then fetch slab kt+2 into the freed registers, at even MFMA spacing
-            constexpr int SLOTS = (KK - 1) * NM;
-            constexpr int STRIDE = SLOTS / LPS > 0 ? SLOTS / LPS : 1;
-            static_assert(!Cfg::VG || SLOTS >= LPS, "not enough MFMA slots for the staged stores");
-            const int t = kk * NM + q;
-            if (!last && t % STRIDE == 0 && t / STRIDE < LPS) {
-              stage_store((s + 1) % NSTAGE, t / STRIDE);
-              stage_fetch(kt0 + s + 2, t / STRIDE);
-            }
-          } else if (SPREAD) {
-            if (q % QPL == QPL / 2) {
-              const int jw = q / QPL;
-              if (last) issue_load(kt0 + s + NSTAGE, s, jw);
-              else issue_load(kt0 + s - 1 + NSTAGE, (s + NSTAGE - 1) % NSTAGE, (kk + 1) * LPW + jw);
-            }
-          } else if (last) {
+          if (last) {
 #pragma unroll
             for (int j = q * LPM; j < (q + 1) * LPM && j < LPS; ++j)
               issue_load(kt0 + s + NSTAGE, s, j);
@@ -482,8 +411,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
       }
     }
   }
-  if (!Cfg::VG) wait_vmcnt<0>();  // drain the redundant tail refills before LDS is reused / the wave exits
-  if (QK && !Cfg::VG) {
+  wait_vmcnt<0>();  // drain the redundant tail refills before LDS is reused / the wave exits
+  if (QK) {
     // The read-ahead of the last slice issued transposing reads whose results nobody uses.  The compiler
     // does not know they are in flight; were their destination registers dead here, it would hand them
     // to whatever comes next (the lane index, store addresses) and a read landing late would overwrite
@@ -690,12 +619,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 }
 
 // ---------------------------------------------------------------------------------------------
-typedef TileCfg<256, 256, 64, 2, 2, 2> Cfg256;
-typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg128;
-typedef TileCfg<256, 256, 64, 2, 4, 2> Cfg256w8;   // 8 wavefronts, 128x64 each: two per SIMD
-typedef TileCfg<256, 256, 32, 2, 4, 4> Cfg256w8k32;  // 8 wavefronts, 4 x 32-deep slabs, spread refill
-typedef TileCfg<256, 256, 64, 2, 4, 2, true> Cfg256w8vg;  // 8 wavefronts, register-staged operands
-typedef TileCfg<128, 128, 64, 2, 2, 2, true> Cfg128vg;
+typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg128;     // 4 wavefronts, 64x64 each; two workgroups per CU
+typedef TileCfg<256, 256, 64, 2, 4, 2> Cfg256w8;   // 8 wavefronts, 128x64 each: two per SIMD, one workgroup per CU
 
 // Tile list dealt to the XCDs in interleaved 32-tile chunks (see the kernel) when the first operand of
 // one matrix is at least 16 MB; below that a contiguous run per XCD keeps whole matrices in one L2.
@@ -791,33 +716,11 @@ hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) 
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.batch <= 0) return hipSuccess;
   if (variant < 0) {
     variant = wants_256_tiles(p) ? 3 : 1;
-    // Tuning knob: DION_GEMM_VARIANT overrides the 256-wide tile configuration.
-    static const int forced = [] {
-      const char* e = getenv("DION_GEMM_VARIANT");
-      return e ? atoi(e) : -1;
-    }();
-    if (forced >= 0 && variant == 3) variant = forced;
-    static const int forced128 = [] {
-      const char* e = getenv("DION_GEMM_VARIANT128");
-      return e ? atoi(e) : -1;
-    }();
-    if (forced128 >= 0 && variant == 1) variant = forced128;
-    // Tuning knob: DION_QK_VG=1 sends the K-major second operand through registers (global -> VGPR ->
-    // ds_write) instead of the DMA; slower since the transposing reads no longer wait for the DMA.
-    static const bool qk_vg = [] {
-      const char* e = getenv("DION_QK_VG");
-      return e && atoi(e) != 0;
-    }();
-    if (p.q_kmajor && qk_vg) variant = variant == 3 ? 6 : (variant == 1 ? 8 : variant);
   }
   if (p.tri && (p.M != p.N)) return hipErrorInvalidValue;
   switch (variant) {
-    case 0: return launch_cfg<Cfg256>(p, stream);
     case 1: return launch_cfg<Cfg128>(p, stream);
     case 3: return launch_cfg<Cfg256w8>(p, stream);
-    case 5: return launch_cfg<Cfg256w8k32>(p, stream);
-    case 6: return launch_cfg<Cfg256w8vg>(p, stream);
-    case 8: return launch_cfg<Cfg128vg>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }
