@@ -507,6 +507,23 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
     return;
   }
 
+  // The addend is loaded two 32x32 tiles at a time, one pair ahead: the loads of a pair are issued before the
+  // stores of the pair before it, so they neither wait for those stores (the memory counter retires in order)
+  // nor cost a round trip to memory per tile.
+  constexpr int GS = 2, NG = (TM * TN) / GS;
+  static_assert((TM * TN) % GS == 0, "addend pairs");
+  bf16_t dreg[HAS_D ? 2 : 1][GS][16];
+  auto load_addend = [&](int g) {
+#pragma unroll
+    for (int s = 0; s < GS; ++s) {
+      const int i = (g * GS + s) / TN, j = (g * GS + s) % TN;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        dreg[g & 1][s][r] = Dp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldd + j * 32];
+    }
+  };
+  if (HAS_D) load_addend(0);
+
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -515,12 +532,10 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 #pragma unroll
       for (int r = 0; r < 16; ++r) v[r] = alpha * acc[i][j][r];
       if (HAS_D) {
-        bf16_t d[16];
+        const int n = i * TN + j;
+        if (n % GS == 0 && n / GS + 1 < NG) load_addend(n / GS + 1);
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          d[r] = Dp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldd + j * 32];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) v[r] += beta * bf16_to_f32(d[r]);
+        for (int r = 0; r < 16; ++r) v[r] += beta * bf16_to_f32(dreg[(n / GS) & 1][n % GS][r]);
       }
       if (on_diag) {
         // element (row, col) of this 32x32 tile sits on the global diagonal
