@@ -47,11 +47,20 @@ static int check_gemm_dims(const char* who, int batch, int m, int n) {
   return DION_OK;
 }
 
+// The GEMM kernels move operands with 16-byte direct-to-LDS loads and store 16 bytes per lane.
+static int check_gemm_ptr(const char* who, const char* arg, const void* ptr) {
+  if (ptr && !aligned16((uint64_t)(uintptr_t)ptr))
+    return fail(DION_E_INVALID, "%s: %s is not 16-byte aligned", who, arg);
+  return DION_OK;
+}
+
 extern "C" int dion_ns_line_1(const void* X, void* A, int batch, int m, int k, void* stream) {
   if (int rc = check_gemm_dims("dion_ns_line_1", batch, m, k)) return rc;
   if (batch == 0 || m == 0) return DION_OK;
   if (k == 0) return fail(DION_E_INVALID, "dion_ns_line_1: k == 0");
   if (!X || !A) return fail(DION_E_INVALID, "dion_ns_line_1: null argument");
+  if (int rc = check_gemm_ptr("dion_ns_line_1", "X", X)) return rc;
+  if (int rc = check_gemm_ptr("dion_ns_line_1", "A", A)) return rc;
   GemmParams p;
   memset(&p, 0, sizeof(p));
   p.P = p.Q = (const bf16_t*)X;
@@ -75,6 +84,8 @@ extern "C" int dion_ns_line_2(const void* A, void* B, int batch, int m, float al
   if (batch == 0 || m == 0) return DION_OK;
   if (!A || !B) return fail(DION_E_INVALID, "dion_ns_line_2: null argument");
   if (A == B) return fail(DION_E_INVALID, "dion_ns_line_2: in-place not supported");
+  if (int rc = check_gemm_ptr("dion_ns_line_2", "A", A)) return rc;
+  if (int rc = check_gemm_ptr("dion_ns_line_2", "B", B)) return rc;
   GemmParams p;
   memset(&p, 0, sizeof(p));
   p.P = p.Q = p.D = (const bf16_t*)A;
@@ -96,6 +107,11 @@ extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void
   if (batch == 0 || m == 0 || n == 0) return DION_OK;
   if (!C && !Ct) return fail(DION_E_INVALID, "dion_ns_line_3: no output");
   if (!B || (!X && !Xt)) return fail(DION_E_INVALID, "dion_ns_line_3: null argument");
+  if (int rc = check_gemm_ptr("dion_ns_line_3", "B", B)) return rc;
+  if (int rc = check_gemm_ptr("dion_ns_line_3", "X", X)) return rc;
+  if (int rc = check_gemm_ptr("dion_ns_line_3", "Xt", Xt)) return rc;
+  if (int rc = check_gemm_ptr("dion_ns_line_3", "C", C)) return rc;
+  if (int rc = check_gemm_ptr("dion_ns_line_3", "Ct", Ct)) return rc;
   GemmParams p;
   memset(&p, 0, sizeof(p));
   p.P = (const bf16_t*)B;
@@ -248,6 +264,9 @@ static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, 
             "small-matrix Newton-Schulz");
     return DION_OK;
   }
+  // the last GEMM stores into the caller's buffer 16 bytes per lane
+  if (out && !aligned16((uint64_t)(uintptr_t)out))
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize: out is not 16-byte aligned");
   if (batch > 65535)
     return fail(DION_E_INVALID,
                 "dion_ns_orthogonalize: %d matrices in one call (at most 65535 outside the small-matrix "

@@ -41,7 +41,8 @@ int dion_abi_version(void);
 /* --------------------------------------------------------------------------------------------
  * Symmetric / polynomial GEMMs of one Newton-Schulz iteration (kernel-level API).
  * Operands are dense row-major bf16 batches; leading dimension == last extent.
- * Extents must be multiples of 128 (the Python layer pads; the full driver below pads itself).
+ * Extents must be multiples of 128 (the Python layer pads; the full driver below pads itself),
+ * operand and result pointers 16-byte aligned (DION_E_INVALID otherwise).
  * ------------------------------------------------------------------------------------------ */
 
 /* A[b] = X[b] X[b]^T.  X [batch,m,k] -> A [batch,m,m]; only tiles on/above the diagonal are
@@ -66,7 +67,8 @@ int dion_ns_line_3(const void* B, const void* X, const void* Xt, void* C, void* 
  * dion/polar_express.py:20-50).
  *
  *   in   [batch, rows, cols]  bf16 or fp32 (in_dtype), dense
- *   out  [batch, rows, cols]  bf16, dense
+ *   out  [batch, rows, cols]  bf16, dense, 16-byte aligned (DION_E_INVALID otherwise; batches that take
+ *        the LDS-resident small-matrix kernel are exempt)
  *   coeffs  host array of n_iters*3 floats (a,b,c per iteration)
  *   X0 = bf16(in) / (||bf16(in)||_F * norm_scale + eps)  per matrix, then n_iters times
  *   A = X X^T; B = b A + c A A; X = a X + B X   on the orientation with rows <= cols.

@@ -139,6 +139,12 @@ def test_argument_validation_happens_before_any_device_work():
     refused(lib.dion_ns_line_2(None, None, 1, 128, f(1.0), f(1.0), None), "null argument")
     refused(lib.dion_ns_line_3(None, None, None, None, None, 1, 128, 128, f(0.0), None), "no output")
     refused(lib.dion_ns_line_1(None, None, 1, 100, 128, None), "multiples of 128")
+    refused(lib.dion_ns_line_1(0x1002, 0x2000, 1, 128, 128, None), "X is not 16-byte aligned")
+    refused(lib.dion_ns_line_2(0x1000, 0x2008, 1, 128, f(1.0), f(1.0), None), "B is not 16-byte aligned")
+    refused(lib.dion_ns_line_3(0x1000, 0x2000, None, 0x3004, None, 1, 128, 128, f(0.0), None),
+            "C is not 16-byte aligned")
+    refused(lib.dion_ns_orthogonalize(0x1000, 0, 0x2002, 1, 128, 128, (ctypes.c_float * 3)(1.0, 1.0, 1.0), 1, f(1.0),
+                                      f(0.0), 0, 0, 0x4000, 1 << 30, None), "out is not 16-byte aligned")
     # empty problems are accepted and do nothing
     assert lib.dion_slice_l1(None, 0, 0, 8, 8, -2, 0, None, None) == 0
     assert lib.dion_gather_slices(None, 0, 1, 8, 8, -2, None, 0, None, None) == 0
