@@ -1,0 +1,101 @@
+"""The GEMM kernels issue their transposing LDS reads (ds_read_b64_tr_b16) from assembly, so the compiler does not
+know that the results are still on their way when the statement has executed: it may hand a destination register
+it considers dead to something else, and a read that lands late then overwrites that value (once: the lane index
+ahead of the epilogue's address arithmetic, a GPU memory fault).  This test compiles gemm_nt.hip to gfx950 assembly
+and walks every kernel that contains such reads in program order (each loop back-edge taken once), modelling the
+LDS return queue (in-order; s_waitcnt lgkmcnt(N) retires all but the newest N entries): no instruction may read or
+write a register while a transposing read into it is in flight.  Needs hipcc, no GPU."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC = os.path.join(ROOT, "dion_amd", "csrc", "gemm_nt.hip")
+
+
+def _regs(tok):
+    tok = tok.rstrip(",")
+    m = re.match(r"v\[(\d+):(\d+)\]$", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"v(\d+)$", tok)
+    return {int(m.group(1))} if m else set()
+
+
+def walk(body):
+    """Returns (number of transposing reads seen, list of hazards) for one kernel's assembly lines."""
+    labels = {l.split(":")[0].strip(): i for i, l in enumerate(body) if re.match(r"\.L\w+:", l.strip())}
+    taken, queue, hazards = set(), [], []
+    pc = steps = n_tr = 0
+    while pc < len(body) and steps < 500000:
+        steps += 1
+        cur, s = pc, body[pc].split(";")[0].strip()
+        pc += 1
+        if not s or s.startswith(".") or s.endswith(":"):
+            continue
+        op, *args = s.split()
+        if op == "s_endpgm":
+            break
+        if op.startswith("s_cbranch") or op == "s_branch":
+            tgt = args[0]
+            if tgt in labels and labels[tgt] < cur and cur not in taken:
+                taken.add(cur)
+                pc = labels[tgt]
+            elif op == "s_branch" and tgt in labels and labels[tgt] > cur:
+                pc = labels[tgt]
+            continue
+        if op == "s_waitcnt":
+            m = re.search(r"lgkmcnt\((\d+)\)", s)
+            if m:
+                del queue[: max(0, len(queue) - int(m.group(1)))]
+            continue
+        inflight = set().union(*[q for q in queue if q]) if queue else set()
+        if op.startswith("ds_read_b64_tr"):
+            dest = _regs(args[0])
+            n_tr += 1
+            if dest & inflight:
+                hazards.append((cur, s))
+            queue.append(dest)
+            continue
+        touched = set().union(*[_regs(a) for a in args]) if args else set()
+        if touched & inflight:
+            hazards.append((cur, s))
+        if op.startswith("ds_") or op.startswith("s_load") or op.startswith("s_buffer_load"):
+            queue.append(set())
+    return n_tr, hazards
+
+
+def test_the_walk_flags_a_register_reused_before_the_wait():
+    bad = ["ds_read_b64_tr_b16 v[10:11], v3", "v_and_b32_e32 v10, 63, v0", "s_waitcnt lgkmcnt(0)", "s_endpgm"]
+    good = ["ds_read_b64_tr_b16 v[10:11], v3", "ds_read_b128 v[20:23], v4", "s_waitcnt lgkmcnt(1)",
+            "v_mfma_f32_32x32x16_bf16 v[0:15], v[20:23], v[10:13], v[0:15]", "v_and_b32_e32 v10, 63, v0", "s_endpgm"]
+    early = ["ds_read_b64_tr_b16 v[10:11], v3", "ds_read_b128 v[20:23], v4", "s_waitcnt lgkmcnt(2)",
+             "v_mfma_f32_32x32x16_bf16 v[0:15], v[20:23], v[10:13], v[0:15]", "s_endpgm"]
+    assert walk(bad)[1] and not walk(good)[1] and walk(early)[1]
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not on PATH")
+def test_no_kernel_touches_a_register_a_transposing_read_is_in_flight_to(tmp_path):
+    out = tmp_path / "gemm_nt.s"
+    cmd = ["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-S", "--cuda-device-only", SRC, "-o", str(out)]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=900)
+    kernels, name, body = {}, None, []
+    for line in out.read_text().split("\n"):
+        if name is None:
+            if re.match(r"_ZN4dion14gemm_nt_kernel\S*:", line):
+                name, body = line.split(":")[0], []
+        else:
+            body.append(line)
+            if "s_endpgm" in line:
+                kernels[name], name = body, None
+    assert len(kernels) >= 20, "expected every gemm_nt_kernel instantiation in the assembly"
+    with_tr = 0
+    for kname, kbody in kernels.items():
+        n_tr, hazards = walk(kbody)
+        with_tr += n_tr > 0
+        assert not hazards, (kname, hazards[:5])
+    assert with_tr >= 8, "the K-major instantiations should contain transposing reads"
