@@ -99,3 +99,7 @@ def test_no_kernel_touches_a_register_a_transposing_read_is_in_flight_to(tmp_pat
         with_tr += n_tr > 0
         assert not hazards, (kname, hazards[:5])
     assert with_tr >= 8, "the K-major instantiations should contain transposing reads"
+    # and nothing is spilled between the first and the last MFMA of a kernel (the software-pipelined loop)
+    for kname, kbody in kernels.items():
+        mfma = [i for i, l in enumerate(kbody) if "v_mfma" in l]
+        assert not [l for l in kbody[mfma[0]:mfma[-1] + 1] if "scratch_" in l], kname
