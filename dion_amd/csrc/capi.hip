@@ -35,7 +35,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 9; }
+extern "C" int dion_abi_version(void) { return 10; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -522,6 +522,59 @@ extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, in
                                      size_t workspace_bytes, void* stream) {
   return ns_run(in, in_dtype, out, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
                 workspace, workspace_bytes, stream, nullptr);
+}
+
+// ---------------------------------------------------------------------------------------------
+// dion_ns_orthogonalize for callers that cannot provide (or allocate) a workspace: the same driver
+// and kernels over a fixed device array that is part of the library's code object.  Each GPU holds
+// its own copy of the array at its own address, resolved once per device; host code never uses the
+// array's name as an address, only the resolved pointer.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[DION_NS_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void** ptr) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev), "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize_static: device ordinal %d (at most %d devices)", dev,
+                kMaxDevices);
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    // Racing first calls resolve the same address; the lookup allocates nothing.
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    if (!p || ((uintptr_t)p & 255) != 0)
+      return fail(DION_E_HIP, "dion_ns_orthogonalize_static: scratch array resolved to %p", p);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *ptr = p;
+  return DION_OK;
+}
+}  // namespace
+
+extern "C" int dion_ns_orthogonalize_static(const void* in, int in_dtype, void* out, int batch, int rows,
+                                            int cols, const float* coeffs, int n_iters, float norm_scale,
+                                            float eps, int flags, int gram_reset, void* stream) {
+  size_t need = 0;
+  if (batch > 0 && rows > 0 && cols > 0 && !(flags & ~(DION_NS_GRAM | DION_NS_CARRY_XT)) && n_iters >= 0 &&
+      !ns_small_path(rows, cols, flags, n_iters))
+    need = make_plan(batch, rows, cols, flags).total;
+  if (need > (size_t)DION_NS_STATIC_SCRATCH_BYTES)
+    return fail(DION_E_WORKSPACE,
+                "dion_ns_orthogonalize_static: %d x (%d x %d) needs %zu bytes of scratch, the library's fixed "
+                "array holds %zu: use dion_ns_orthogonalize with a caller workspace",
+                batch, rows, cols, need, (size_t)DION_NS_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0)
+    if (int rc = static_scratch(&ws)) return rc;
+  // Nothing in the workspace has to start at zero: the prepare kernel writes every element of the
+  // padded X (zero padding included) and every later buffer is fully written before it is read.
+  return ns_run(in, in_dtype, out, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset, ws,
+                need, stream, nullptr);
 }
 
 extern "C" size_t dion_ns_update_workspace_bytes(int batch, int rows, int cols, int flags, int n_iters) {

@@ -88,6 +88,22 @@ int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, in
                           const float* coeffs, int n_iters, float norm_scale, float eps, int flags,
                           int gram_reset, void* workspace, size_t workspace_bytes, void* stream);
 
+/* dion_ns_orthogonalize without a workspace argument and without any allocation: the library's own
+ * fixed device array (DION_NS_STATIC_SCRATCH_BYTES, part of the code object; every GPU the library
+ * runs on holds one copy until the process ends) takes the workspace's place.  No counterpart in
+ * the reference: it exists for callers that cannot allocate device memory or pass a workspace --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same
+ * arguments, same kernels and bit-identical results as dion_ns_orthogonalize.  A problem whose
+ * dion_ns_workspace_bytes() exceeds DION_NS_STATIC_SCRATCH_BYTES is refused with DION_E_WORKSPACE
+ * (dion_last_error() names both sizes).  The array's device address is looked up on the first call
+ * per device (hipGetSymbolAddress; make that first call outside a graph capture).  All calls on one
+ * GPU share the array: calls that overlap in time on the same GPU (different streams or threads)
+ * race; calls ordered on one stream are safe.  Nothing in the array needs to start at zero. */
+#define DION_NS_STATIC_SCRATCH_BYTES (64u << 20)
+int dion_ns_orthogonalize_static(const void* in, int in_dtype, void* out, int batch, int rows, int cols,
+                                 const float* coeffs, int n_iters, float norm_scale, float eps, int flags,
+                                 int gram_reset, void* stream);
+
 /* Orthogonalization and Muon update in one call: what dion_ns_orthogonalize followed by dion_muon_post
  * (bf16 update, no row_scale) does to the parameters, bit for bit, without the pass that writes the
  * orthogonalized matrices and the pass that reads them back.  Replaces the pair
