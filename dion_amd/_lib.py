@@ -14,9 +14,8 @@ LIB_PATH = os.path.join(_HERE, "libdion_hip.so")
 DION_BF16 = 0
 DION_F32 = 1
 DION_NS_GRAM = 1
-DION_NS_CARRY_XT = 2
 DION_NS_STATIC_SCRATCH_BYTES = 64 << 20
-ABI_VERSION = 10  # dion_abi_version() of the library these signatures describe
+ABI_VERSION = 11  # dion_abi_version() of the library these signatures describe
 
 _u64p = ctypes.POINTER(ctypes.c_uint64)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -28,13 +27,13 @@ SIGNATURES = {
     "dion_abi_version": (c_int, []),
     "dion_ns_line_1": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "dion_ns_line_2": (c_int, [c_void_p, c_void_p, c_int, c_int, c_float, c_float, c_void_p]),
-    "dion_ns_line_3": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                               c_float, c_void_p]),
+    "dion_ns_line_3": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "dion_ns_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "dion_ns_orthogonalize": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, _f32p, c_int,
                                       c_float, c_float, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "dion_ns_orthogonalize_static": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, _f32p, c_int,
                                              c_float, c_float, c_int, c_int, c_void_p]),
+    "dion_ns_plan_audit": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_size_t]),
     "dion_ns_update_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "dion_ns_orthogonalize_update": (c_int, [c_void_p, c_int, _u64p, c_int, c_int, c_int, c_int, c_int, _f32p,
                                              c_int, c_float, c_float, c_int, c_int, c_void_p, c_float, c_void_p,

@@ -5,6 +5,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <vector>
+
 #include "../../include/dion_hip.h"
 #include "elementwise.h"
 
@@ -35,7 +37,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 10; }
+extern "C" int dion_abi_version(void) { return 11; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -69,12 +71,12 @@ extern "C" int dion_ns_line_1(const void* X, void* A, int batch, int m, int k, v
   p.strideC = p.strideCt = (int64_t)m * m;
   p.ldp = p.ldq = k;
   p.ldc = p.ldct = m;
-  p.M = p.N = p.Mst = p.Nst = m;
+  p.M = p.N = m;
   p.K = k;
   p.batch = batch;
   p.tri = 1;
   p.alpha = 1.0f;
-  HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_1");
+  HIP_TRY(launch_gemm_nt(p, (hipStream_t)stream), "dion_ns_line_1");
   return DION_OK;
 }
 
@@ -92,119 +94,50 @@ extern "C" int dion_ns_line_2(const void* A, void* B, int batch, int m, float al
   p.C = p.Ct = (bf16_t*)B;
   p.strideP = p.strideQ = p.strideD = p.strideC = p.strideCt = (int64_t)m * m;
   p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = m;
-  p.M = p.N = p.K = p.Mst = p.Nst = m;
+  p.M = p.N = p.K = m;
   p.batch = batch;
   p.tri = 1;
   p.alpha = alpha;
   p.beta = beta;
-  HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_2");
+  HIP_TRY(launch_gemm_nt(p, (hipStream_t)stream), "dion_ns_line_2");
   return DION_OK;
 }
 
-extern "C" int dion_ns_line_3(const void* B, const void* X, const void* Xt, void* C, void* Ct,
-                              int batch, int m, int n, float a, void* stream) {
+extern "C" int dion_ns_line_3(const void* B, const void* X, void* C, int batch, int m, int n, float a,
+                              void* stream) {
   if (int rc = check_gemm_dims("dion_ns_line_3", batch, m, n)) return rc;
   if (batch == 0 || m == 0 || n == 0) return DION_OK;
-  if (!C && !Ct) return fail(DION_E_INVALID, "dion_ns_line_3: no output");
-  if (!B || (!X && !Xt)) return fail(DION_E_INVALID, "dion_ns_line_3: null argument");
+  if (!B || !X || !C) return fail(DION_E_INVALID, "dion_ns_line_3: null argument");
+  if (C == X) return fail(DION_E_INVALID, "dion_ns_line_3: in-place not supported");
   if (int rc = check_gemm_ptr("dion_ns_line_3", "B", B)) return rc;
   if (int rc = check_gemm_ptr("dion_ns_line_3", "X", X)) return rc;
-  if (int rc = check_gemm_ptr("dion_ns_line_3", "Xt", Xt)) return rc;
   if (int rc = check_gemm_ptr("dion_ns_line_3", "C", C)) return rc;
-  if (int rc = check_gemm_ptr("dion_ns_line_3", "Ct", Ct)) return rc;
   GemmParams p;
   memset(&p, 0, sizeof(p));
   p.P = (const bf16_t*)B;
-  p.Q = (const bf16_t*)Xt;
-  p.D = (const bf16_t*)X;
+  p.Q = (const bf16_t*)X;  // read as it lies: reduction index along rows
+  p.q_kmajor = 1;
+  p.D = a != 0.0f ? (const bf16_t*)X : nullptr;  // a == 0: pure product, X is not read a second time
   p.C = (bf16_t*)C;
-  p.Ct = (bf16_t*)Ct;
   p.strideP = (int64_t)m * m;
-  p.strideQ = p.strideD = p.strideC = p.strideCt = (int64_t)m * n;
+  p.strideQ = p.strideD = p.strideC = (int64_t)m * n;
   p.ldp = m;
-  p.ldq = m;
-  p.ldd = n;
-  p.ldc = n;
-  p.ldct = m;
-  p.M = p.Mst = m;
-  p.N = p.Nst = n;
+  p.ldq = p.ldd = p.ldc = n;
+  p.M = m;
+  p.N = n;
   p.K = m;
   p.batch = batch;
-  p.tri = 0;
   p.alpha = 1.0f;
   p.beta = a;
-  if (a == 0.0f) p.D = nullptr;  // pure product: the form the driver uses after folding a*I into B
-  if (!Ct && X) {
-    // X' alone: read X with the reduction index along rows; X^T is not needed
-    p.Q = (const bf16_t*)X;
-    p.ldq = n;
-    p.q_kmajor = 1;
-  } else if (!Xt) {
-    return fail(DION_E_INVALID, "dion_ns_line_3: Xt is required when Ct is requested");
-  }
-  if (p.D == nullptr && a != 0.0f) return fail(DION_E_INVALID, "dion_ns_line_3: X is required when a != 0");
-  HIP_TRY(launch_gemm_nt(p, -1, (hipStream_t)stream), "dion_ns_line_3");
+  HIP_TRY(launch_gemm_nt(p, (hipStream_t)stream), "dion_ns_line_3");
   return DION_OK;
 }
 
 // ---------------------------------------------------------------------------------------------
-// Whole orthogonalization
+// Whole orthogonalization.  A call is planned first -- buffer layout in the workspace and the full
+// list of kernel launches with their operands -- then the list is checked on the host against the
+// buffers the call owns, and only then launched.
 // ---------------------------------------------------------------------------------------------
-namespace {
-// Optional padding (elements) of the rows of the workspace matrices, for experiments with row
-// pitches that are not powers of two.  Measured on MI355X: pitches of 4 KiB multiples cost nothing
-// (the L2 channel hash spreads them), so the default is 0.
-static int ld_pad() {
-  static const int pad = [] {
-    const char* e = getenv("DION_LD_PAD");
-    int v = e ? atoi(e) : 0;
-    return v < 0 ? 0 : (v / 8) * 8;
-  }();
-  return pad;
-}
-
-struct NsPlan {
-  int m, n, mp, np, tall, nblk;
-  int ldx, ldxt, lda;  // row pitch (elements) of X [mp][np], X^T [np][mp], A/B [mp][mp]
-  size_t x_bytes, a_bytes, partial_bytes, inv_bytes, total;
-};
-
-NsPlan make_plan(int batch, int rows, int cols, int flags) {
-  NsPlan pl;
-  pl.tall = rows > cols;
-  pl.m = pl.tall ? cols : rows;
-  pl.n = pl.tall ? rows : cols;
-  const int g = gemm_pad_granule(pl.m, pl.n, batch);
-  pl.mp = round_up(pl.m, g);
-  pl.np = round_up(pl.n, g);
-  const int64_t numel = (int64_t)rows * cols;
-  int64_t nb = numel / (256 * 32);
-  if (nb < 1) nb = 1;
-  if (nb > 1024) nb = 1024;
-  pl.nblk = (int)nb;
-  pl.ldx = pl.np + ld_pad();
-  pl.ldxt = pl.mp + ld_pad();
-  pl.lda = pl.mp + ld_pad();
-  const size_t x_elems = (size_t)pl.mp * pl.ldx > (size_t)pl.np * pl.ldxt ? (size_t)pl.mp * pl.ldx
-                                                                          : (size_t)pl.np * pl.ldxt;
-  pl.x_bytes = align256((size_t)batch * x_elems * 2);
-  pl.a_bytes = align256((size_t)batch * pl.mp * pl.lda * 2);
-  pl.partial_bytes = align256((size_t)batch * pl.nblk * 4);
-  pl.inv_bytes = align256((size_t)batch * 4);
-  // X, Xt ping-pong pairs (default X-only form: the X pair and one X^T for a padded tall result);
-  // A, B (+ Q, Z, T for the Gram recurrence)
-  const int n_sq = (flags & DION_NS_GRAM) ? 6 : 2;
-  const int n_x = (flags & DION_NS_CARRY_XT) ? 4 : 3;
-  pl.total = n_x * pl.x_bytes + n_sq * pl.a_bytes + pl.partial_bytes + pl.inv_bytes;
-  return pl;
-}
-}  // namespace
-
-extern "C" size_t dion_ns_workspace_bytes(int batch, int rows, int cols, int flags) {
-  if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
-  return make_plan(batch, rows, cols, flags).total;
-}
-
 static bool table_aligned(const uint64_t* t, int n);
 static int check_state_dtype(const char* who, const char* arg, int dtype) {
   if (dtype != DION_BF16 && dtype != DION_F32)
@@ -214,6 +147,44 @@ static int check_state_dtype(const char* who, const char* arg, int dtype) {
 static inline int dt(int dtype) { return dtype == DION_BF16 ? 0 : 1; }
 
 namespace {
+struct NsPlan {
+  int m, n, mp, np, tall, nblk;
+  bool gram;  // the Gram-matrix recurrence is used (requested and worth it for this aspect ratio)
+  size_t x_bytes, a_bytes, partial_bytes, inv_bytes, total;
+};
+
+// The Gram recurrence trades rectangular GEMMs for m x m ones: 6 m^2 n + 20 m^3 executed FLOP
+// against 15 m^2 n + 5 m^3 for the standard iteration (five iterations, one restart), so it only
+// pays for n > 5/3 m; it also squares the condition number between restarts, which costs accuracy
+// on inputs that are not long (measured: 2.4e-2 from the exact result at n = 2.5 m, under 1e-2
+// from n = 3 m).  Both forms apply the same polynomial: below n = 3 m the standard iteration is
+// run whatever the flag says.
+bool gram_pays(int m, int n) { return (int64_t)n >= 3 * (int64_t)m; }
+
+NsPlan make_plan(int batch, int rows, int cols, int flags) {
+  NsPlan pl;
+  pl.tall = rows > cols;
+  pl.m = pl.tall ? cols : rows;
+  pl.n = pl.tall ? rows : cols;
+  pl.gram = (flags & DION_NS_GRAM) && gram_pays(pl.m, pl.n);
+  const int g = gemm_pad_granule(pl.m, pl.n, batch);
+  pl.mp = round_up(pl.m, g);
+  pl.np = round_up(pl.n, g);
+  const int64_t numel = (int64_t)rows * cols;
+  int64_t nb = numel / (256 * 32);
+  if (nb < 1) nb = 1;
+  if (nb > 1024) nb = 1024;
+  pl.nblk = (int)nb;
+  pl.x_bytes = align256((size_t)batch * pl.mp * pl.np * 2);
+  pl.a_bytes = align256((size_t)batch * pl.mp * pl.mp * 2);
+  pl.partial_bytes = align256((size_t)batch * pl.nblk * 4);
+  pl.inv_bytes = align256((size_t)batch * 4);
+  // X ping-pong pair + one X^T (the last product of a padded tall input); A, B (six m x m buffers
+  // for the Gram recurrence); norm partials and reciprocal norms
+  pl.total = 3 * pl.x_bytes + (pl.gram ? 6 : 2) * pl.a_bytes + pl.partial_bytes + pl.inv_bytes;
+  return pl;
+}
+
 // The Muon update that consumes the orthogonalized matrices (dion_ns_orthogonalize_update).
 struct PostSpec {
   const uint64_t* X_ptrs;
@@ -225,27 +196,80 @@ struct PostSpec {
   int cautious;
 };
 
-// per-head regime: whole iteration resident in LDS, one workgroup per matrix, no workspace
+// per-head regime: whole iteration resident in LDS, one workgroup per matrix, no workspace.  The Gram
+// flag changes nothing here: the recurrence saves memory traffic of rectangular GEMMs, and a matrix
+// that never leaves LDS has none; the standard iteration applies the same polynomial.
 bool ns_small_path(int rows, int cols, int flags, int n_iters) {
-  return !(flags & DION_NS_GRAM) && n_iters <= kMaxSmallIters && ns_small_fits(rows, cols) &&
-         !getenv("DION_NO_SMALL_KERNEL");
+  (void)flags;
+  return n_iters <= kMaxSmallIters && ns_small_fits(rows, cols);
 }
 
 // The update rides on the last GEMM when that GEMM produces the caller's tensor directly: at least
-// one iteration, the X-only form, no padding between the matrices and the tiles, not the
-// LDS-resident kernel.
+// one iteration, no padding between the matrices and the tiles, not the LDS-resident kernel.
 bool ns_update_fuses(int batch, int rows, int cols, int flags, int n_iters) {
-  if (n_iters <= 0 || (flags & DION_NS_CARRY_XT) || ns_small_path(rows, cols, flags, n_iters)) return false;
+  if (n_iters <= 0 || ns_small_path(rows, cols, flags, n_iters)) return false;
   const NsPlan pl = make_plan(batch, rows, cols, flags);
   return pl.mp == pl.m && pl.np == pl.n;
 }
-}  // namespace
 
-// Orthogonalization proper.  With `post` (only when ns_update_fuses) the last GEMM applies the update
-// to the parameters and `out` is not written.
-static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, int cols, const float* coeffs,
-                  int n_iters, float norm_scale, float eps, int flags, int gram_reset, void* workspace,
-                  size_t workspace_bytes, void* stream, const PostSpec* post) {
+// One kernel launch of a planned call.
+struct NsStep {
+  enum Kind { kNorm, kPrepare, kGemm, kGemmUpdate, kUnpad, kSmall } kind;
+  const char* what;
+  GemmParams g;    // kGemm, kGemmUpdate
+  FusedPost fp;    // kGemmUpdate
+  int x_code;      // kGemmUpdate: 0 bf16, 1 fp32 parameters
+  bool transposed; // kGemmUpdate: the product updates X[col][row]
+  // kNorm, kPrepare, kSmall: the caller's input
+  const void* in;
+  int in_dtype, batch, R, C;
+  float norm_scale, eps;
+  float* partial;
+  int nblk;
+  float* inv;
+  // kPrepare: X (same orientation as the input) and / or its transpose, padded to Rp x Cp
+  bf16_t* same;
+  int Rp, Cp, ld_same;
+  int64_t stride_same;
+  bf16_t* trans;
+  int ld_trans;
+  int64_t stride_trans;
+  // kUnpad: padded source -> dense destination;  kSmall: dst = the caller's output
+  const bf16_t* src;
+  int64_t src_stride;
+  int ld;
+  bf16_t* dst;
+  NsCoeffs co;  // kSmall
+};
+
+struct NsCall {
+  std::vector<NsStep> steps;
+  // what the call may read and write: [lo, hi) byte ranges
+  const char *in_lo, *in_hi, *out_lo, *out_hi, *ws_lo, *ws_hi;
+  // parameters updated in place by a fused update: n_ptrs ranges of x_bytes each
+  const uint64_t* X_ptrs;
+  int n_ptrs;
+  size_t x_bytes;
+};
+
+NsStep blank_step(NsStep::Kind kind, const char* what) {
+  NsStep s;
+  memset((void*)&s, 0, sizeof(s));
+  s.kind = kind;
+  s.what = what;
+  return s;
+}
+
+// Builds the launch list of one orthogonalization (no HIP call is made).  With `post` (only when
+// ns_update_fuses) the last GEMM applies the update to the parameters and `out` is not written.
+int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int cols, const float* coeffs,
+             int n_iters, float norm_scale, float eps, int flags, int gram_reset, void* workspace,
+             size_t workspace_bytes, const PostSpec* post, NsCall& call) {
+  call.steps.clear();
+  call.in_lo = call.in_hi = call.out_lo = call.out_hi = call.ws_lo = call.ws_hi = nullptr;
+  call.X_ptrs = nullptr;
+  call.n_ptrs = 0;
+  call.x_bytes = 0;
   if (batch < 0 || rows < 0 || cols < 0 || n_iters < 0)
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: negative extent");
   if (in_dtype != DION_BF16 && in_dtype != DION_F32)
@@ -253,15 +277,32 @@ static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, 
   if (batch == 0 || rows == 0 || cols == 0) return DION_OK;
   if (!in || (!out && !post) || (n_iters > 0 && !coeffs))
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: null argument");
-  if (flags & ~(DION_NS_GRAM | DION_NS_CARRY_XT)) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
-  hipStream_t st = (hipStream_t)stream;
+  if (flags & ~DION_NS_GRAM) return fail(DION_E_INVALID, "dion_ns_orthogonalize: flags 0x%x", flags);
+  const size_t mat_elems = (size_t)rows * cols;
+  call.in_lo = (const char*)in;
+  call.in_hi = call.in_lo + (size_t)batch * mat_elems * (in_dtype == DION_BF16 ? 2 : 4);
+  if (out) {
+    call.out_lo = (const char*)out;
+    call.out_hi = call.out_lo + (size_t)batch * mat_elems * 2;
+  }
+  if (post) {
+    call.X_ptrs = post->X_ptrs;
+    call.n_ptrs = post->n_ptrs;
+    call.x_bytes = (size_t)post->mats_per_ptr * mat_elems * (post->x_dtype == DION_BF16 ? 2 : 4);
+  }
   if (ns_small_path(rows, cols, flags, n_iters)) {
-    NsCoeffs co;
-    memset(&co, 0, sizeof(co));
-    co.n = n_iters;
-    for (int i = 0; i < n_iters * 3; ++i) co.c[i / 3][i % 3] = coeffs[i];
-    HIP_TRY(launch_ns_small(in, in_dtype, (bf16_t*)out, batch, rows, cols, co, norm_scale, eps, st),
-            "small-matrix Newton-Schulz");
+    NsStep s = blank_step(NsStep::kSmall, "small-matrix Newton-Schulz");
+    s.in = in;
+    s.in_dtype = in_dtype;
+    s.dst = (bf16_t*)out;
+    s.batch = batch;
+    s.R = rows;
+    s.C = cols;
+    s.norm_scale = norm_scale;
+    s.eps = eps;
+    s.co.n = n_iters;
+    for (int i = 0; i < n_iters * 3; ++i) s.co.c[i / 3][i % 3] = coeffs[i];
+    call.steps.push_back(s);
     return DION_OK;
   }
   // the last GEMM stores into the caller's buffer 16 bytes per lane
@@ -278,20 +319,16 @@ static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, 
                 pl.total);
   if (((uintptr_t)workspace & 255) != 0)
     return fail(DION_E_INVALID, "dion_ns_orthogonalize: workspace not 256-byte aligned");
+  call.ws_lo = (const char*)workspace;
+  call.ws_hi = call.ws_lo + workspace_bytes;
 
   char* w = (char*)workspace;
   bf16_t* X[2];
-  bf16_t* Xt[2];
   X[0] = (bf16_t*)w; w += pl.x_bytes;
   X[1] = (bf16_t*)w; w += pl.x_bytes;
-  Xt[0] = (bf16_t*)w; w += pl.x_bytes;
-  if (flags & DION_NS_CARRY_XT) {
-    Xt[1] = (bf16_t*)w; w += pl.x_bytes;
-  } else {
-    Xt[1] = Xt[0];  // only ever written by the last product
-  }
+  bf16_t* Xt = (bf16_t*)w; w += pl.x_bytes;
   bf16_t* sq[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};  // m x m scratch
-  for (int i = 0; i < ((flags & DION_NS_GRAM) ? 6 : 2); ++i) {
+  for (int i = 0; i < (pl.gram ? 6 : 2); ++i) {
     sq[i] = (bf16_t*)w;
     w += pl.a_bytes;
   }
@@ -299,92 +336,110 @@ static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, 
   float* inv = (float*)w; w += pl.inv_bytes;
 
   const int mp = pl.mp, np = pl.np;
-  const int ldx = pl.ldx, ldxt = pl.ldxt, lda = pl.lda;
-  const int64_t sX = (int64_t)mp * ldx, sXt = (int64_t)np * ldxt, sA = (int64_t)mp * lda;
-  HIP_TRY(launch_frobenius_inv(in, in_dtype, batch, (int64_t)rows * cols, norm_scale, eps, partial,
-                               pl.nblk, inv, st),
-          "frobenius norm");
-  // Default: X' = B X reads X itself (reduction index along rows) and no X^T is carried.
-  // DION_NS_CARRY_XT keeps X and X^T side by side instead.
-  // (With no iteration at all the result is the prepared input: keep both layouts then, the output
-  // copy reads X^T for a tall input.)
-  const bool nn = (flags & DION_NS_CARRY_XT) == 0 && n_iters > 0;
-  if (pl.tall)
-    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, nn ? nullptr : Xt[0], np, mp, ldxt, sXt,
-                              X[0], ldx, sX, st),
-            "prepare");
-  else
-    HIP_TRY(launch_ns_prepare(in, in_dtype, batch, rows, cols, inv, X[0], mp, np, ldx, sX,
-                              nn ? nullptr : Xt[0], ldxt, sXt, st),
-            "prepare");
+  const int64_t sX = (int64_t)mp * np, sA = (int64_t)mp * mp;
+  {
+    NsStep s = blank_step(NsStep::kNorm, "frobenius norm");
+    s.in = in;
+    s.in_dtype = in_dtype;
+    s.batch = batch;
+    s.R = rows;
+    s.C = cols;
+    s.norm_scale = norm_scale;
+    s.eps = eps;
+    s.partial = partial;
+    s.nblk = pl.nblk;
+    s.inv = inv;
+    call.steps.push_back(s);
+  }
+  {
+    // Only X (short side along rows) is carried between iterations: X' = B X reads X with the
+    // reduction index along rows.  With no iteration at all the result is the prepared input, and
+    // the output copy of a tall input reads X^T: prepare that layout instead.
+    NsStep s = blank_step(NsStep::kPrepare, "prepare");
+    s.in = in;
+    s.in_dtype = in_dtype;
+    s.batch = batch;
+    s.R = rows;
+    s.C = cols;
+    s.inv = inv;
+    if (pl.tall) {
+      s.Rp = np;
+      s.Cp = mp;
+      s.same = n_iters > 0 ? nullptr : Xt;
+      s.ld_same = mp;
+      s.stride_same = sX;
+      s.trans = n_iters > 0 ? X[0] : nullptr;
+      s.ld_trans = np;
+      s.stride_trans = sX;
+    } else {
+      s.Rp = mp;
+      s.Cp = np;
+      s.same = X[0];
+      s.ld_same = np;
+      s.stride_same = sX;
+    }
+    call.steps.push_back(s);
+  }
 
   const bool direct = (mp == pl.m && np == pl.n);
 
-  // ---- the four GEMM shapes of the iteration, all through launch_gemm_nt
+  // ---- the GEMM shapes of the iteration
   // sym(P, Q -> C): C = alpha P Q^T + beta D + diag I for symmetric m x m operands whose product
   // is symmetric; upper tiles computed, mirrored on store.
   // With tri == false the whole product is computed: needed when symmetry of the result rests on
   // the (bf16-rounded, hence only approximate) commutation of P and Q -- mirroring such a product
   // plants a commutator-sized error.
-  auto sym = [&](const bf16_t* P, const bf16_t* Q, const bf16_t* D, bf16_t* C, float alpha, float beta,
-                 float diag, bool tri = true) -> hipError_t {
-    GemmParams p;
-    memset(&p, 0, sizeof(p));
+  auto sym = [&](const char* what, const bf16_t* P, const bf16_t* Q, const bf16_t* D, bf16_t* C, float alpha,
+                 float beta, float diag, bool tri = true) {
+    NsStep s = blank_step(NsStep::kGemm, what);
+    GemmParams& p = s.g;
     p.P = P;
     p.Q = Q;
     p.D = D;
     p.C = C;
     p.Ct = tri ? C : nullptr;
     p.strideP = p.strideQ = p.strideD = p.strideC = p.strideCt = sA;
-    p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = lda;
-    p.M = p.N = p.K = p.Mst = p.Nst = mp;
+    p.ldp = p.ldq = p.ldd = p.ldc = p.ldct = mp;
+    p.M = p.N = p.K = mp;
     p.batch = batch;
     p.tri = tri ? 1 : 0;
     p.alpha = alpha;
     p.beta = beta;
     p.diag = diag;
-    return launch_gemm_nt(p, -1, st);
+    call.steps.push_back(s);
   };
   // gram(Xc -> R): R = Xc Xc^T
-  auto gram = [&](const bf16_t* Xc, bf16_t* R) -> hipError_t {
-    GemmParams p;
-    memset(&p, 0, sizeof(p));
+  auto gram = [&](const char* what, const bf16_t* Xc, bf16_t* R) {
+    NsStep s = blank_step(NsStep::kGemm, what);
+    GemmParams& p = s.g;
     p.P = p.Q = Xc;
     p.C = p.Ct = R;
     p.strideP = p.strideQ = sX;
     p.strideC = p.strideCt = sA;
-    p.ldp = p.ldq = ldx;
-    p.ldc = p.ldct = lda;
-    p.M = p.N = p.Mst = p.Nst = mp;
+    p.ldp = p.ldq = np;
+    p.ldc = p.ldct = mp;
+    p.M = p.N = mp;
     p.K = np;
     p.batch = batch;
     p.tri = 1;
     p.alpha = 1.0f;
-    return launch_gemm_nt(p, -1, st);
+    call.steps.push_back(s);
   };
-  // apply(S, Xtc -> Xn, Xtn | out): X' = S X given X^T (S symmetric m x m).  `final` writes the
-  // caller's tensor in its own orientation when no padding is in the way.
-  // In the X-only form (nn) the last product of a tall input is written transposed (the caller's
-  // orientation), every other one as X' alone.
-  auto apply = [&](const bf16_t* S, const bf16_t* Xc, const bf16_t* Xtc, bf16_t* Xn, bf16_t* Xtn,
-                   bool last, bool final_direct) -> hipError_t {
+  // apply(S, Xc -> Xn | Xt | out | parameters): X' = S X (S symmetric m x m).  The last product of a
+  // tall input is written transposed (the caller's orientation); when no padding is in the way
+  // (`final_direct`) it goes straight into the caller's tensor, or into the update of the parameters.
+  auto apply = [&](const char* what, const bf16_t* S, const bf16_t* Xc, bf16_t* Xn, bool last, bool final_direct) {
     GemmParams p;
     memset(&p, 0, sizeof(p));
     p.P = S;
     p.strideP = sA;
-    p.ldp = lda;
-    if (nn) {
-      p.Q = Xc;
-      p.strideQ = sX;
-      p.ldq = ldx;
-      p.q_kmajor = 1;
-    } else {
-      p.Q = Xtc;
-      p.strideQ = sXt;
-      p.ldq = ldxt;
-    }
-    p.M = p.Mst = mp;
-    p.N = p.Nst = np;
+    p.ldp = mp;
+    p.Q = Xc;
+    p.strideQ = sX;
+    p.ldq = np;
+    p.q_kmajor = 1;
+    p.M = mp;
+    p.N = np;
     p.K = mp;
     p.batch = batch;
     p.alpha = 1.0f;
@@ -392,64 +447,68 @@ static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, 
       // the product is consumed by the update: one launch per kMaxPtrs parameters
       const int mpp = post->mats_per_ptr;
       if (pl.tall) {
-        p.strideCt = (int64_t)mp * np;
+        p.strideCt = sX;
         p.ldct = mp;
       } else {
-        p.strideC = (int64_t)mp * np;
+        p.strideC = sX;
         p.ldc = np;
       }
       for (int c0 = 0; c0 < post->n_ptrs; c0 += kMaxPtrs) {
         const int c = (post->n_ptrs - c0) < kMaxPtrs ? (post->n_ptrs - c0) : kMaxPtrs;
         const int64_t b0 = (int64_t)c0 * mpp;
-        GemmParams q = p;
-        q.P = p.P + b0 * p.strideP;
-        q.Q = p.Q + b0 * p.strideQ;
-        q.batch = c * mpp;
-        FusedPost fp;
-        memset(&fp, 0, sizeof(fp));
-        memcpy(fp.X.p, post->X_ptrs + c0, (size_t)c * sizeof(uint64_t));
-        fp.mats_per_ptr = mpp;
-        fp.vec_ok = table_aligned(post->X_ptrs + c0, c) ? 1 : 0;
-        fp.lr_dev = post->lr_dev;
-        fp.wd_dev = post->wd_dev;
-        fp.wd_host = post->wd_host;
-        fp.adj_ratio = post->adj_ratio;
-        fp.cautious = post->cautious;
-        if (hipError_t e = launch_gemm_nt_post(q, fp, dt(post->x_dtype), pl.tall != 0, st)) return e;
+        NsStep s = blank_step(NsStep::kGemmUpdate, what);
+        s.g = p;
+        s.g.P = p.P + b0 * p.strideP;
+        s.g.Q = p.Q + b0 * p.strideQ;
+        s.g.batch = c * mpp;
+        memcpy(s.fp.X.p, post->X_ptrs + c0, (size_t)c * sizeof(uint64_t));
+        s.fp.mats_per_ptr = mpp;
+        s.fp.vec_ok = table_aligned(post->X_ptrs + c0, c) ? 1 : 0;
+        s.fp.lr_dev = post->lr_dev;
+        s.fp.wd_dev = post->wd_dev;
+        s.fp.wd_host = post->wd_host;
+        s.fp.adj_ratio = post->adj_ratio;
+        s.fp.cautious = post->cautious;
+        s.x_code = dt(post->x_dtype);
+        s.transposed = pl.tall != 0;
+        call.steps.push_back(s);
       }
-      return hipSuccess;
+      return;
     }
     if (final_direct) {
       if (pl.tall) {
         p.Ct = (bf16_t*)out;
-        p.strideCt = (int64_t)mp * np;
+        p.strideCt = sX;
         p.ldct = mp;
       } else {
         p.C = (bf16_t*)out;
-        p.strideC = (int64_t)mp * np;
+        p.strideC = sX;
         p.ldc = np;
       }
+    } else if (last && pl.tall) {
+      p.Ct = Xt;
+      p.strideCt = sX;
+      p.ldct = mp;
     } else {
-      p.C = (nn && last && pl.tall) ? nullptr : Xn;
-      p.Ct = (nn && !(last && pl.tall)) ? nullptr : Xtn;
+      p.C = Xn;
       p.strideC = sX;
-      p.strideCt = sXt;
-      p.ldc = ldx;
-      p.ldct = ldxt;
+      p.ldc = np;
     }
-    return launch_gemm_nt(p, -1, st);
+    NsStep s = blank_step(NsStep::kGemm, what);
+    s.g = p;
+    call.steps.push_back(s);
   };
 
   int cur = 0;
   bool wrote_out = false;
-  if (!(flags & DION_NS_GRAM)) {
+  if (!pl.gram) {
     for (int it = 0; it < n_iters; ++it) {
       const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
-      HIP_TRY(gram(X[cur], sq[0]), "A = X X^T");
+      gram("A = X X^T", X[cur], sq[0]);
       // a*I folded into B: the next GEMM needs no addend (one fewer pass over X)
-      HIP_TRY(sym(sq[0], sq[0], sq[0], sq[1], c, b, a), "B = c A A + b A + a I");
+      sym("B = c A A + b A + a I", sq[0], sq[0], sq[0], sq[1], c, b, a);
       const bool fin = (it == n_iters - 1) && direct;
-      HIP_TRY(apply(sq[1], X[cur], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], it == n_iters - 1, fin), "X = B X");
+      apply("X = B X", sq[1], X[cur], X[cur ^ 1], it == n_iters - 1, fin);
       wrote_out = fin;
       cur ^= 1;
     }
@@ -468,24 +527,24 @@ static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, 
       return -1;
     };
     int r = take(), q = -1;
-    HIP_TRY(gram(X[cur], sq[r]), "R = X X^T");
+    gram("R = X X^T", X[cur], sq[r]);
     for (int it = 0; it < n_iters; ++it) {
       const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
       if (it == gram_reset && it > 0 && q >= 0) {
-        HIP_TRY(apply(sq[q], X[cur], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], false, false), "X = Q X (restart)");
+        apply("X = Q X (restart)", sq[q], X[cur], X[cur ^ 1], false, false);
         cur ^= 1;
         used[q] = false;
         q = -1;
-        HIP_TRY(gram(X[cur], sq[r]), "R = X X^T (restart)");
+        gram("R = X X^T (restart)", X[cur], sq[r]);
       }
       const int z = take();
-      HIP_TRY(sym(sq[r], sq[r], sq[r], sq[z], c, b, a), "Z = a I + b R + c R R");
+      sym("Z = a I + b R + c R R", sq[r], sq[r], sq[r], sq[z], c, b, a);
       const bool need_r = !(it == n_iters - 1 || (it + 1 == gram_reset));
       if (need_r) {
         const int t = take();
-        HIP_TRY(sym(sq[z], sq[r], nullptr, sq[t], 1.0f, 0.0f, 0.0f, false), "T = Z R");
+        sym("T = Z R", sq[z], sq[r], nullptr, sq[t], 1.0f, 0.0f, 0.0f, false);
         const int rn = take();
-        HIP_TRY(sym(sq[t], sq[z], nullptr, sq[rn], 1.0f, 0.0f, 0.0f), "R = T Z");
+        sym("R = T Z", sq[t], sq[z], nullptr, sq[rn], 1.0f, 0.0f, 0.0f);
         used[t] = false;
         used[r] = false;
         r = rn;
@@ -494,26 +553,169 @@ static int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, 
         q = z;  // Q = Z (Q was the identity)
       } else {
         const int qn = take();
-        HIP_TRY(sym(sq[z], sq[q], nullptr, sq[qn], 1.0f, 0.0f, 0.0f, false), "Q = Z Q");
+        sym("Q = Z Q", sq[z], sq[q], nullptr, sq[qn], 1.0f, 0.0f, 0.0f, false);
         used[q] = false;
         used[z] = false;
         q = qn;
       }
     }
     if (q >= 0) {
-      HIP_TRY(apply(sq[q], X[cur], Xt[cur], X[cur ^ 1], Xt[cur ^ 1], true, direct), "X = Q X");
+      apply("X = Q X", sq[q], X[cur], X[cur ^ 1], true, direct);
       wrote_out = direct;
       cur ^= 1;
     }
   }
   if (!wrote_out) {
     if (post) return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: update not applied (internal)");
-    if (pl.tall)
-      HIP_TRY(launch_unpad(Xt[cur], sXt, ldxt, (bf16_t*)out, batch, rows, cols, st), "unpad");
-    else
-      HIP_TRY(launch_unpad(X[cur], sX, ldx, (bf16_t*)out, batch, rows, cols, st), "unpad");
+    NsStep s = blank_step(NsStep::kUnpad, "unpad");
+    // a tall result lies transposed-back in Xt: written there by the last product, or by the
+    // prepare step when there was no iteration
+    s.src = pl.tall ? Xt : X[cur];
+    s.src_stride = sX;
+    s.ld = pl.tall ? mp : np;
+    s.dst = (bf16_t*)out;
+    s.batch = batch;
+    s.R = rows;
+    s.C = cols;
+    call.steps.push_back(s);
   }
   return DION_OK;
+}
+
+// ---- host-side bounds check of a planned call: every byte a launch reads lies inside the caller's
+// input or the workspace, every byte it writes inside the workspace, the caller's output or (fused
+// update) one parameter; tile shapes divide the padded extents.
+bool inside(const void* lo, size_t bytes, const char* r_lo, const char* r_hi) {
+  const char* p = (const char*)lo;
+  return r_lo && p >= r_lo && p <= r_hi && bytes <= (size_t)(r_hi - p);
+}
+
+// bytes spanned by `batch` matrices of `rows` x `cols` elements of `es` bytes, row pitch ld, batch stride
+size_t span_bytes(int batch, int64_t stride, int rows, int ld, int cols, int es) {
+  if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
+  return ((size_t)(batch - 1) * (size_t)stride + (size_t)(rows - 1) * (size_t)ld + (size_t)cols) * (size_t)es;
+}
+
+int ns_audit(const NsCall& call) {
+  auto rd = [&](const void* p, size_t bytes) {
+    return inside(p, bytes, call.in_lo, call.in_hi) || inside(p, bytes, call.ws_lo, call.ws_hi);
+  };
+  auto wr = [&](const void* p, size_t bytes) {
+    return inside(p, bytes, call.ws_lo, call.ws_hi) || inside(p, bytes, call.out_lo, call.out_hi);
+  };
+  int idx = 0;
+  for (const NsStep& s : call.steps) {
+    const char* bad = nullptr;
+    switch (s.kind) {
+      case NsStep::kNorm: {
+        const size_t es = s.in_dtype == DION_BF16 ? 2 : 4;
+        if (!rd(s.in, (size_t)s.batch * s.R * s.C * es)) bad = "input";
+        else if (!wr(s.partial, (size_t)s.batch * s.nblk * 4)) bad = "norm partials";
+        else if (!wr(s.inv, (size_t)s.batch * 4)) bad = "reciprocal norms";
+        break;
+      }
+      case NsStep::kPrepare: {
+        const size_t es = s.in_dtype == DION_BF16 ? 2 : 4;
+        if (s.Rp % 64 || s.Cp % 64 || s.Rp < s.R || s.Cp < s.C) bad = "padded extents";
+        else if (!rd(s.in, (size_t)s.batch * s.R * s.C * es)) bad = "input";
+        else if (!rd(s.inv, (size_t)s.batch * 4)) bad = "reciprocal norms";
+        else if (s.same && !wr(s.same, span_bytes(s.batch, s.stride_same, s.Rp, s.ld_same, s.Cp, 2))) bad = "X";
+        else if (s.trans && !wr(s.trans, span_bytes(s.batch, s.stride_trans, s.Cp, s.ld_trans, s.Rp, 2)))
+          bad = "X^T";
+        else if (!s.same && !s.trans) bad = "no destination";
+        break;
+      }
+      case NsStep::kGemm:
+      case NsStep::kGemmUpdate: {
+        const GemmParams& p = s.g;
+        const int tile = gemm_tile_edge(p);
+        if (p.M % tile || p.N % tile || p.K % 128 || (p.tri && p.M != p.N)) bad = "tile does not divide the extents";
+        else if (!rd(p.P, span_bytes(p.batch, p.strideP, p.M, p.ldp, p.K, 2))) bad = "first operand";
+        else if (!(p.q_kmajor ? rd(p.Q, span_bytes(p.batch, p.strideQ, p.K, p.ldq, p.N, 2))
+                              : rd(p.Q, span_bytes(p.batch, p.strideQ, p.N, p.ldq, p.K, 2))))
+          bad = "second operand";
+        else if (p.D && !rd(p.D, span_bytes(p.batch, p.strideD, p.M, p.ldd, p.N, 2))) bad = "addend";
+        else if (p.C && !wr(p.C, span_bytes(p.batch, p.strideC, p.M, p.ldc, p.N, 2))) bad = "product";
+        else if (p.Ct && !wr(p.Ct, span_bytes(p.batch, p.strideCt, p.N, p.ldct, p.M, 2))) bad = "transposed product";
+        else if (s.kind == NsStep::kGemm && !p.C && !p.Ct) bad = "no destination";
+        else if (s.kind == NsStep::kGemmUpdate) {
+          // matrix b updates parameter b / mats_per_ptr at matrix offset b % mats_per_ptr
+          const int es = s.x_code == 0 ? 2 : 4;
+          const int mpp = s.fp.mats_per_ptr;
+          const size_t one = s.transposed ? span_bytes(1, 0, p.N, p.ldct, p.M, es) : span_bytes(1, 0, p.M, p.ldc, p.N, es);
+          const size_t stride = (size_t)(s.transposed ? p.strideCt : p.strideC) * es;
+          if (mpp <= 0 || p.batch > kMaxPtrs * mpp || p.C || p.Ct) bad = "update batch";
+          else if ((size_t)(mpp - 1) * stride + one > call.x_bytes) bad = "parameter extent";
+          else
+            for (int i = 0; i < (p.batch + mpp - 1) / mpp && !bad; ++i)
+              if (!s.fp.X.p[i]) bad = "null parameter";
+        }
+        break;
+      }
+      case NsStep::kUnpad:
+        if (!rd(s.src, span_bytes(s.batch, s.src_stride, s.R, s.ld, s.C, 2))) bad = "padded source";
+        else if (!wr(s.dst, (size_t)s.batch * s.R * s.C * 2)) bad = "output";
+        break;
+      case NsStep::kSmall: {
+        const size_t es = s.in_dtype == DION_BF16 ? 2 : 4;
+        if (!rd(s.in, (size_t)s.batch * s.R * s.C * es)) bad = "input";
+        else if (!wr(s.dst, (size_t)s.batch * s.R * s.C * 2)) bad = "output";
+        break;
+      }
+    }
+    if (bad)
+      return fail(DION_E_INVALID, "dion_ns_orthogonalize: launch %d (%s) would access its %s outside the call's buffers",
+                  idx, s.what, bad);
+    ++idx;
+  }
+  return DION_OK;
+}
+
+int ns_execute(const NsCall& call, hipStream_t st) {
+  for (const NsStep& s : call.steps) {
+    hipError_t e = hipSuccess;
+    switch (s.kind) {
+      case NsStep::kNorm:
+        e = launch_frobenius_inv(s.in, s.in_dtype, s.batch, (int64_t)s.R * s.C, s.norm_scale, s.eps, s.partial,
+                                 s.nblk, s.inv, st);
+        break;
+      case NsStep::kPrepare:
+        e = launch_ns_prepare(s.in, s.in_dtype, s.batch, s.R, s.C, s.inv, s.same, s.Rp, s.Cp, s.ld_same,
+                              s.stride_same, s.trans, s.ld_trans, s.stride_trans, st);
+        break;
+      case NsStep::kGemm:
+        e = launch_gemm_nt(s.g, st);
+        break;
+      case NsStep::kGemmUpdate:
+        e = launch_gemm_nt_post(s.g, s.fp, s.x_code, s.transposed, st);
+        break;
+      case NsStep::kUnpad:
+        e = launch_unpad(s.src, s.src_stride, s.ld, s.dst, s.batch, s.R, s.C, st);
+        break;
+      case NsStep::kSmall:
+        e = launch_ns_small(s.in, s.in_dtype, s.dst, s.batch, s.R, s.C, s.co, s.norm_scale, s.eps, st);
+        break;
+    }
+    if (e != hipSuccess) return hip_fail(e, s.what);
+  }
+  return DION_OK;
+}
+
+int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, int cols, const float* coeffs,
+           int n_iters, float norm_scale, float eps, int flags, int gram_reset, void* workspace,
+           size_t workspace_bytes, void* stream, const PostSpec* post) {
+  NsCall call;
+  if (int rc = ns_build(in, in_dtype, out, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
+                        workspace, workspace_bytes, post, call))
+    return rc;
+  if (int rc = ns_audit(call)) return rc;
+  return ns_execute(call, (hipStream_t)stream);
+}
+}  // namespace
+
+extern "C" size_t dion_ns_workspace_bytes(int batch, int rows, int cols, int flags) {
+  if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
+  return make_plan(batch, rows, cols, flags).total;
 }
 
 extern "C" int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, int rows,
@@ -560,7 +762,7 @@ extern "C" int dion_ns_orthogonalize_static(const void* in, int in_dtype, void* 
                                             int cols, const float* coeffs, int n_iters, float norm_scale,
                                             float eps, int flags, int gram_reset, void* stream) {
   size_t need = 0;
-  if (batch > 0 && rows > 0 && cols > 0 && !(flags & ~(DION_NS_GRAM | DION_NS_CARRY_XT)) && n_iters >= 0 &&
+  if (batch > 0 && rows > 0 && cols > 0 && !(flags & ~DION_NS_GRAM) && n_iters >= 0 &&
       !ns_small_path(rows, cols, flags, n_iters))
     need = make_plan(batch, rows, cols, flags).total;
   if (need > (size_t)DION_NS_STATIC_SCRATCH_BYTES)
@@ -579,7 +781,7 @@ extern "C" int dion_ns_orthogonalize_static(const void* in, int in_dtype, void* 
 
 extern "C" size_t dion_ns_update_workspace_bytes(int batch, int rows, int cols, int flags, int n_iters) {
   if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
-  const size_t ns = align256(make_plan(batch, rows, cols, flags).total);
+  const size_t ns = ns_small_path(rows, cols, flags, n_iters) ? 0 : align256(make_plan(batch, rows, cols, flags).total);
   if (ns_update_fuses(batch, rows, cols, flags, n_iters)) return ns;
   return ns + align256((size_t)batch * rows * cols * 2);
 }
@@ -600,24 +802,69 @@ extern "C" int dion_ns_orthogonalize_update(const void* in, int in_dtype, const 
   if (!X_ptrs || !lr_dev) return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: null argument");
   for (int i = 0; i < n_ptrs; ++i)
     if (!X_ptrs[i]) return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: parameter %d is null", i);
-  if (workspace_bytes < dion_ns_update_workspace_bytes(batch, rows, cols, flags, n_iters))
-    return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize_update: workspace %zu < %zu bytes", workspace_bytes,
-                dion_ns_update_workspace_bytes(batch, rows, cols, flags, n_iters));
+  const size_t need = dion_ns_update_workspace_bytes(batch, rows, cols, flags, n_iters);
+  if (workspace_bytes < need)
+    return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize_update: workspace %zu < %zu bytes", workspace_bytes, need);
   if (ns_update_fuses(batch, rows, cols, flags, n_iters)) {
     const PostSpec ps = {X_ptrs, x_dtype, n_ptrs, mats_per_ptr, lr_dev, adj_ratio, wd_dev, wd_host, cautious};
     return ns_run(in, in_dtype, nullptr, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
                   workspace, workspace_bytes, stream, &ps);
   }
-  // padded shapes, the X / X^T form, the LDS-resident kernel: orthogonalize into the tail of the
-  // workspace, then the plain update pass
-  const size_t ns = align256(make_plan(batch, rows, cols, flags).total);
+  // padded shapes and the LDS-resident kernel: orthogonalize into the tail of the workspace (the
+  // last align256(batch * rows * cols * 2) bytes of what dion_ns_update_workspace_bytes reports),
+  // then the plain update pass
+  const size_t tail = align256((size_t)batch * rows * cols * 2);
+  const size_t ns = need - tail;
   if (!workspace) return fail(DION_E_WORKSPACE, "dion_ns_orthogonalize_update: workspace is null");
+  if (((uintptr_t)workspace & 255) != 0)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize_update: workspace not 256-byte aligned");
   void* tmp = (char*)workspace + ns;
   if (int rc = ns_run(in, in_dtype, tmp, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
                       workspace, ns, stream, nullptr))
     return rc;
   return dion_muon_post(X_ptrs, x_dtype, tmp, DION_BF16, n_ptrs, (int64_t)mats_per_ptr * rows * cols, cols,
                         nullptr, lr_dev, nullptr, adj_ratio, wd_dev, wd_host, cautious, stream);
+}
+
+// Host-only check of the planning code: builds the launch list of dion_ns_orthogonalize
+// (with_update == 0) or of the fused form of dion_ns_orthogonalize_update (with_update != 0, when
+// the shape fuses) over synthetic, never dereferenced addresses and checks it as every real call
+// is checked before its first launch.  audit_ws_bytes > 0 checks against a workspace of that size
+// instead of the size the plan was laid out for.
+extern "C" int dion_ns_plan_audit(int batch, int rows, int cols, int in_dtype, int n_iters, int flags,
+                                  int gram_reset, int with_update, int x_dtype, int mats_per_ptr,
+                                  size_t audit_ws_bytes) {
+  if (batch <= 0 || rows <= 0 || cols <= 0 || n_iters < 0 || n_iters > 16 || mats_per_ptr <= 0)
+    return fail(DION_E_INVALID, "dion_ns_plan_audit: bad size");
+  if (int rc = check_state_dtype("dion_ns_plan_audit", "x_dtype", x_dtype)) return rc;
+  float coeffs[48];
+  for (int i = 0; i < 48; ++i) coeffs[i] = 1.0f;
+  const bool small = ns_small_path(rows, cols, flags, n_iters);
+  const size_t ws_bytes = small ? 0 : make_plan(batch, rows, cols, flags).total;
+  // disjoint synthetic regions, 1 TiB apart
+  char* const base = (char*)(uintptr_t)0x100000000000ull;
+  const size_t gap = (size_t)1 << 40;
+  void* in = base;
+  void* out = base + gap;
+  void* ws = base + 2 * gap;
+  NsCall call;
+  std::vector<uint64_t> xp;
+  PostSpec ps;
+  const bool fused = with_update && ns_update_fuses(batch, rows, cols, flags, n_iters);
+  if (with_update && !fused)
+    return fail(DION_E_INVALID, "dion_ns_plan_audit: this shape does not take the fused update");
+  if (fused) {
+    if (batch % mats_per_ptr) return fail(DION_E_INVALID, "dion_ns_plan_audit: batch %% mats_per_ptr != 0");
+    const int n_ptrs = batch / mats_per_ptr;
+    for (int i = 0; i < n_ptrs; ++i) xp.push_back((uint64_t)(uintptr_t)(base + (size_t)(4 + i) * gap));
+    ps = {xp.data(), x_dtype, n_ptrs, mats_per_ptr, (const float*)(base + 3 * gap), 1.0f, nullptr, 0.0f, 0};
+  }
+  if (int rc = ns_build(in, in_dtype, fused ? nullptr : out, batch, rows, cols, coeffs, n_iters, 1.0f, 0.0f, flags,
+                        gram_reset, small ? nullptr : ws, ws_bytes, fused ? &ps : nullptr, call))
+    return rc;
+  if (audit_ws_bytes > 0 && call.ws_lo) call.ws_hi = call.ws_lo + audit_ws_bytes;
+  if (int rc = ns_audit(call)) return rc;
+  return (int)call.steps.size();
 }
 
 // ---------------------------------------------------------------------------------------------

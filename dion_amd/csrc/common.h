@@ -172,18 +172,17 @@ static inline hipError_t set_max_dynamic_lds_once(const void* fn, int bytes, std
 
 // One batched C = alpha * P * Q^T + beta * D problem, all operands row-major bf16 with the
 // reduction dimension contiguous ("NT" GEMM).  M, N, K are the computed extents and must be
-// multiples of the tile the launcher picks; Mst/Nst bound the stores (<= M, N) so the last
-// GEMM of a chain can write into an unpadded destination.
+// multiples of the tile the launcher picks; whole tiles are stored, so destinations are padded
+// to the tile as well.
 struct GemmParams {
   const bf16_t* P;   // [batch][M][K], leading dimension ldp
   const bf16_t* Q;   // [batch][N][K], leading dimension ldq (== P when tri); [batch][K][N] if q_kmajor
   const bf16_t* D;   // optional [batch][M][N] addend, leading dimension ldd
-  bf16_t* C;         // optional [batch][Mst][Nst]
-  bf16_t* Ct;        // optional [batch][Nst][Mst] (transposed copy; == C when tri -> mirror)
+  bf16_t* C;         // optional [batch][M][N]
+  bf16_t* Ct;        // optional [batch][N][M] (transposed copy; == C when tri -> mirror)
   int64_t strideP, strideQ, strideD, strideC, strideCt;  // batch strides in elements
   int ldp, ldq, ldd, ldc, ldct;
   int M, N, K;
-  int Mst, Nst;
   int batch;
   int tri;           // 1: Q == P, only tiles with tile_row <= tile_col are computed, Ct mirrors
   int q_kmajor;      // 1: Q is stored [K][N] (reduction index along rows); not with tri
@@ -192,8 +191,11 @@ struct GemmParams {
   float diag;        // added to C[i][i] (global diagonal); used with tri to fold a*I into B
 };
 
-// Returns hipSuccess or the launch error.  variant < 0 picks by shape.
-hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream);
+// Returns hipSuccess or the launch error; the tile configuration is picked by shape.
+hipError_t launch_gemm_nt(const GemmParams& p, hipStream_t stream);
+// Tile edge (128 or 256) launch_gemm_nt / launch_gemm_nt_post use for this problem: M and N must be
+// multiples of it, K of 128.
+int gemm_tile_edge(const GemmParams& p);
 // C = P * Q with Q K-major (p.q_kmajor, no tri, no D), the product consumed by the fused Muon update
 // instead of being stored: `transposed` false updates X[row][col] (ldc / strideC describe X),
 // true updates X[col][row] (ldct / strideCt).  x_dtype 0 = bf16, 1 = fp32.  p.batch <= kMaxPtrs *

@@ -19,8 +19,6 @@
 // (v_mfma_f32_32x32x16_bf16).  Operand tiles reach a two-slot LDS ring through direct-to-LDS
 // loads (global_load_lds_dwordx4, no VGPR staging); XOR swizzles keep the LDS writes and the
 // fragment reads bank-conflict free.
-#include <stdlib.h>
-
 #include <type_traits>
 
 #include "common.h"
@@ -639,13 +637,7 @@ typedef TileCfg<256, 256, 64, 2, 4, 2> Cfg256w8;   // 8 wavefronts, 128x64 each:
 
 // Tile list dealt to the XCDs in interleaved 32-tile chunks (see the kernel) when the first operand of
 // one matrix is at least 16 MB; below that a contiguous run per XCD keeps whole matrices in one L2.
-static bool xcd_interleave_pays(const GemmParams& p) {
-  static const long thresh = [] {
-    const char* e = getenv("DION_XCD_INTERLEAVE_BYTES");
-    return e ? atol(e) : (16L << 20);
-  }();
-  return (int64_t)p.M * p.K * 2 >= thresh;
-}
+static bool xcd_interleave_pays(const GemmParams& p) { return (int64_t)p.M * p.K * 2 >= (16L << 20); }
 
 template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false, int POST = 0>
 static hipError_t launch_epi(const GemmParams& p, hipStream_t stream,
@@ -664,6 +656,7 @@ static hipError_t launch_epi(const GemmParams& p, hipStream_t stream,
   return hipGetLastError();
 }
 
+// The operand / result combinations the Newton-Schulz drivers use.
 template <class Cfg>
 static hipError_t launch_cfg(const GemmParams& p, hipStream_t stream) {
   if (p.M % Cfg::BM || p.N % Cfg::BN || p.K % (Cfg::BK * Cfg::NSTAGE)) return hipErrorInvalidValue;
@@ -675,12 +668,9 @@ static hipError_t launch_cfg(const GemmParams& p, hipStream_t stream) {
     if (d && c && !ct) return launch_epi<Cfg, true, true, false, true>(p, stream);    // a X + B X
     return hipErrorInvalidValue;
   }
-  if (!d && c && ct) return launch_epi<Cfg, false, true, true>(p, stream);   // A = X X^T
-  if (d && c && ct) return launch_epi<Cfg, true, true, true>(p, stream);     // B, X' (both layouts)
-  if (d && c && !ct) return launch_epi<Cfg, true, true, false>(p, stream);   // last X'
-  if (d && !c && ct) return launch_epi<Cfg, true, false, true>(p, stream);   // last (X')^T
-  if (!d && c && !ct) return launch_epi<Cfg, false, true, false>(p, stream); // plain product
-  if (!d && !c && ct) return launch_epi<Cfg, false, false, true>(p, stream); // transposed product
+  if (p.tri && !d && c && ct) return launch_epi<Cfg, false, true, true>(p, stream);   // A = X X^T, R = T Z
+  if (p.tri && d && c && ct) return launch_epi<Cfg, true, true, true>(p, stream);     // B = c A A + b A (+ a I)
+  if (!p.tri && !d && c && !ct) return launch_epi<Cfg, false, true, false>(p, stream); // full product of two symmetric matrices
   return hipErrorInvalidValue;
 }
 
@@ -692,16 +682,14 @@ int gemm_pad_granule(int m, int n, int batch) {
   return syrk_tiles >= 256 ? 256 : 128;
 }
 
-// 256-wide tiles only when there are enough of them to keep 256 CUs busy for a few rounds; below that
-// the 128-wide tiles (two workgroups per CU) win.
+// 256-wide tiles only when there are enough of them (512) to keep 256 CUs busy for a few rounds; below
+// that the 128-wide tiles (two workgroups per CU) win.
 static bool wants_256_tiles(const GemmParams& p) {
-  static const long thresh = [] {
-    const char* e = getenv("DION_TILE_THRESH");
-    return e ? atol(e) : 512L;
-  }();
   const long t256 = (long)(p.M / 256) * (p.tri ? (p.M / 256 + 1) / 2 + 0 : p.N / 256) * p.batch;
-  return p.M % 256 == 0 && p.N % 256 == 0 && t256 >= thresh;
+  return p.M % 256 == 0 && p.N % 256 == 0 && t256 >= 512L;
 }
+
+int gemm_tile_edge(const GemmParams& p) { return wants_256_tiles(p) ? 256 : 128; }
 
 template <class Cfg>
 static hipError_t launch_post_cfg(const GemmParams& p, const FusedPost& post, int x_dtype, bool transposed,
@@ -727,17 +715,10 @@ hipError_t launch_gemm_nt_post(const GemmParams& p, const FusedPost& post, int x
                             : launch_post_cfg<Cfg128>(p, post, x_dtype, transposed, stream);
 }
 
-hipError_t launch_gemm_nt(const GemmParams& p, int variant, hipStream_t stream) {
+hipError_t launch_gemm_nt(const GemmParams& p, hipStream_t stream) {
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.batch <= 0) return hipSuccess;
-  if (variant < 0) {
-    variant = wants_256_tiles(p) ? 3 : 1;
-  }
   if (p.tri && (p.M != p.N)) return hipErrorInvalidValue;
-  switch (variant) {
-    case 1: return launch_cfg<Cfg128>(p, stream);
-    case 3: return launch_cfg<Cfg256w8>(p, stream);
-    default: return hipErrorInvalidValue;
-  }
+  return wants_256_tiles(p) ? launch_cfg<Cfg256w8>(p, stream) : launch_cfg<Cfg128>(p, stream);
 }
 
 }  // namespace dion

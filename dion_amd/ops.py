@@ -13,7 +13,7 @@ from torch import Tensor
 from torch.utils._python_dispatch import is_traceable_wrapper_subclass
 
 from . import _lib
-from ._lib import DION_BF16, DION_F32, DION_NS_GRAM, DION_NS_CARRY_XT, check, ptr_table
+from ._lib import DION_BF16, DION_F32, DION_NS_GRAM, check, ptr_table
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -155,8 +155,8 @@ def ns_line_3(B: Tensor, X: Tensor, a: float, *, out: Optional[Tensor] = None) -
     mp, np_ = Xp.shape[-2:]
     res = torch.empty(b, mp, np_, dtype=torch.bfloat16, device=X.device)
     lib = _lib.load()
-    check(lib.dion_ns_line_3(Bp.data_ptr(), Xp.data_ptr(), None, res.data_ptr(), None, b, mp,
-                             np_, float(a), _stream_handle(X.device)), "ns_line_3")
+    check(lib.dion_ns_line_3(Bp.data_ptr(), Xp.data_ptr(), res.data_ptr(), b, mp, np_, float(a),
+                             _stream_handle(X.device)), "ns_line_3")
     res = res[:, :m, :n]
     if squeeze:
         res = res[0]
@@ -167,12 +167,11 @@ def ns_line_3(B: Tensor, X: Tensor, a: float, *, out: Optional[Tensor] = None) -
 
 
 def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: float, epsilon: float,
-                     gram: bool = False, gram_reset: int = 0, carry_xt: bool = False) -> Tensor:
+                     gram: bool = False, gram_reset: int = 0) -> Tensor:
     """Batched Newton-Schulz / Polar-Express orthogonalization of ``G[..., rows, cols]``.
 
     X0 = bf16(G) / (||bf16(G)||_F * norm_scale + epsilon), then ``len(coeffs)`` quintic
     iterations on the orientation with rows <= cols; result is bf16 with the shape of ``G``.
-    ``carry_xt`` keeps X and X^T side by side between iterations instead of X alone (same result).
     """
     _require_gpu(G, "G")
     if G.ndim < 2:
@@ -187,7 +186,7 @@ def ns_orthogonalize(G: Tensor, coeffs: Sequence[Sequence[float]], norm_scale: f
     if out.numel() == 0:
         return out.reshape(shape)
     carr, n_iters = _flat_coeffs(coeffs)
-    flags = (DION_NS_GRAM if gram else 0) | (DION_NS_CARRY_XT if carry_xt else 0)
+    flags = DION_NS_GRAM if gram else 0
     lib = _lib.load()
     chunk = 32768  # one library call takes at most 65535 matrices
     for b0 in range(0, batch, chunk):
@@ -210,7 +209,7 @@ def _flat_coeffs(coeffs):
 
 def ns_orthogonalize_update(G: Tensor, X: List[Tensor], coeffs: Sequence[Sequence[float]], norm_scale: float,
                             epsilon: float, lr: Tensor, adj_ratio: float, weight_decay, cautious_wd: bool = False,
-                            gram: bool = False, gram_reset: int = 0, carry_xt: bool = False) -> None:
+                            gram: bool = False, gram_reset: int = 0) -> None:
     """``muon_post(X, ns_orthogonalize(G, ...), lr, adj_ratio, weight_decay, cautious_wd)`` in one library
     call, with the same result bit for bit (dion/muon.py:249-277).  ``G`` is ``[..., rows, cols]`` with
     ``len(X) * mats`` matrices; every ``X[i]`` is a contiguous fp32 or bf16 parameter of ``mats * rows *
@@ -235,11 +234,11 @@ def ns_orthogonalize_update(G: Tensor, X: List[Tensor], coeffs: Sequence[Sequenc
     xp, xcode = _state_ptrs(X, "X", mats_per_ptr * rows * cols)
     lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, G.device)
     if batch > 32768:  # past one library call: the two-pass form, which splits the batch
-        O = ns_orthogonalize(G3, coeffs, norm_scale, epsilon, gram, gram_reset, carry_xt)
+        O = ns_orthogonalize(G3, coeffs, norm_scale, epsilon, gram, gram_reset)
         muon_post(X, O.view(n, -1), lr, adj_ratio, weight_decay, cautious_wd)
         return
     carr, n_iters = _flat_coeffs(coeffs)
-    flags = (DION_NS_GRAM if gram else 0) | (DION_NS_CARRY_XT if carry_xt else 0)
+    flags = DION_NS_GRAM if gram else 0
     lib = _lib.load()
     ws = _workspace(G.device, lib.dion_ns_update_workspace_bytes(batch, rows, cols, flags, n_iters))
     check(lib.dion_ns_orthogonalize_update(G3.data_ptr(), _dtype_code(G3, "G"), xp, xcode, n, mats_per_ptr, rows,

@@ -54,12 +54,11 @@ int dion_ns_line_1(const void* X, void* A, int batch, int m, int k, void* stream
  * (dion/newton_schulz_triton.py:290-333, kernel :206-287). */
 int dion_ns_line_2(const void* A, void* B, int batch, int m, float alpha, float beta, void* stream);
 
-/* C[b] = a X[b] + B[b] X[b] given X^T: B [batch,m,m] symmetric, X [batch,m,n], Xt = X^T
- * [batch,n,m].  Writes C [batch,m,n] and/or Ct = C^T [batch,n,m] (either may be NULL).  With
- * a == 0 the addend is skipped altogether (X is not read).
+/* C[b] = a X[b] + B[b] X[b]: B [batch,m,m] symmetric, X and C [batch,m,n] (C != X).  X is read as
+ * it lies (reduction index along rows; transposing LDS reads in the kernel), so no X^T is needed.
+ * With a == 0 the addend is skipped altogether (X is read once).
  * Replaces ns_line_3 (dion/newton_schulz_triton.py:450-491) and the baddbmm at :557-563. */
-int dion_ns_line_3(const void* B, const void* X, const void* Xt, void* C, void* Ct, int batch,
-                   int m, int n, float a, void* stream);
+int dion_ns_line_3(const void* B, const void* X, void* C, int batch, int m, int n, float a, void* stream);
 
 /* --------------------------------------------------------------------------------------------
  * Whole orthogonalization: the operator behind `newton_schulz_func(input, epsilon)`
@@ -73,16 +72,14 @@ int dion_ns_line_3(const void* B, const void* X, const void* Xt, void* C, void* 
  *   X0 = bf16(in) / (||bf16(in)||_F * norm_scale + eps)  per matrix, then n_iters times
  *   A = X X^T; B = b A + c A A; X = a X + B X   on the orientation with rows <= cols.
  *   flags: DION_NS_GRAM selects the Gram-matrix recurrence (call site
- *   dion/megabatch_base.py:77-94) with a restart at iteration `gram_reset` (<=0: none).
+ *   dion/megabatch_base.py:77-94) with a restart at iteration `gram_reset` (<=0: none).  Both forms
+ *   apply the same polynomial; the recurrence only saves work for long matrices, so it is used
+ *   when max(rows, cols) >= 3 min(rows, cols) and the standard iteration otherwise.
  * workspace: device scratch of at least dion_ns_workspace_bytes() bytes, 256-byte aligned.
+ * Every launch of a call is checked on the host against the buffers the call owns (in, out,
+ * workspace) before the first one is issued.
  * ------------------------------------------------------------------------------------------ */
 #define DION_NS_GRAM 1
-/* By default only X is kept between iterations: X' = B X reads X with the reduction index along
- * rows (register-staged loads, transposing LDS reads).  DION_NS_CARRY_XT selects the other form,
- * X and X^T carried side by side with both GEMM operands contiguous along the reduction index
- * (one more store per iteration, a workspace one X larger).  Same arithmetic, bit-identical
- * result. */
-#define DION_NS_CARRY_XT 2
 size_t dion_ns_workspace_bytes(int batch, int rows, int cols, int flags);
 int dion_ns_orthogonalize(const void* in, int in_dtype, void* out, int batch, int rows, int cols,
                           const float* coeffs, int n_iters, float norm_scale, float eps, int flags,
@@ -104,13 +101,25 @@ int dion_ns_orthogonalize_static(const void* in, int in_dtype, void* out, int ba
                                  const float* coeffs, int n_iters, float norm_scale, float eps, int flags,
                                  int gram_reset, void* stream);
 
+/* Host-only self-check of the planning code (no device work, usable without a GPU): builds the launch
+ * list of dion_ns_orthogonalize (with_update == 0) or of the fused form of
+ * dion_ns_orthogonalize_update (with_update != 0; DION_E_INVALID if the shape does not fuse) over
+ * synthetic, never dereferenced addresses and runs the bounds check every real call runs before
+ * its first launch: each launch's reads inside the input or the workspace, its writes inside the
+ * workspace, the output or one parameter, tile shapes dividing the padded extents.  Returns the
+ * number of kernel launches, or a negative DION_E_* code (dion_last_error() names the launch and
+ * the operand).  audit_ws_bytes > 0 checks against a workspace of that many bytes instead of the
+ * size the plan was laid out for.  No counterpart in the reference. */
+int dion_ns_plan_audit(int batch, int rows, int cols, int in_dtype, int n_iters, int flags, int gram_reset,
+                       int with_update, int x_dtype, int mats_per_ptr, size_t audit_ws_bytes);
+
 /* Orthogonalization and Muon update in one call: what dion_ns_orthogonalize followed by dion_muon_post
  * (bf16 update, no row_scale) does to the parameters, bit for bit, without the pass that writes the
  * orthogonalized matrices and the pass that reads them back.  Replaces the pair
  * `muon_update_newton_schulz` + `muon_update_post_orthogonalize`, dion/muon.py:249-277.
  * in: [n_ptrs * mats_per_ptr, rows, cols] as for dion_ns_orthogonalize; X_ptrs: host array of n_ptrs
  * device pointers, each to mats_per_ptr contiguous [rows, cols] matrices of x_dtype, updated in place.
- * When the matrices fill whole tiles (rows, cols multiples of 128; X-only form; more than 64 rows or
+ * When the matrices fill whole tiles (rows, cols multiples of 128; more than 64 rows or
  * columns on the short side) the last GEMM applies the update in its epilogue; otherwise the library
  * runs the two passes itself, through the tail of the workspace.  Workspace size from
  * dion_ns_update_workspace_bytes (same flags and n_iters).  lr / weight decay as for dion_muon_post. */

@@ -79,7 +79,9 @@ def test_library_exports_every_declared_symbol():
     n = lib.dion_ns_workspace_bytes(2, 768, 3072, 0)
     assert n >= 2 * 768 * 3072 * 2 * 3  # X ping-pong pair + one X^T
     assert lib.dion_ns_workspace_bytes(2, 3072, 768, 0) == n
-    assert lib.dion_ns_workspace_bytes(2, 768, 3072, _lib.DION_NS_CARRY_XT) >= n + 2 * 768 * 3072 * 2
+    # Gram recurrence: four more m x m buffers, but only where it is used (long matrices)
+    assert lib.dion_ns_workspace_bytes(2, 768, 3072, _lib.DION_NS_GRAM) >= n + 4 * 2 * 768 * 768 * 2
+    assert lib.dion_ns_workspace_bytes(2, 768, 1024, _lib.DION_NS_GRAM) == lib.dion_ns_workspace_bytes(2, 768, 1024, 0)
 
 
 def test_missing_library_is_a_hard_error(monkeypatch, tmp_path):
@@ -137,12 +139,11 @@ def test_argument_validation_happens_before_any_device_work():
             "in_dtype")
     refused(lib.dion_ns_line_1(None, None, 1, 128, 128, None), "null argument")
     refused(lib.dion_ns_line_2(None, None, 1, 128, f(1.0), f(1.0), None), "null argument")
-    refused(lib.dion_ns_line_3(None, None, None, None, None, 1, 128, 128, f(0.0), None), "no output")
+    refused(lib.dion_ns_line_3(None, None, None, 1, 128, 128, f(0.0), None), "null argument")
     refused(lib.dion_ns_line_1(None, None, 1, 100, 128, None), "multiples of 128")
     refused(lib.dion_ns_line_1(0x1002, 0x2000, 1, 128, 128, None), "X is not 16-byte aligned")
     refused(lib.dion_ns_line_2(0x1000, 0x2008, 1, 128, f(1.0), f(1.0), None), "B is not 16-byte aligned")
-    refused(lib.dion_ns_line_3(0x1000, 0x2000, None, 0x3004, None, 1, 128, 128, f(0.0), None),
-            "C is not 16-byte aligned")
+    refused(lib.dion_ns_line_3(0x1000, 0x2000, 0x3004, 1, 128, 128, f(0.0), None), "C is not 16-byte aligned")
     refused(lib.dion_ns_orthogonalize(0x1000, 0, 0x2002, 1, 128, 128, (ctypes.c_float * 3)(1.0, 1.0, 1.0), 1, f(1.0),
                                       f(0.0), 0, 0, 0x4000, 1 << 30, None), "out is not 16-byte aligned")
     # empty problems are accepted and do nothing

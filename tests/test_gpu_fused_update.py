@@ -14,7 +14,7 @@ BF = torch.bfloat16
 
 
 def _run_both(shape, n, xdtype, cautious, gram=False, wd=0.01, offset_view=False, coeffs=None, norm_scale=1.0,
-              eps=1e-7, carry_xt=False):
+              eps=1e-7):
     from dion_amd import newton_schulz as ns
     from dion_amd import ops
 
@@ -37,11 +37,10 @@ def _run_both(shape, n, xdtype, cautious, gram=False, wd=0.01, offset_view=False
     lr = torch.tensor(0.02, device=DEV)
     rows, cols = shape[-2:]
     Xa, Xb = fresh(), fresh()
-    O = ops.ns_orthogonalize(U.view(-1, rows, cols), coeffs, norm_scale, eps, gram=gram, gram_reset=2,
-                             carry_xt=carry_xt)
+    O = ops.ns_orthogonalize(U.view(-1, rows, cols), coeffs, norm_scale, eps, gram=gram, gram_reset=2)
     ops.muon_post(Xa, O.view(n, -1), lr, 0.7, wd, cautious)
     ops.ns_orthogonalize_update(U.view(-1, rows, cols), Xb, coeffs, norm_scale, eps, lr, 0.7, wd, cautious,
-                                gram=gram, gram_reset=2, carry_xt=carry_xt)
+                                gram=gram, gram_reset=2)
     return X0, O.view(n, *shape), Xa, Xb
 
 
@@ -94,7 +93,7 @@ def test_more_parameters_than_one_launch_holds(shape):
     assert all(torch.equal(a, b) for a, b in zip(Xa, Xb))
 
 
-@pytest.mark.parametrize("shape", [(256, 512), (512, 256)])
+@pytest.mark.parametrize("shape", [(256, 512), (512, 256), (256, 768), (768, 256)])
 def test_schedules_and_options(shape):
     from dion_amd import newton_schulz as ns
 
@@ -102,7 +101,6 @@ def test_schedules_and_options(shape):
                dict(coeffs=ns.POLAR_EXPRESS_COEFFS, norm_scale=1.02, eps=1e-6),
                dict(coeffs=[ns.KJ_COEFFS] * 3),
                dict(coeffs=[]),  # no iteration: the prepared input is the update
-               dict(carry_xt=True),
                dict(wd=torch.tensor(0.05, device=DEV))):
         _X0, _O, Xa, Xb = _run_both(shape, 2, torch.float32, False, **kw)
         assert all(torch.equal(a, b) for a, b in zip(Xa, Xb)), kw

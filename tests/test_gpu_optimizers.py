@@ -36,8 +36,8 @@ def _run_steps(cls, params, kwargs, n_steps=3):
 @pytest.mark.parametrize("shape", [(256, 1024), (1024, 256), (768, 768)])
 def test_muon_step_vs_oracle(shape, ns_kwargs, ns_name):
     """GPT-small-like group: bf16 N(0, 0.02) grads, fp32 zero momentum, mu 0.95 nesterov, wd 0.01,
-    lr 0.02, three steps.  Momentum bit exact; orthogonalized update within 2e-2 of the exact
-    result (see test_gpu_newton_schulz.py for why the bound is against exact arithmetic);
+    lr 0.02, three steps.  Momentum bit exact; orthogonalized update within 2e-2 of the reference's eager
+    path for NS5, within 2e-2 of the exact result for Polar-Express (see test_gpu_golden.py for why);
     parameters within 1e-5 relative when both sides apply the same update."""
     from dion import Muon
 
@@ -62,7 +62,18 @@ def test_muon_step_vs_oracle(shape, ns_kwargs, ns_name):
             # update actually applied on the GPU, recovered from the parameters
             a = 1 - torch.tensor(0.02) * torch.tensor(0.01)
             u_gpu = (x_before[i].cpu() * a - params[i].data.cpu()) / (0.02 * ratio)
-            assert _rel(u_gpu, Uo[i].float()) <= (2e-2 if ns_name == "ns5" else 6e-2)
+            if ns_name == "ns5":
+                assert _rel(u_gpu, Uo[i].float()) <= 2e-2
+            else:
+                # Polar-Express: the reference's eager path is itself 4-5e-2 from the exact result
+                # (tests/test_gpu_golden.py); hold the applied update to 2e-2 of exact and to the
+                # distance independent roundings of those sizes allow from the eager path.  (u_gpu
+                # is recovered from fp32 parameters: 2e-3 of slack for that division.)
+                _, u_in = oracle.muon_pre(G[i], M[i], 0.95, True)
+                exact = torch.from_numpy(oracle.ns_fp64(u_in.float().numpy(), oracle.POLAR_EXPRESS_COEFFS, 1.02, 1e-8))
+                e_ref = _rel(Uo[i].float(), exact)
+                assert _rel(u_gpu, exact) <= 2.2e-2
+                assert _rel(u_gpu, Uo[i].float()) <= 1.05 * (e_ref ** 2 + 2.2e-2 ** 2) ** 0.5
             # same-U parity of the fp32 parameter update
             x_same = oracle.muon_post(x_before[i].cpu(), u_gpu.to(torch.bfloat16), 0.02, ratio, 0.01)
             assert _rel(params[i].data, x_same) <= 1e-5

@@ -1,7 +1,10 @@
-"""Pins the CPU oracle (oracle/dion_oracle.py) without running the reference: closed forms,
-invariants, brute force on tiny inputs and the bounds the reference's own tests state.  A dropped
+"""Pins the CPU oracle (oracle/dion_oracle.py): closed forms, invariants, brute force on tiny inputs, the
+bounds the reference's own tests state, and -- for the bf16 rounding sequence of the orthogonalization
+functions, which nothing else fixes -- the output vectors the reference's own functions wrote
+(tests/golden/ns_vectors.npz, made by tests/golden/make_vectors.py).  A dropped
 term, a wrong sign or a transposed operand in the oracle fails at least one of these."""
 import math
+import os
 
 import numpy as np
 import pytest
@@ -99,6 +102,87 @@ def test_bf16_paths_track_fp64():
     k1 = o.kj_ns_bf16(G).float()
     k2 = o.kj_ns_bf16(G.T.contiguous()).float().T
     assert float((k1 - k2).norm() / k1.norm()) < 6e-2
+
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ns_vectors.npz")
+GOLDEN_SHAPES = [(64, 128), (128, 64), (128, 128), (4, 64, 128), (96, 160), (160, 96)]
+
+
+def golden_case(z, name, kind, shape):
+    """(input bf16 tensor, reference output bf16 tensor) of tests/golden/ns_vectors.npz."""
+    tag = "x".join(str(v) for v in shape)
+
+    def t(a):
+        return torch.from_numpy(a.astype(np.int16)).view(torch.bfloat16)
+
+    return t(z[f"in_{tag}"]), t(z[f"{name}_{kind}_{tag}"])
+
+
+def _rel(a, b) -> float:
+    a = a.double() if isinstance(a, torch.Tensor) else torch.from_numpy(np.asarray(a, dtype=np.float64))
+    b = b.double() if isinstance(b, torch.Tensor) else torch.from_numpy(np.asarray(b, dtype=np.float64))
+    return float((a - b).norm() / b.norm())
+
+
+@pytest.mark.parametrize("shape", GOLDEN_SHAPES)
+def test_eager_restatements_equal_the_references_own_outputs_bit_for_bit(shape):
+    """ns_bf16 / polar_express_bf16 / kj_ns_bf16 against the vectors the reference's undecorated functions
+    wrote on the same inputs (tests/golden/make_vectors.py): same torch-CPU ops in the same order, so the
+    bf16 bits must be equal.  A dropped term, a wrong coefficient, a transposed operand or a different
+    normalisation order in the oracle changes them."""
+    z = np.load(GOLDEN)
+    G, want = golden_case(z, "ns5", "eager", shape)
+    assert torch.equal(o.ns_bf16(G, o.NS5_COEFFS, 1.0, 1e-7), want)
+    G, want = golden_case(z, "pe", "eager", shape)
+    assert torch.equal(o.polar_express_bf16(G, eps=1e-6), want)
+    if len(shape) == 2:
+        G, want = golden_case(z, "kj", "eager", shape)
+        assert torch.equal(o.kj_ns_bf16(G, 5, 1e-7), want)
+
+
+@pytest.mark.parametrize("name,coeffs,scale,eps", [("ns5", o.NS5_COEFFS, 1.0, 1e-7),
+                                                   ("pe", o.POLAR_EXPRESS_COEFFS, 1.02, 1e-6),
+                                                   ("kj", o.KJ_COEFFS, 1.0, 1e-7)])
+def test_reference_outputs_follow_the_fp64_restatement(name, coeffs, scale, eps):
+    """Both of the reference's own paths (eager and torch.compile'd, golden vectors) sit within their bf16
+    noise of ns_fp64 with the cited coefficient table: pins ns_fp64 and the tables against real reference
+    output.  The noise levels themselves are what the GPU tolerances are derived from: NS5 <= 2e-2;
+    Polar-Express up to 4.6e-2 (eager) / 3.6e-2 (compiled); KJ up to 3.1e-2 / 2.2e-2 -- and the reference's
+    two paths differ from EACH OTHER by more than 2e-2 on every Polar-Express and KJ case."""
+    z = np.load(GOLDEN)
+    bound = {"ns5": (2.0e-2, 1.6e-2), "pe": (4.8e-2, 3.8e-2), "kj": (3.3e-2, 2.4e-2)}[name]
+    for shape in GOLDEN_SHAPES:
+        if name == "kj" and len(shape) != 2:
+            continue
+        G, eager = golden_case(z, name, "eager", shape)
+        _, comp = golden_case(z, name, "compiled", shape)
+        x = o.ns_fp64(G.float().numpy(), coeffs, scale, eps)
+        assert _rel(eager, x) <= bound[0], (shape, _rel(eager, x))
+        assert _rel(comp, x) <= bound[1], (shape, _rel(comp, x))
+        if name != "ns5":
+            assert _rel(comp, eager) > 2e-2, (shape, _rel(comp, eager))
+
+
+@pytest.mark.parametrize("fn,coeffs,scale", [
+    (lambda g: o.kj_ns_bf16(g, 5, 0.0), o.KJ_COEFFS, 1.0),
+    (lambda g: o.polar_express_bf16(g, eps=0.0), o.POLAR_EXPRESS_COEFFS, 1.02),
+    (lambda g: o.ns_bf16(g, o.NS5_COEFFS, 1.0, 0.0), o.NS5_COEFFS, 1.0),
+    (lambda g: o.ns_bf16_fused(g, o.POLAR_EXPRESS_COEFFS, 1.02, 0.0), o.POLAR_EXPRESS_COEFFS, 1.02),
+])
+def test_bf16_restatements_map_singular_values_through_the_quintics(fn, coeffs, scale):
+    """Closed form for the bf16 paths: on G = U diag(s) V^T the result is U diag(phi(s / (scale ||s||))) V^T
+    within bf16 noise, wide and tall.  Dropping the c A A term, or a sign, moves phi by O(1)."""
+    m, n = 48, 96
+    s = np.linspace(0.3, 1.0, m)
+    U, V, G = _rand_svd(m, n, s, 5)
+    phi = o.scalar_map(s / (np.linalg.norm(s) * scale), coeffs)
+    want = (U * phi) @ V.T
+    got = fn(torch.from_numpy(G).float()).float().numpy().astype(np.float64)
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 6e-2
+    got_t = fn(torch.from_numpy(G.T.copy()).float()).float().numpy().astype(np.float64)
+    assert np.linalg.norm(got_t - want.T) / np.linalg.norm(want) < 6e-2
+    sv = np.linalg.svd(got, compute_uv=False)
+    assert abs(sv.max() - phi.max()) < 0.08 and abs(sv.min() - phi.min()) < 0.08
 
 
 def test_muon_pre_first_step_closed_form():
