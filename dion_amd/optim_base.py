@@ -18,6 +18,50 @@ from . import newton_schulz as ns
 from . import scalar_opts
 
 
+class LiveScalars:
+    """Hyper-parameters the kernels read from device memory instead of taking by value.
+
+    The reference keeps ``lr`` of every param group in a 0-d float32 device tensor whose identity
+    never changes, and ``weight_decay`` too once the caller has passed it as a Tensor
+    (dion/megabatch_base.py:417-501): LR schedulers and hand-rolled schedules keep assigning floats
+    to ``group["lr"]``, a captured graph keeps reading the same address.  This class owns those
+    tensors, one per (group index, name).
+    """
+
+    def __init__(self):
+        self._slots: Dict[Tuple[int, str], Tensor] = {}
+
+    def tensors(self) -> List[Tensor]:
+        return list(self._slots.values())
+
+    def _wanted(self, index: int, group: dict) -> Tuple[str, ...]:
+        # weight decay stays live once it has been: a later float assignment updates the tensor
+        if isinstance(group.get("weight_decay"), Tensor) or (index, "weight_decay") in self._slots:
+            return ("lr", "weight_decay")
+        return ("lr",)
+
+    def bind(self, index: int, group: dict) -> None:
+        if not group["params"]:
+            return
+        device = group["params"][0].device
+        for name in self._wanted(index, group):
+            slot = self._slots.get((index, name))
+            current = group[name]
+            if slot is not None and current is slot:
+                continue  # nothing was assigned since the last bind
+            if device.type == "cuda" and torch.cuda.is_current_stream_capturing():
+                # a write recorded into a graph would replay the capture-time value forever
+                raise RuntimeError(
+                    f"group {index}: {name} was assigned ({type(current).__name__}) while a graph capture is in "
+                    "progress; assign hyper-parameters before capture starts"
+                )
+            if slot is None or slot.device != device:
+                slot = torch.zeros((), dtype=torch.float32, device=device)
+                self._slots[(index, name)] = slot
+            slot.copy_(current) if isinstance(current, Tensor) else slot.fill_(float(current))
+            group[name] = slot
+
+
 class OrthoOptimizer(Optimizer):
     """Base class: orchestration, state and validation.  Subclasses implement
     ``_shape_group_phases`` (a generator: work before / during / after the orthogonalization)."""
@@ -67,26 +111,26 @@ class OrthoOptimizer(Optimizer):
 
         # State for every parameter exists from construction on, so state_dict() has the same keys
         # before and after the first step (dion/megabatch_base.py:114-137).
-        self._state_prepopulated = False
-        self._hyper_tensors: Dict[Tuple[int, str], Tensor] = {}
-        self._live_names: Dict[int, Tuple[str, ...]] = {}
+        self._scalars = LiveScalars()
+        self._constructed = False
         for group in self.param_groups:
-            self._prepopulate(group)
-        self._sync_hyperparam_tensors()
-        self._state_prepopulated = True
+            self._create_state(group)
+        self.bind_live_scalars()
+        self._constructed = True
 
     # ------------------------------------------------------------------ state
-    def _prepopulate(self, group: dict) -> None:
+    def _create_state(self, group: dict) -> None:
         for p in group["params"]:
             self._get_or_initialize_state(p, group["algorithm"])
 
     def add_param_group(self, param_group: dict) -> None:
+        """torch calls this from ``Optimizer.__init__`` for every group and users call it later; only a
+        late group needs its state and device scalars made here (construction does it for all at once)."""
         super().add_param_group(param_group)
-        if getattr(self, "_state_prepopulated", False):
-            index = len(self.param_groups) - 1
-            for name in self._live_hyperparams(index):
-                self._ensure_hyperparam_tensor(index, name)
-            self._prepopulate(self.param_groups[-1])
+        if not getattr(self, "_constructed", False):
+            return
+        self._scalars.bind(len(self.param_groups) - 1, self.param_groups[-1])
+        self._create_state(self.param_groups[-1])
 
     def _get_or_initialize_state(self, param: Tensor, algo: str) -> dict:
         state = self.state[param]
@@ -99,143 +143,96 @@ class OrthoOptimizer(Optimizer):
         return state
 
     # ------------------------------------------------- live hyper-parameters
-    def _live_hyperparams(self, index: int) -> Tuple[str, ...]:
-        """``lr`` always lives in a persistent 0-d device tensor; ``weight_decay`` does once the
-        caller has supplied a Tensor for it (dion/megabatch_base.py:417-448)."""
-        live = self._live_names.get(index)
-        if live is None or "weight_decay" not in live:
-            if isinstance(self.param_groups[index].get("weight_decay"), Tensor):
-                live = ("lr", "weight_decay")
-            elif live is None:
-                live = ("lr",)
-            self._live_names[index] = live
-        return live
+    def bind_live_scalars(self) -> None:
+        """Make ``group["lr"]`` (and a ``weight_decay`` the caller gave as a Tensor) of every group the
+        group's own persistent 0-d device tensor, carrying whatever value is assigned right now."""
+        for index, group in enumerate(self.param_groups):
+            self._scalars.bind(index, group)
 
-    def _ensure_hyperparam_tensor(self, index: int, name: str) -> Optional[Tensor]:
-        """Keep ``param_groups[index][name]`` bound to one 0-d float32 device tensor whose identity
-        never changes; floats (or foreign tensors) assigned by the caller are copied into it
-        (dion/megabatch_base.py:450-501)."""
-        group = self.param_groups[index]
-        if not group["params"]:
-            return None
-        value = group[name]
-        tensor = self._hyper_tensors.get((index, name))
-        if value is tensor and tensor is not None:
-            return tensor
-        device = group["params"][0].device
-        if device.type == "cuda" and torch.cuda.is_current_stream_capturing():
-            raise RuntimeError(
-                f"param group {index} has a {name} that is not its persistent device tensor "
-                f"({type(value).__name__}) and graph capture is already underway; sync {name} "
-                "before capturing."
-            )
-        if tensor is None or tensor.device != device:
-            tensor = torch.empty((), dtype=torch.float32, device=device)
-            self._hyper_tensors[(index, name)] = tensor
-        if isinstance(value, Tensor):
-            tensor.copy_(value)
-        else:
-            tensor.fill_(value)
-        group[name] = tensor
-        return tensor
+    def live_scalar_tensors(self) -> List[Tensor]:
+        """The persistent device tensors the step kernels read hyper-parameters from."""
+        return self._scalars.tensors()
 
-    @property
-    def _hyperparam_tensors(self) -> Dict[Tuple[int, str], Tensor]:
-        """The persistent device tensors behind ``lr`` (and an opted-in ``weight_decay``); a graph
-        wrapper compares their count before and after capture (dion/cuda_graph.py:212-229)."""
-        return self._hyper_tensors
-
-    def _advance_host_step_counters(self) -> None:
-        """Host-side bookkeeping of one step that a graph replay does not execute
-        (dion/cuda_graph.py:307-311)."""
+    def count_skipped_host_step(self) -> None:
+        """The one piece of host state a step changes (``group["step"]``), for a caller that ran the
+        step's device work without running ``step()`` -- a graph replay."""
         for group in self.param_groups:
             group["step"] += 1
 
-    def _sync_hyperparam_tensors(self) -> None:
-        for index in range(len(self.param_groups)):
-            for name in self._live_hyperparams(index):
-                self._ensure_hyperparam_tensor(index, name)
-
     def state_dict(self):
+        """Checkpoints carry plain floats where a group holds a 0-d tensor, so they load into any
+        optimizer on any device (dion/megabatch_base.py:521-538)."""
         sd = super().state_dict()
-        for group in sd["param_groups"]:
-            for key, value in group.items():
-                if key != "params" and isinstance(value, Tensor) and value.ndim == 0:
-                    group[key] = value.item()
+        sd["param_groups"] = [
+            {k: (v.item() if k != "params" and isinstance(v, Tensor) and v.ndim == 0 else v) for k, v in g.items()}
+            for g in sd["param_groups"]
+        ]
         return sd
 
     def load_state_dict(self, state_dict):
         super().load_state_dict(state_dict)
-        self._sync_hyperparam_tensors()
+        self.bind_live_scalars()
+        # AdamW's device step counter: float32 on the parameter's device whatever the checkpoint
+        # held, and rebuilt from the group's host counter when the checkpoint predates it
         for group in self.param_groups:
             if group["algorithm"] != "adamw":
                 continue
             for p in group["params"]:
-                state = self.state.get(p)
-                if state is None:
+                if p not in self.state:
                     continue
-                step = state.get("step_dev")
-                if step is None:
-                    step = torch.full((), float(group["step"]), dtype=torch.float32, device=p.device)
-                elif step.dtype != torch.float32 or step.device != p.device:
-                    step = step.to(dtype=torch.float32, device=p.device)
-                state["step_dev"] = step
+                saved = self.state[p].get("step_dev")
+                value = float(group["step"]) if saved is None else float(saved)
+                self.state[p]["step_dev"] = torch.full((), value, dtype=torch.float32, device=p.device)
 
     # ------------------------------------------------------------ validation
+    # How a group's 2D weights are cut into independent matrices: ``num_heads`` equal row bands
+    # (per-head orthogonalization, dion/megabatch_base.py:304-364) or ``split_sizes`` uneven row blocks
+    # (fused projections, :911-981).  One or the other, never with flatten.
+    @staticmethod
+    def _positive_int(value) -> bool:
+        return isinstance(value, int) and not isinstance(value, bool) and value >= 1
+
     def _resolve_num_heads(self, group: dict) -> Optional[int]:
-        num_heads = group.get("num_heads")
-        if num_heads is None:
+        heads = group.get("num_heads")
+        if heads is None:
             return None
-        if isinstance(num_heads, bool) or not isinstance(num_heads, int) or num_heads < 1:
-            raise ValueError(f"num_heads must be a positive integer if set, got {num_heads!r}.")
-        if num_heads == 1:
-            return None
+        if not self._positive_int(heads):
+            raise ValueError(f"num_heads: expected a positive integer or None, got {heads!r}")
+        if heads == 1:
+            return None  # one head is the whole matrix
         if group.get("flatten"):
-            raise ValueError(
-                "num_heads > 1 is incompatible with flatten=True: flattening the per-head 3D view "
-                "collapses heads back into a single 2D matrix, defeating per-head Newton-Schulz."
-            )
-        return num_heads
+            raise ValueError("num_heads > 1 cannot be combined with flatten=True (flattening would merge the heads "
+                             "back into one matrix)")
+        return heads
 
     def _resolve_split_sizes(self, group: dict) -> Optional[Tuple[int, ...]]:
-        split_sizes = group.get("split_sizes")
-        if split_sizes is None:
+        blocks = group.get("split_sizes")
+        if blocks is None:
             return None
-        if not isinstance(split_sizes, (tuple, list)) or len(split_sizes) < 2:
-            raise ValueError(
-                f"split_sizes must be a tuple or list of at least 2 block sizes, got {split_sizes!r}."
-            )
-        if any(isinstance(s, bool) or not isinstance(s, int) or s < 1 for s in split_sizes):
-            raise ValueError(f"split_sizes entries must be positive integers, got {split_sizes!r}.")
+        if not isinstance(blocks, (tuple, list)) or len(blocks) < 2 or not all(self._positive_int(b) for b in blocks):
+            raise ValueError(f"split_sizes: expected a tuple or list of two or more positive integers, got {blocks!r}")
         if self._resolve_num_heads(group) is not None:
-            raise ValueError(
-                "split_sizes is incompatible with num_heads > 1: use num_heads for uniform per-head "
-                "splits or split_sizes for uneven row blocks, not both."
-            )
+            raise ValueError("split_sizes and num_heads > 1 are two ways of cutting the same rows: give one of them")
         if group.get("flatten"):
-            raise ValueError(
-                "split_sizes is incompatible with flatten=True: split_sizes applies to 2D parameters only."
-            )
-        return tuple(split_sizes)
+            raise ValueError("split_sizes cannot be combined with flatten=True (it applies to 2D parameters)")
+        return tuple(blocks)
 
     @staticmethod
     def _validate_split_shape(split_sizes: Tuple[int, ...], shape) -> None:
         if len(shape) != 2:
-            raise ValueError(f"split_sizes is only supported for 2D parameters, got shape {tuple(shape)}.")
+            raise ValueError(f"split_sizes needs a 2D parameter, got shape {tuple(shape)}")
         if sum(split_sizes) != shape[0]:
-            raise ValueError(
-                f"split_sizes {split_sizes} must sum to dim 0 of the parameter (got shape {tuple(shape)})."
-            )
+            raise ValueError(f"split_sizes {split_sizes} add up to {sum(split_sizes)}, not to the {shape[0]} rows of a "
+                             f"parameter of shape {tuple(shape)}")
 
     @staticmethod
     def _head_geometry(num_heads: int, shape) -> Tuple[int, int, int]:
         """(mats, rows, cols) of the per-head view of a 2D weight (dion/megabatch_base.py:304-364)."""
         if len(shape) != 2:
-            raise ValueError(f"num_heads is only supported for 2D parameters, got shape {tuple(shape)}.")
-        if shape[0] % num_heads != 0:
-            raise ValueError(
-                f"num_heads ({num_heads}) must divide dim 0 of the parameter (got shape {tuple(shape)})."
-            )
+            raise ValueError(f"num_heads needs a 2D parameter, got shape {tuple(shape)}")
+        if shape[0] % num_heads:
+            raise ValueError(f"num_heads={num_heads} does not divide the {shape[0]} rows of a parameter of shape "
+                             f"{tuple(shape)}")
         return num_heads, shape[0] // num_heads, shape[1]
 
     # ------------------------------------------------------------------ step
@@ -245,7 +242,7 @@ class OrthoOptimizer(Optimizer):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
-        self._sync_hyperparam_tensors()
+        self.bind_live_scalars()
 
         ortho, lion, adamw = [], [], []
         for group in self.param_groups:

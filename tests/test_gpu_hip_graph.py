@@ -68,11 +68,11 @@ def test_replay_matches_eager_bit_for_bit(cls_name, kwargs):
         s_e.step()
         s_g.step()
         o_g.zero_grad(set_to_none=False)
-    assert o_g._graph is not None
+    assert o_g.captured
     assert [g["step"] for g in inner.param_groups] == [g["step"] for g in o_e.param_groups]
     assert float(inner.state[p_g[-2]]["step_dev"]) == 8.0
     o_g.release()
-    assert o_g._graph is None
+    assert not o_g.captured
 
 
 def test_float_lr_assignment_reaches_the_graph_and_late_live_wd_is_refused():
@@ -97,7 +97,7 @@ def test_float_lr_assignment_reaches_the_graph_and_late_live_wd_is_refused():
         for a, b in zip(p_e, p_g):
             assert torch.equal(a.data, b.data), step
     inner.param_groups[0]["weight_decay"] = torch.tensor(0.5, device=DEV)
-    with pytest.raises(RuntimeError, match="after the graph was captured"):
+    with pytest.raises(RuntimeError, match="did not exist when the step was recorded"):
         o_g.step()
 
 
@@ -109,8 +109,35 @@ def test_capture_refuses_params_without_grad():
     for p in params[:-1]:
         p.grad = torch.randn_like(p)
     opt.step()  # warm-up step is eager and simply skips the param without a gradient
-    with pytest.raises(RuntimeError, match="grad=None at graph capture"):
+    with pytest.raises(RuntimeError, match="have no gradient yet"):
         opt.step()
+
+
+def test_replay_refuses_a_gradient_buffer_that_moved():
+    """The recorded kernels address .grad by raw pointer: a gradient that was re-created elsewhere would
+    be ignored silently, so the wrapper refuses to replay; after release() it records again."""
+    from dion.cuda_graph import CudaGraphOptimizer
+
+    params, inner = _build("Muon", {}, 14)
+    wrap = CudaGraphOptimizer(inner, warmup_steps=1)
+    for p in params:
+        p.grad = torch.randn_like(p)
+    wrap.step()
+    wrap.step()
+    assert wrap.captured
+    wrap.step()  # a plain replay is fine
+    keep = params[0].grad
+    params[0].grad = torch.randn_like(params[0])  # a new buffer, as zero_grad(set_to_none=True) + backward leaves
+    assert params[0].grad.data_ptr() != keep.data_ptr()
+    before = [p.data.clone() for p in params]
+    with pytest.raises(RuntimeError, match="no longer the tensor it was recorded with"):
+        wrap.step()
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, p.data) for a, p in zip(before, params)), "a refused replay must not run"
+    wrap.release()
+    wrap.step()
+    wrap.step()
+    assert wrap.captured
 
 
 def _zero_grads(params):
@@ -132,23 +159,23 @@ def test_frozen_parameter_is_allowed_and_release_rewarms():
     params[0].grad = None
     params[0].requires_grad_(False)
     wrap.step()
-    assert wrap._graph is not None
+    assert wrap.captured
     wrap.release()
-    assert wrap._graph is None and wrap._step_count == 0
+    assert not wrap.captured and wrap.eager_steps_done == 0
     wrap.release()
     wrap.step()
-    assert wrap._graph is None
+    assert not wrap.captured
     wrap.step()
-    assert wrap._graph is not None
+    assert wrap.captured
 
     params, inner = _build("Dion2", dict(fraction=0.25), 8)
     wrap = CudaGraphOptimizer(inner, warmup_steps=3)
     _zero_grads(params)
     wrap.step()
     wrap.step()
-    assert wrap._graph is None and wrap._step_count == 2
+    assert not wrap.captured and wrap.eager_steps_done == 2
     wrap.release()
-    assert wrap._step_count == 0
+    assert wrap.eager_steps_done == 0
 
 
 def test_failed_capture_leaves_no_graph_and_lr_sync_under_capture_is_an_error():
@@ -166,11 +193,11 @@ def test_failed_capture_leaves_no_graph_and_lr_sync_under_capture_is_an_error():
     inner.step = boom
     with pytest.raises(RuntimeError, match="capture blew up"):
         wrap.step()
-    assert wrap._graph is None
+    assert not wrap.captured
     inner.step = real_step
     torch.cuda.synchronize()
     wrap.step()  # captures now
-    assert wrap._graph is not None
+    assert wrap.captured
 
     # writing the lr tensor inside a capture would bake the capture-time value into every replay
     params, opt = _build("Dion2", dict(fraction=0.25), 9)
@@ -183,7 +210,7 @@ def test_failed_capture_leaves_no_graph_and_lr_sync_under_capture_is_an_error():
         for g in opt.param_groups:
             g["lr"] = 0.5
         with pytest.raises(RuntimeError, match="capture"):
-            opt._sync_hyperparam_tensors()
+            opt.bind_live_scalars()
     del graph
     torch.cuda.synchronize()
 
@@ -237,7 +264,7 @@ def test_scheduled_lr_tracks_after_resume_and_closure(cls_name, kwargs):
         assert o_g.step(lambda: torch.tensor(3.0)) == 3.0
         for a, b in zip(p_e, p_g):
             assert torch.equal(a.data, b.data), (cls_name, step)
-    assert o_g._graph is not None
+    assert o_g.captured
 
 
 def test_add_param_group_rewarms_before_recapturing():
@@ -248,14 +275,14 @@ def test_add_param_group_rewarms_before_recapturing():
     _zero_grads(params)
     for _ in range(3):
         wrap.step()
-    assert wrap._graph is not None
+    assert wrap.captured
     extra = torch.nn.Parameter(torch.randn(128, 256, device=DEV) * 0.02)
     extra.grad = torch.zeros_like(extra)
     wrap.add_param_group(dict(params=[extra]))
-    assert wrap._graph is None and wrap._step_count == 0
+    assert not wrap.captured and wrap.eager_steps_done == 0
     wrap.step()
     wrap.step()
-    assert wrap._graph is None       # two eager steps for the new group first
+    assert not wrap.captured       # two eager steps for the new group first
     wrap.step()
-    assert wrap._graph is not None
+    assert wrap.captured
     assert isinstance(inner.param_groups[-1]["lr"], torch.Tensor)

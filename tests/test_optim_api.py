@@ -64,7 +64,7 @@ def test_lr_is_a_persistent_tensor_and_state_dict_is_portable():
     assert sd["param_groups"][0]["lr"] == pytest.approx(0.02)
     # a float assigned by a hand-rolled schedule is copied into the same tensor on sync
     opt.param_groups[0]["lr"] = 0.05
-    opt._sync_hyperparam_tensors()
+    opt.bind_live_scalars()
     assert opt.param_groups[0]["lr"] is lr and float(lr) == pytest.approx(0.05)
     opt2 = Muon(_params([(16, 32)]), lr=0.5)
     opt2.load_state_dict(sd)
@@ -196,11 +196,11 @@ def test_graph_wrapper_host_contract():
         opt.zero_grad(set_to_none=True)
     assert p[0].grad is not None and float(p[0].grad.abs().sum()) == 0.0
     opt.add_param_group({"params": _params([(8, 8)])})
-    assert len(inner.param_groups) == 2 and opt._step_count == 0
+    assert len(inner.param_groups) == 2 and opt.eager_steps_done == 0 and not opt.captured
     opt.load_state_dict(inner.state_dict())
-    assert inner._hyperparam_tensors is inner._hyper_tensors
+    assert [t.data_ptr() for t in inner.live_scalar_tensors()] == [g["lr"].data_ptr() for g in inner.param_groups]
     steps = [g["step"] for g in inner.param_groups]
-    inner._advance_host_step_counters()
+    inner.count_skipped_host_step()
     assert [g["step"] for g in inner.param_groups] == [s + 1 for s in steps]
 
 
