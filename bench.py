@@ -120,6 +120,8 @@ def main() -> int:
                     help="also time momentum / orthogonalization / update of every shape group on its own "
                          "(adds a 'groups' list to the JSON line)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-variants", action="store_true",
+                    help="skip timing the step with the Polar-Express and Gram schedules (default Muon run only)")
     ap.add_argument("--no-kernel-timing", action="store_true")
     args = ap.parse_args()
 
@@ -206,6 +208,28 @@ def main() -> int:
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     value = total_flops / (ms_per_step * 1e-3) * 1e-12
 
+    # ---- the other orthogonalization schedules of the same step (default Muon run only): one warm
+    # step and three timed ones each, on the same parameters
+    variants = None
+    if args.optimizer == "muon" and args.ns == "ns5" and not args.graph and not args.two_call_update \
+            and not args.no_variants:
+        variants = {}
+        for vname, vkw in (("polar_express", dict(use_polar_express=True)),
+                           ("gram", dict(use_polar_express=True, use_gram_newton_schulz=True))):
+            fresh = [{k: g[k] for k in ("params", "num_heads") if k in g} for g in groups]
+            vopt = Muon(fresh, lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, adjust_lr="spectral_norm", **vkw)
+            vopt.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                vopt.step()
+            torch.cuda.synchronize()
+            vms = (time.perf_counter() - t0) * 1e3 / 3
+            variants[vname] = {"ms_per_step": round(vms, 3),
+                               "tflops": round(total_flops / (vms * 1e-3) * 1e-12, 2),
+                               "pct_of_bf16_peak": round(100.0 * total_flops / (vms * 1e-3) * 1e-12 / PEAK_BF16_TFLOPS, 2)}
+            del vopt
+
     result = {
         "metric": "Newton-Schulz TFLOP/s (% bf16 MFMA peak) + full optimizer-step ms, 1 GPU",
         "value": round(value, 2),
@@ -235,6 +259,9 @@ def main() -> int:
         },
         "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
     }
+    if variants is not None:
+        # same step, same FLOP convention (the standard iteration's count), other schedules
+        result["variants"] = variants
 
     # ---- free the model, then time kernels of the headline shape group on their own
     del opt
@@ -271,10 +298,31 @@ def main() -> int:
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) / iters
 
+        # The three GEMMs of one iteration on the headline group, each timed on its own with events on
+        # the launch stream.  "executed" counts the MFMA work actually issued (upper-triangle tiles only
+        # for the two symmetric products), "algorithmic" the full product.
+        A = torch.empty(B, m, m, device=dev, dtype=torch.bfloat16)
+        tile = 256 if (m % 256 == 0 and n % 256 == 0) else 128
+        T = m // tile
+        tri = (T + 1) / (2.0 * T)
+        ms1 = time_kernel(lambda: lib.dion_ns_line_1(X.data_ptr(), A.data_ptr(), B, m, n, st))
+        ms2 = time_kernel(lambda: lib.dion_ns_line_2(Bm.data_ptr(), A.data_ptr(), B, m, 1.0, 1.0, st))
         # dominant kernel: X' = B X with a*I folded into B, reading X as it lies; one launch per NS
         # iteration
-        ms3 = time_kernel(lambda: lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), None, C.data_ptr(), None,
-                                                     B, m, n, 0.0, st))
+        ms3 = time_kernel(lambda: lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), C.data_ptr(), B, m, n, 0.0, st))
+        del A
+
+        def gemm_row(ms, flop_full, executed_share):
+            ex = flop_full * executed_share / (ms * 1e-3) * 1e-12
+            return {"ms": round(ms, 4), "tflops_executed": round(ex, 1),
+                    "frac_executed": round(ex / PEAK_BF16_TFLOPS, 4),
+                    "tflops_algorithmic": round(flop_full / (ms * 1e-3) * 1e-12, 1)}
+
+        result["gemms"] = {
+            "A = X X^T": gemm_row(ms1, 2.0 * B * m * m * n, tri),
+            "B = c A A + b A + a I": gemm_row(ms2, 2.0 * B * m * m * m, tri),
+            "X' = B X": gemm_row(ms3, 2.0 * B * m * m * n, 1.0),
+        }
         flop3 = 2.0 * B * m * m * n
         achieved = flop3 / (ms3 * 1e-3) * 1e-12
         result["roofline"] = {
