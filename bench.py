@@ -310,6 +310,16 @@ def main() -> int:
         # dominant kernel: X' = B X with a*I folded into B, reading X as it lies; one launch per NS
         # iteration
         ms3 = time_kernel(lambda: lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), C.data_ptr(), B, m, n, 0.0, st))
+        # the vendor library's bf16 GEMM (hipBLASLt behind torch.bmm) on the same operands, same box, same
+        # run: the full product X X^T ("NT": both operands contiguous along the reduction index) and
+        # B X ("NN": X read as it lies, the form of the dominant launch)
+        ms_v_nt = time_kernel(lambda: torch.bmm(X, X.mT, out=A))
+        ms_v_nn = time_kernel(lambda: torch.bmm(Bm, X, out=C))
+        result["vendor_bf16_gemm"] = {
+            "X X^T, full product": {"ms": round(ms_v_nt, 4),
+                                    "tflops": round(2.0 * B * m * m * n / (ms_v_nt * 1e-3) * 1e-12, 1)},
+            "B X": {"ms": round(ms_v_nn, 4), "tflops": round(2.0 * B * m * m * n / (ms_v_nn * 1e-3) * 1e-12, 1)},
+        }
         del A
 
         def gemm_row(ms, flop_full, executed_share):
