@@ -119,6 +119,9 @@ def main() -> int:
     ap.add_argument("--breakdown", action="store_true",
                     help="also time momentum / orthogonalization / update of every shape group on its own "
                          "(adds a 'groups' list to the JSON line)")
+    ap.add_argument("--stream-compare", action="store_true",
+                    help="time muon_pre / muon_post on the headline group next to a plain device copy that moves the "
+                         "same number of bytes (adds a 'streaming' object to the JSON line)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-variants", action="store_true",
                     help="skip timing the step with the Polar-Express and Gram schedules (default Muon run only)")
@@ -363,6 +366,56 @@ def main() -> int:
             "pct_of_bf16_peak": round(100.0 * ns_tf / PEAK_BF16_TFLOPS, 2),
         }
         del X
+        torch.cuda.empty_cache()
+
+    if args.stream_compare:
+        # memory-bound kernels of the step against a plain copy with the same read and write volume, same
+        # run: muon_pre reads 6 B and writes 6 B per element (G bf16 + M fp32 -> M fp32 + U bf16), muon_post
+        # reads 6 B and writes 4 B (U bf16 + X fp32 -> X fp32)
+        name, rows, cols, count = max(spec, key=lambda g: g[1] * g[2] * g[3])
+        count = min(count, 16)
+        Gs = [torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen).to(torch.bfloat16)
+              for _ in range(count)]
+        Ms = [torch.zeros(rows, cols, device=dev) for _ in range(count)]
+        Xs = [torch.empty(rows, cols, device=dev).normal_(0.0, 0.02, generator=gen) for _ in range(count)]
+        n_el = count * rows * cols
+        lr_t = torch.tensor(0.02, device=dev)
+
+        def ev(f, iters=10):
+            f()
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                f()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / iters
+
+        ms_pre = ev(lambda: ops.muon_pre(Gs, Ms, 0.95, True))
+        U = ops.muon_pre(Gs, Ms, 0.95, True)
+        ms_post = ev(lambda: ops.muon_post(Xs, U.view(count, -1), lr_t, 0.5, 0.01))
+        src = torch.empty(n_el * 6, dtype=torch.uint8, device=dev).view(torch.float32)
+        dst = torch.empty_like(src)
+        ms_copy = ev(lambda: dst.copy_(src))                 # device-to-device memcpy (no kernel in a trace)
+        ms_mul = ev(lambda: torch.mul(src, 1.0, out=dst))    # the plainest streaming kernel: one read, one write
+        src2 = torch.empty_like(src)
+        ms_add = ev(lambda: torch.add(src, src2, out=dst))   # two read streams, one write stream
+
+        def row(ms, nbytes):
+            return {"ms": round(ms, 4), "GBps": round(nbytes / (ms * 1e-3) * 1e-9, 1),
+                    "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / (PEAK_HBM_GBS * 1e9), 4)}
+
+        result["streaming"] = {
+            "group": f"{count}x({rows}x{cols}) {name}",
+            "muon_pre (12 B/element)": row(ms_pre, n_el * 12),
+            "muon_post (10 B/element)": row(ms_post, n_el * 10),
+            "device memcpy, 6 B read + 6 B written per element": row(ms_copy, n_el * 12),
+            "torch.mul(src, 1, out=dst) fp32, 6 B read + 6 B written per element": row(ms_mul, n_el * 12),
+            "torch.add(src, src2, out=dst) fp32, 12 B read + 6 B written per element": row(ms_add, n_el * 18),
+        }
+        del Gs, Ms, Xs, U, src, src2, dst
         torch.cuda.empty_cache()
 
     if args.breakdown:

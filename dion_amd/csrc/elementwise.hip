@@ -258,9 +258,11 @@ __global__ __launch_bounds__(256) void muon_pre_kernel(PtrTab G, PtrTab M, bf16_
   if (VEC) {
     // Two 8-element chunks per thread per trip, all loads issued before the arithmetic: up to 96
     // bytes of reads in flight per lane.
+    // A workgroup owns contiguous tiles of 512 chunks (4096 elements), one tile per trip and normally
+    // one trip: the workgroups in flight sweep one window of memory front to back.
     const int64_t nv = numel >> 3;
-    for (int64_t i0 = (int64_t)blockIdx.x * 256 + threadIdx.x; i0 < nv; i0 += 2 * stride) {
-      const int64_t i1 = i0 + stride;
+    for (int64_t i0 = (int64_t)blockIdx.x * 512 + threadIdx.x; i0 < nv; i0 += 2 * stride) {
+      const int64_t i1 = i0 + 256;
       const bool has1 = i1 < nv;
       float gv[2][8], mv[2][8];
       st_load8<GT>(g, i0, gv[0]);
@@ -291,6 +293,14 @@ __global__ __launch_bounds__(256) void muon_pre_kernel(PtrTab G, PtrTab M, bf16_
   }
 }
 
+// Workgroups for the tile-per-workgroup kernels: one per 512 chunks, at most 2^20.
+static int ew_tiles(int64_t chunks) {
+  int64_t b = (chunks + 511) / 512;
+  if (b > (1 << 20)) b = 1 << 20;
+  if (b < 1) b = 1;
+  return (int)b;
+}
+
 static int ew_blocks(int64_t work_items) {
   int64_t b = (work_items + 255) / 256;
   if (b > 2048) b = 2048;
@@ -300,7 +310,7 @@ static int ew_blocks(int64_t work_items) {
 
 hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, bf16_t* U, int n,
                            int64_t numel, float mu, int nesterov, bool vec, hipStream_t st) {
-  dim3 grid(ew_blocks(vec ? (numel >> 3) : numel), n);
+  dim3 grid(vec ? ew_tiles(numel >> 3) : ew_blocks(numel), n);
 #define PRE_LAUNCH(GT, MT, V) \
   hipLaunchKernelGGL((muon_pre_kernel<GT, MT, V>), grid, dim3(256), 0, st, G, M, U, numel, mu, nesterov)
 #define PRE_LAUNCH_M(GT, V) \
@@ -339,19 +349,29 @@ __global__ __launch_bounds__(256) void muon_post_kernel(PtrTab X, const UT* __re
   const float* rs = row_scale ? row_scale + (int64_t)p * rows : nullptr;
   const int64_t stride = (int64_t)gridDim.x * 256;
   if (VEC) {
+    // contiguous tiles of 512 chunks (4096 elements) per workgroup, two chunks per lane, all loads first
     const int64_t nv = numel >> 3;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nv; i += stride) {
-      float uv[8], xv[8];
-      st_load8<UT>(u, i, uv);
-      if (rs) {  // cols % 8 == 0 on this path, so the 8 elements share a row
-        const float s = rs[(i << 3) / cols];
+    for (int64_t i0 = (int64_t)blockIdx.x * 512 + threadIdx.x; i0 < nv; i0 += 2 * stride) {
+      const int64_t i1 = i0 + 256;
+      const bool has1 = i1 < nv;
+      float uv[2][8], xv[2][8];
+      st_load8<UT>(u, i0, uv[0]);
+      if (has1) st_load8<UT>(u, i1, uv[1]);
+      st_load8<XT>(x, i0, xv[0]);
+      if (has1) st_load8<XT>(x, i1, xv[1]);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) uv[e] = __fmul_rn(uv[e], s);
+      for (int c = 0; c < 2; ++c) {
+        if (c == 1 && !has1) break;
+        const int64_t i = c == 0 ? i0 : i1;
+        if (rs) {  // cols % 8 == 0 on this path, so the 8 elements share a row
+          const float s = rs[(i << 3) / cols];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) uv[c][e] = __fmul_rn(uv[c][e], s);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xv[c][e] = muon_post_one(xv[c][e], uv[c][e], a, coeff, b, cautious);
+        st_store8<XT>(x, i, xv[c]);
       }
-      st_load8<XT>(x, i, xv);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) xv[e] = muon_post_one(xv[e], uv[e], a, coeff, b, cautious);
-      st_store8<XT>(x, i, xv);
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
@@ -366,7 +386,7 @@ hipError_t launch_muon_post(const PtrTab& X, int x_dtype, const void* U, int u_d
                             int cols, const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
                             float adj_ratio, const float* wd_dev, float wd_host, int cautious, bool vec,
                             hipStream_t st) {
-  dim3 grid(ew_blocks(vec ? (numel >> 3) : numel), n);
+  dim3 grid(vec ? ew_tiles(numel >> 3) : ew_blocks(numel), n);
 #define POST_LAUNCH(UT, XT, V)                                                                      \
   hipLaunchKernelGGL((muon_post_kernel<UT, XT, V>), grid, dim3(256), 0, st, X, (const UT*)U, numel, \
                      cols, row_scale, lr_dev, adj_lr_dev, adj_ratio, wd_dev, wd_host, cautious)
