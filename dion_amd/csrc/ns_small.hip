@@ -15,7 +15,8 @@
 namespace dion {
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
-constexpr int kMaxChunks = 36;  // 16-byte chunks a thread may hold while loading (n_pad <= 1152)
+constexpr int kThreads = 512;    // eight wavefronts: two per SIMD, so LDS and MFMA latencies of one hide behind the other
+constexpr int kMaxChunks = 18;  // 16-byte chunks a thread may hold while loading (n_pad <= 1152)
 #define LDS3(p) ((__attribute__((address_space(3))) s16x4*)(p))
 
 static __device__ __forceinline__ bf16x8 join_tr(s16x4 lo, s16x4 hi) {
@@ -25,7 +26,7 @@ static __device__ __forceinline__ bf16x8 join_tr(s16x4 lo, s16x4 hi) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in, bf16_t* __restrict__ out,
+__global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict__ in, bf16_t* __restrict__ out,
                                                        int rows, int cols, int n_pad, NsCoeffs co,
                                                        float norm_scale, float eps) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -45,7 +46,7 @@ __global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in,
 
   // ---- load (raw bf16 values), zero padding, sum of squares, scale, store to LDS
   float ss = 0.f;
-  const bool vec = (cols % 8 == 0) && ((((uintptr_t)src) & 15) == 0) && n_pad * 8 <= kMaxChunks * 256;
+  const bool vec = (cols % 8 == 0) && ((((uintptr_t)src) & 15) == 0) && n_pad * 8 <= kMaxChunks * kThreads;
   if (vec) {
     // Each thread keeps its 16-byte chunks in registers between the reduction and the scaled
     // store, so the matrix is read from HBM once and LDS is written once.
@@ -54,7 +55,7 @@ __global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in,
     uint4 raw[kMaxChunks];
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
-      const int idx = tid + c * 256;
+      const int idx = tid + c * kThreads;
       raw[c] = make_uint4(0, 0, 0, 0);
       if (idx < nchunks) {
         const int r = idx / cpr, c0 = (idx - r * cpr) * 8;  // input row, first input column
@@ -86,11 +87,11 @@ __global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in,
     for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
     if (lane == 0) red[wave] = ss;
     __syncthreads();
-    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float total = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
     const float sc = 1.0f / (sqrtf(total) * norm_scale + eps);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
-      const int idx = tid + c * 256;
+      const int idx = tid + c * kThreads;
       if (idx < nchunks) {
         const int r = idx / cpr, c0 = (idx - r * cpr) * 8;
         const uint32_t w[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in,
       }
     }
   } else {
-    for (int idx = tid; idx < 64 * n_pad; idx += 256) {
+    for (int idx = tid; idx < 64 * n_pad; idx += kThreads) {
       const int i = idx / n_pad, j = idx - i * n_pad;  // X[i][j]
       float v = 0.f;
       if (i < m && j < n) {
@@ -129,9 +130,9 @@ __global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in,
     for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
     if (lane == 0) red[wave] = ss;
     __syncthreads();
-    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float total = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
     const float sc = 1.0f / (sqrtf(total) * norm_scale + eps);
-    for (int idx = tid; idx < 64 * n_pad; idx += 256) {
+    for (int idx = tid; idx < 64 * n_pad; idx += kThreads) {
       const int i = idx / n_pad, j = idx - i * n_pad;
       bf16_t* p = (bf16_t*)(Xs + i * xp + j * 2);
       *p = f32_to_bf16(bf16_to_f32(*p) * sc);
@@ -140,53 +141,71 @@ __global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in,
   __syncthreads();
 
   const int frow = lane & 31, fhalf = lane >> 5;
-  const int ti = wave >> 1, tj = wave & 1;  // this wavefront's 32x32 tile of A / B
-  const int nslice = n_pad / 16;
+  // A and B (64 x 64) are computed as sixteen 16x16 tiles, two per wavefront (same 16 rows, two
+  // neighbouring 16-column blocks), with v_mfma_f32_16x16x32_bf16: lane l holds row / column l % 16
+  // and the eight k values 8 * (l / 16) .. + 7 of a 32-deep step; accumulator element r is row
+  // 4 * (l / 16) + r, column l % 16.
+  const int r16 = lane & 15, kq = lane >> 4;
+  const int ti = wave >> 1, tj0 = (wave & 1) * 2;
+  const int nstep = n_pad / 32;
 
   for (int it = 0; it < co.n; ++it) {
     const float a = co.c[it][0], b = co.c[it][1], c = co.c[it][2];
-    // ---- A = X X^T: one 32x32 tile per wavefront, two accumulators to break the MFMA chain
+    // ---- A = X X^T: even and odd k steps go to separate accumulators to break the MFMA chains
     {
-      f32x16 acc0, acc1;
+      f32x4 acc[2][2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc0[r] = acc1[r] = 0.f;
-      const char* pa = Xs + (ti * 32 + frow) * xp + fhalf * 16;
-      const char* pb = Xs + (tj * 32 + frow) * xp + fhalf * 16;
-      for (int s = 0; s < nslice; s += 2) {
-        const bf16x8 a0 = *(const bf16x8*)(pa + s * 32), b0 = *(const bf16x8*)(pb + s * 32);
-        const bf16x8 a1 = *(const bf16x8*)(pa + s * 32 + 32), b1 = *(const bf16x8*)(pb + s * 32 + 32);
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc1, 0, 0, 0);
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[h][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const char* pa = Xs + (ti * 16 + r16) * xp + kq * 16;
+      const char* pb0 = Xs + (tj0 * 16 + r16) * xp + kq * 16;
+      const char* pb1 = pb0 + 16 * xp;
+#pragma unroll 2
+      for (int s = 0; s < nstep; s += 2) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const bf16x8 fa = *(const bf16x8*)(pa + (s + h) * 64);
+          const bf16x8 f0 = *(const bf16x8*)(pb0 + (s + h) * 64);
+          const bf16x8 f1 = *(const bf16x8*)(pb1 + (s + h) * 64);
+          acc[h][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, f0, acc[h][0], 0, 0, 0);
+          acc[h][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, f1, acc[h][1], 0, 0, 0);
+        }
       }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = ti * 32 + (r >> 2) * 8 + 4 * fhalf + (r & 3);
-        *(bf16_t*)(As + row * ap + (tj * 32 + frow) * 2) = f32_to_bf16(acc0[r] + acc1[r]);
-      }
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = ti * 16 + kq * 4 + r;
+          *(bf16_t*)(As + row * ap + ((tj0 + j) * 16 + r16) * 2) = f32_to_bf16(acc[0][j][r] + acc[1][j][r]);
+        }
     }
     __syncthreads();
     // ---- B = c A A + b A + a I  (A symmetric: rows of A serve both operands)
     {
-      f32x16 acc;
+      f32x4 acc[2];
+      acc[0] = acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const bf16x8 fa = *(const bf16x8*)(As + (ti * 32 + frow) * ap + s * 32 + fhalf * 16);
-        const bf16x8 fb = *(const bf16x8*)(As + (tj * 32 + frow) * ap + s * 32 + fhalf * 16);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+      for (int s = 0; s < 2; ++s) {
+        const bf16x8 fa = *(const bf16x8*)(As + (ti * 16 + r16) * ap + s * 64 + kq * 16);
+        const bf16x8 f0 = *(const bf16x8*)(As + (tj0 * 16 + r16) * ap + s * 64 + kq * 16);
+        const bf16x8 f1 = *(const bf16x8*)(As + ((tj0 + 1) * 16 + r16) * ap + s * 64 + kq * 16);
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, f0, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, f1, acc[1], 0, 0, 0);
       }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = ti * 32 + (r >> 2) * 8 + 4 * fhalf + (r & 3);
-        const int col = tj * 32 + frow;
-        float v = c * acc[r] + b * bf16_to_f32(*(const bf16_t*)(As + row * ap + col * 2));
-        if (row == col) v += a;
-        *(bf16_t*)(Bs + row * ap + col * 2) = f32_to_bf16(v);
-      }
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = ti * 16 + kq * 4 + r;
+          const int col = (tj0 + j) * 16 + r16;
+          float v = c * acc[j][r] + b * bf16_to_f32(*(const bf16_t*)(As + row * ap + col * 2));
+          if (row == col) v += a;
+          *(bf16_t*)(Bs + row * ap + col * 2) = f32_to_bf16(v);
+        }
     }
     __syncthreads();
-    // ---- X = B X: wavefront w owns column tiles w, w+4, ...; both row tiles per column tile, so
+    // ---- X = B X: wavefront w owns column tiles w, w+8, ...; both row tiles per column tile, so
     // the whole 64 x 32 column block is read before it is overwritten.
     {
       bf16x8 fB[2][4];
@@ -201,7 +220,10 @@ __global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in,
       const int trow = 8 * (g16 >> 1) + (t16 >> 2);
       const int tcol = (g16 & 1) * 16 + (t16 & 3) * 4;
       const bool last = (it == co.n - 1);
-      for (int jt = wave; jt < n_pad / 32; jt += 4) {
+      // The MFMA operands are swapped (X fragment first): the accumulators then hold (B X)^T tiles, i.e.
+      // lane l owns output row i*32 + l%32 and, per group of four accumulator elements, four consecutive
+      // output columns -- one 8-byte store per group instead of four 2-byte ones.
+      for (int jt = wave; jt < n_pad / 32; jt += 8) {
         f32x16 acc[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -213,36 +235,63 @@ __global__ __launch_bounds__(256) void ns_small_kernel(const T* __restrict__ in,
           const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS3(px + (s * 16) * xp));
           const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS3(px + (s * 16 + 4) * xp));
           const bf16x8 fx = join_tr(lo, hi);
-          acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fB[0][s], fx, acc[0], 0, 0, 0);
-          acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fB[1][s], fx, acc[1], 0, 0, 0);
+          acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fx, fB[0][s], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fx, fB[1][s], acc[1], 0, 0, 0);
         }
-        const int col = jt * 32 + frow;
+        const int col0 = jt * 32 + 4 * fhalf;  // + 8 * g: first of four consecutive columns
         if (!last) {
 #pragma unroll
           for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int row = i * 32 + (r >> 2) * 8 + 4 * fhalf + (r & 3);
-              *(bf16_t*)(Xs + row * xp + col * 2) = f32_to_bf16(acc[i][r]);
+            for (int g = 0; g < 4; ++g) {
+              uint2 o;
+              o.x = pack_bf16x2(acc[i][4 * g], acc[i][4 * g + 1]);
+              o.y = pack_bf16x2(acc[i][4 * g + 2], acc[i][4 * g + 3]);
+              *(uint2*)(Xs + (i * 32 + frow) * xp + (col0 + 8 * g) * 2) = o;
             }
-        } else if (col < n) {
+        } else if (!tall) {
+          const bool vec4 = (cols % 4 == 0) && ((((uintptr_t)dst) & 7) == 0);
 #pragma unroll
-          for (int i = 0; i < 2; ++i)
+          for (int i = 0; i < 2; ++i) {
+            const int row = i * 32 + frow;
+            if (row >= m) continue;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int row = i * 32 + (r >> 2) * 8 + 4 * fhalf + (r & 3);
-              if (row < m) {
-                const int64_t g = tall ? (int64_t)col * cols + row : (int64_t)row * cols + col;
-                dst[g] = f32_to_bf16(acc[i][r]);
+            for (int g = 0; g < 4; ++g) {
+              const int col = col0 + 8 * g;
+              bf16_t* q = dst + row * cols + col;
+              if (vec4 && col + 3 < n) {
+                uint2 o;
+                o.x = pack_bf16x2(acc[i][4 * g], acc[i][4 * g + 1]);
+                o.y = pack_bf16x2(acc[i][4 * g + 2], acc[i][4 * g + 3]);
+                *(uint2*)q = o;
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  if (col + e < n) q[e] = f32_to_bf16(acc[i][4 * g + e]);
               }
             }
+          }
+        } else {
+          // tall input: X holds the transpose, output element (col, row); lanes run along `row`
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const int row = i * 32 + frow;
+            if (row >= m) continue;
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int col = col0 + 8 * g + e;
+                if (col < n) dst[col * cols + row] = f32_to_bf16(acc[i][4 * g + e]);
+              }
+          }
         }
       }
     }
     __syncthreads();
   }
   if (co.n == 0) {  // normalisation only
-    for (int idx = tid; idx < m * n; idx += 256) {
+    for (int idx = tid; idx < m * n; idx += kThreads) {
       const int i = idx / n, j = idx - i * n;
       const int64_t g = tall ? (int64_t)j * cols + i : (int64_t)i * cols + j;
       dst[g] = *(const bf16_t*)(Xs + i * xp + j * 2);
@@ -269,10 +318,10 @@ hipError_t launch_ns_small(const void* in, int in_dtype, bf16_t* out, int batch,
   if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<float>, 150 * 1024, done_f32))
     return e;
   if (in_dtype == 0)
-    hipLaunchKernelGGL(ns_small_kernel<bf16_t>, dim3(batch), dim3(256), bytes, st, (const bf16_t*)in, out, rows,
+    hipLaunchKernelGGL(ns_small_kernel<bf16_t>, dim3(batch), dim3(kThreads), bytes, st, (const bf16_t*)in, out, rows,
                        cols, n_pad, co, norm_scale, eps);
   else
-    hipLaunchKernelGGL(ns_small_kernel<float>, dim3(batch), dim3(256), bytes, st, (const float*)in, out, rows,
+    hipLaunchKernelGGL(ns_small_kernel<float>, dim3(batch), dim3(kThreads), bytes, st, (const float*)in, out, rows,
                        cols, n_pad, co, norm_scale, eps);
   return hipGetLastError();
 }
