@@ -323,10 +323,15 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
   // Fragment reads of a slice go out in the order A0, B0..B(TN-1), A1..A(TM-1); LDS returns in order, so once
   // at most the TM-1 reads issued after the last B fragment are outstanding, every B fragment has arrived.
-  auto qk_wait = [&]() {
-    if (QK) __builtin_amdgcn_s_waitcnt(0xC07F | ((TM - 1) << 8));  // lgkmcnt(TM-1) only
-  };
+  // The wait is an asm statement that takes the fragments it guards as read-write operands: to the compiler
+  // they are (re)defined here, so no use of them can be scheduled ahead of the wait.
   bf16x8 fa[2][TM], fb[2][TN];
+  auto qk_wait = [&](int f) {
+    if constexpr (QK) {
+      static_assert(TN == 2, "operand list of the wait below");
+      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(fb[f][0]), "+v"(fb[f][1]) : "n"(TM - 1));
+    }
+  };
   // Fragment read r (0..NR-1) of slice kk of ring slot buf into fragment set f, in the order the
   // MFMAs (row-major over the TM x TN accumulators) first need them: A0, B0..B(TN-1), A1..A(TM-1).
   auto read_frag = [&](int buf, int kk, int f, int r) {
@@ -388,7 +393,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
         const bool last = (kk == KK - 1);
         // slab kt+1 landed, slab kt fully read
         if (last) pipeline_barrier<(NSTAGE - 2) * LPS>();
-        qk_wait();
+        qk_wait(cur);
 #pragma unroll
         for (int q = 0; q < NM; ++q) {
           acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(

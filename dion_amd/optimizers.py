@@ -127,7 +127,13 @@ class _MomentumOrtho(OrthoOptimizer):
 
 class Muon(_MomentumOrtho):
     """Muon on one MI355X.  Same arguments as the reference ``Muon`` (dion/muon.py:61-78);
-    ``distributed_mesh`` must be None and ``use_triton`` selects nothing."""
+    ``distributed_mesh`` must be None and ``use_triton`` selects nothing.
+
+    ``flatten=True`` updates every parameter with three or more dimensions as its own
+    ``[shape[0], prod(shape[1:])]`` matrix, as the reference documents it (dion/muon.py:42-44).  The
+    reference's batched code path flattens the stack of same-shape parameters instead
+    (dion/megabatch_base.py:903-904), which orthogonalizes one ``N x numel`` matrix across the N
+    parameters of a shape group; results for such groups therefore differ from the reference's."""
 
     def __init__(self, params, distributed_mesh=None, lr: float = 0.01, mu: float = 0.95,
                  betas: Tuple[float, float] = (0.9, 0.95), weight_decay: Union[float, Tensor] = 0.01,

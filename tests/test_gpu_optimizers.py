@@ -396,3 +396,40 @@ def test_nordion2_num_heads_matches_3d_param_and_alias():
         o3.step()
     assert torch.equal(p2.data.view(H, d, n_in), p3.data)
     assert torch.equal(o2.state[p2]["variance_neuron"].view(-1), o3.state[p3]["variance_neuron"].view(-1))
+
+
+def test_flatten_orthogonalizes_each_parameter_as_its_own_matrix():
+    """flatten=True on a group of N > 1 same-shape 3-D parameters (convolution-like [out, in, k]): every
+    parameter is updated as its own [out, in*k] matrix, with the lr adjustment of that matrix -- the documented
+    contract (dion/muon.py:42-44, adjust_lr with flatten at dion/megabatch_base.py:984-1002).  The reference's
+    stacked code path flattens the whole stack instead (X.flatten(start_dim=1) on [N, out, in, k],
+    dion/megabatch_base.py:903-904), which mixes the N parameters into one N x (out*in*k) matrix; this build does
+    not reproduce that.  Checked against the oracle applied to each parameter's 2-D view."""
+    from dion import Muon
+
+    torch.manual_seed(3)
+    n, shape = 3, (96, 32, 5)
+    X = [torch.randn(shape) * 0.02 for _ in range(n)]
+    G = [(torch.randn(shape) * 0.02).to(torch.bfloat16) for _ in range(n)]
+    params = [torch.nn.Parameter(x.clone().to(DEV)) for x in X]
+    for p, g in zip(params, G):
+        p.grad_dtype = None
+        p.grad = g.to(DEV)
+    opt = Muon(params, lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, flatten=True, use_polar_express=False)
+    opt.step()
+    flat = (shape[0], shape[1] * shape[2])
+    ratio = oracle.adjust_lr_ratio(shape, "spectral_norm", flatten=True)
+    assert ratio == pytest.approx((flat[0] / flat[1]) ** 0.5)
+    a = 1 - torch.tensor(0.02) * torch.tensor(0.01)
+    for i in range(n):
+        (xo,), (mo,), (uo,) = oracle.muon_step([X[i].view(flat)], [G[i].view(flat)], [torch.zeros(flat)], 0.02, 0.95,
+                                               0.01, True, None, ns="ns5", epsilon=1e-8, adj_ratio=ratio)
+        assert torch.equal(opt.state[params[i]]["momentum"].cpu().view(flat), mo)
+        u_gpu = (X[i].view(flat) * a - params[i].data.cpu().view(flat)) / (0.02 * ratio)
+        assert _rel(u_gpu, uo.float()) <= 2e-2
+    # and the parameters do not influence one another: a group of one gives the same bits
+    solo = torch.nn.Parameter(X[1].clone().to(DEV))
+    solo.grad_dtype = None
+    solo.grad = G[1].to(DEV)
+    Muon([solo], lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, flatten=True, use_polar_express=False).step()
+    assert torch.equal(solo.data, params[1].data)
