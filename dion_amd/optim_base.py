@@ -287,15 +287,14 @@ class OrthoOptimizer(Optimizer):
         for _ in self._shape_group_phases(group, params):
             pass
 
-    # Shape groups are independent.  A group whose GEMMs cannot fill the GPU on their own (a few
-    # hundred tiles) is run on one of a handful of side streams so that several such groups
-    # overlap; mid-sized groups (kernels of three or four rounds of workgroups) share two streams,
-    # which fills the partial last round of one group's kernels with the other's; large groups run
-    # one after another on the caller's stream, where a second stream only costs L2 locality.  The reference reaches
+    # Shape groups are independent.  Groups whose kernels are a few rounds of workgroups or less (GPT-small:
+    # a few hundred tiles per launch; GPT-1.3B: three or four rounds) alternate between two side streams, so that
+    # the partial last round of one group's kernels is filled by the other's; more streams than two measured
+    # slower (the launches then share L2 and the power budget three or four ways).  Large groups run one after
+    # another on the caller's stream, where a second stream only costs L2 locality.  The reference reaches
     # the same goal by interleaving up to three generator tasks (dion/megabatch_base.py:193).
-    _SMALL_GROUP_FLOP = 4e12    # below: launches of a few microseconds, four streams
-    _MEDIUM_GROUP_FLOP = 3e13   # below: kernels of a few rounds of workgroups, two streams fill the tails
-    _N_SIDE_STREAMS = 4
+    _MEDIUM_GROUP_FLOP = 3e13   # below: two streams fill the tails
+    _N_SIDE_STREAMS = 2
 
     @staticmethod
     def _group_flop(params: List[Tensor]) -> float:
@@ -332,8 +331,6 @@ class OrthoOptimizer(Optimizer):
             return
         device = small[0][1][0].device
         pool = self._side_pool(device)
-        if any(self._group_flop(w[1]) >= self._SMALL_GROUP_FLOP for w in small):
-            pool = pool[:2]
         main = torch.cuda.current_stream(device)
         fork = main.record_event()
         used = []
