@@ -687,11 +687,16 @@ int gemm_pad_granule(int m, int n, int batch) {
   return syrk_tiles >= 256 ? 256 : 128;
 }
 
-// 256-wide tiles only when there are enough of them (512) to keep 256 CUs busy for a few rounds; below
-// that the 128-wide tiles (two workgroups per CU) win.
+// 256-wide tiles when there are enough of them: a full product from 384 tiles (one and a half rounds of the
+// 256 CUs; 432 tiles of 12 x (768 x 3072) run 14 % faster than the 1728 128-wide ones, 108 tiles of
+// 12 x (768 x 768) 20 % slower), a symmetric one from 160 (16 x 1024-wide: 5 % faster; 72 tiles of
+// 12 x 768-wide: 70 % slower).  Rounds that are not full cost less than their geometry says: the part is
+// power-limited, and the CUs that are busy run faster while others idle.  Below the thresholds the 128-wide
+// tiles (two workgroups per CU) win.
 static bool wants_256_tiles(const GemmParams& p) {
-  const long t256 = (long)(p.M / 256) * (p.tri ? (p.M / 256 + 1) / 2 + 0 : p.N / 256) * p.batch;
-  return p.M % 256 == 0 && p.N % 256 == 0 && t256 >= 512L;
+  const long T = p.M / 256;
+  const long t256 = (p.tri ? T * (T + 1) / 2 : T * (p.N / 256)) * p.batch;
+  return p.M % 256 == 0 && p.N % 256 == 0 && t256 >= (p.tri ? 160L : 384L);
 }
 
 int gemm_tile_edge(const GemmParams& p) { return wants_256_tiles(p) ? 256 : 128; }
