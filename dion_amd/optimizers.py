@@ -301,7 +301,10 @@ class NorDion2(OrthoOptimizer):
     rows, so that a selected slice is a whole neuron); those rows of ``M`` decay by ``mu``; the
     selected block is orthogonalized; NorMuon's per-row second-moment normalisation runs on it
     against the selected entries of ``variance_neuron``; the scaled rows update ``X``.
-    ``assembled_selection`` as for ``Dion2``."""
+    ``assembled_selection`` as for ``Dion2``.  ``flatten=True`` on a parameter with three or more dimensions
+    orthogonalizes its selected block as one ``[shape[0], -1]`` matrix per parameter (the reference's batched
+    path flattens across the stack of same-shape parameters, dion/megabatch_base.py:903-904); selection and
+    the per-neuron normalisation are those of the unflattened layout."""
 
     assembled_selection = False
 
@@ -345,8 +348,6 @@ class NorDion2(OrthoOptimizer):
             raise NotImplementedError("split_sizes is currently supported only by Muon and NorMuon.")
         shape = params[0].shape
         flatten = group["flatten"]
-        if flatten and len(shape) >= 3:
-            raise NotImplementedError("NorDion2: flatten=True is built for 2D parameters only.")
         if num_heads is not None:
             mats, rows, cols = self._head_geometry(num_heads, shape)
             ratio_shape = (mats, rows, cols)
@@ -365,6 +366,9 @@ class NorDion2(OrthoOptimizer):
         V = [s["variance_neuron"].view(mats, rows, 1) for s in states]
 
         if self.assembled_selection and group["selection_scope"] == "global":
+            if flatten and len(shape) >= 3:
+                raise NotImplementedError("NorDion2: whole-matrix selection with flatten=True is built for "
+                                          "2D parameters only.")
             # accumulate -> select inside the orthogonalization call -> masked normalisation and update
             # (dion/nordion2.py:291-335)
             U_full = global_scope.dion2_pre_accumulate(G, M)
@@ -386,7 +390,12 @@ class NorDion2(OrthoOptimizer):
         U_sel, idx, imap = ops.dion2_select(G, M, k, select_dim, group["mu"])
         yield
         _note_stream(U_sel)
-        O = self._orthogonalize(U_sel.view(n * mats, k, cols), float(group["epsilon"]))
+        if flatten and len(shape) >= 3:
+            # leading dim stays, the selected rows of all the other dims form one long row (per parameter,
+            # as in Muon and Dion2 here; dion/megabatch_base.py:903-904 flattens the stack instead)
+            O = self._orthogonalize(U_sel.view(n, shape[0], -1), float(group["epsilon"]))
+        else:
+            O = self._orthogonalize(U_sel.view(n * mats, k, cols), float(group["epsilon"]))
         del U_sel
         yield
         _note_stream(O)
