@@ -17,6 +17,8 @@ namespace dion {
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 constexpr int kThreads = 512;    // eight wavefronts: two per SIMD, so LDS and MFMA latencies of one hide behind the other
 constexpr int kMaxChunks = 18;  // 16-byte chunks a thread may hold while loading (n_pad <= 1152)
+constexpr int kPartialBytes = 4 * 3 * 64 * 16;  // A = X X^T: f32x4 per lane, three tiles, four wavefront groups
+constexpr int kMaxLds = 160 * 1024 - 1024;      // dynamic LDS of one workgroup: the static part (reduction scratch) takes the first KB
 #define LDS3(p) ((__attribute__((address_space(3))) s16x4*)(p))
 
 static __device__ __forceinline__ bf16x8 join_tr(s16x4 lo, s16x4 hi) {
@@ -141,44 +143,77 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
   __syncthreads();
 
   const int frow = lane & 31, fhalf = lane >> 5;
-  // A and B (64 x 64) are computed as sixteen 16x16 tiles, two per wavefront (same 16 rows, two
-  // neighbouring 16-column blocks), with v_mfma_f32_16x16x32_bf16: lane l holds row / column l % 16
-  // and the eight k values 8 * (l / 16) .. + 7 of a 32-deep step; accumulator element r is row
+  // A and B (64 x 64) are computed as 16x16 tiles with v_mfma_f32_16x16x32_bf16: lane l holds row / column
+  // l % 16 and the eight k values 8 * (l / 16) .. + 7 of a 32-deep step; accumulator element r is row
   // 4 * (l / 16) + r, column l % 16.
   const int r16 = lane & 15, kq = lane >> 4;
-  const int ti = wave >> 1, tj0 = (wave & 1) * 2;
+  const int ti = wave >> 1, tj0 = (wave & 1) * 2;  // B = poly(A): two neighbouring tiles of one tile row
   const int nstep = n_pad / 32;
+  // A = X X^T is symmetric: ten of its sixteen tiles are computed, the others are their mirror images.
+  // Four groups of wavefronts take the tiles (row block, column block)
+  //   (0,0) (0,1) (0,2) | (3,3) (3,0) (3,1) | (1,1) (1,2) | (2,2) (2,3)
+  // -- always the group's first row block against itself and its one or two other row blocks, so a k step
+  // costs a group three (two) fragment reads for three (two) MFMAs, the same fragments serving as both
+  // operands -- and the two wavefronts of a group split the k steps, even and odd.  (One tile row per
+  // wavefront pair over the full k range, the previous form, read 2.4 times as many fragment bytes and
+  // computed all sixteen tiles; this phase was LDS-bound.)
+  const int ag = wave >> 1, akh = wave & 1;
+  const int rb0 = ag == 0 ? 0 : ag == 1 ? 3 : ag == 2 ? 1 : 2;
+  const int rb1 = ag == 0 ? 1 : ag == 1 ? 0 : ag == 2 ? 2 : 3;
+  const int rb2 = ag == 0 ? 2 : 1;
+  const bool three = ag < 2;
+  float* Ps = (float*)(Bs + 64 * ap);  // partial sums of the odd-k wavefronts: [group][tile][lane] f32x4
 
   for (int it = 0; it < co.n; ++it) {
     const float a = co.c[it][0], b = co.c[it][1], c = co.c[it][2];
-    // ---- A = X X^T: even and odd k steps go to separate accumulators to break the MFMA chains
+    // ---- A = X X^T
     {
-      f32x4 acc[2][2];
+      f32x4 acc[3];
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[h][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const char* pa = Xs + (ti * 16 + r16) * xp + kq * 16;
-      const char* pb0 = Xs + (tj0 * 16 + r16) * xp + kq * 16;
-      const char* pb1 = pb0 + 16 * xp;
+      for (int t = 0; t < 3; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const char* p0 = Xs + (rb0 * 16 + r16) * xp + kq * 16;
+      const char* p1 = Xs + (rb1 * 16 + r16) * xp + kq * 16;
+      const char* p2 = Xs + (rb2 * 16 + r16) * xp + kq * 16;
+      if (three) {
 #pragma unroll 2
-      for (int s = 0; s < nstep; s += 2) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const bf16x8 fa = *(const bf16x8*)(pa + (s + h) * 64);
-          const bf16x8 f0 = *(const bf16x8*)(pb0 + (s + h) * 64);
-          const bf16x8 f1 = *(const bf16x8*)(pb1 + (s + h) * 64);
-          acc[h][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, f0, acc[h][0], 0, 0, 0);
-          acc[h][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, f1, acc[h][1], 0, 0, 0);
+        for (int s = akh; s < nstep; s += 2) {
+          const bf16x8 f0 = *(const bf16x8*)(p0 + s * 64);
+          const bf16x8 f1 = *(const bf16x8*)(p1 + s * 64);
+          const bf16x8 f2 = *(const bf16x8*)(p2 + s * 64);
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f0, acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f1, acc[1], 0, 0, 0);
+          acc[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f2, acc[2], 0, 0, 0);
+        }
+      } else {
+#pragma unroll 2
+        for (int s = akh; s < nstep; s += 2) {
+          const bf16x8 f0 = *(const bf16x8*)(p0 + s * 64);
+          const bf16x8 f1 = *(const bf16x8*)(p1 + s * 64);
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f0, acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f1, acc[1], 0, 0, 0);
         }
       }
+      float* pp = Ps + ((ag * 3) * 64 + lane) * 4;
+      if (akh == 1) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+        for (int t = 0; t < 3; ++t) *(f32x4*)(pp + t * 256) = acc[t];
+      }
+      __syncthreads();
+      if (akh == 0) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int row = ti * 16 + kq * 4 + r;
-          *(bf16_t*)(As + row * ap + ((tj0 + j) * 16 + r16) * 2) = f32_to_bf16(acc[0][j][r] + acc[1][j][r]);
+        for (int t = 0; t < 3; ++t) {
+          if (t == 2 && !three) break;
+          const f32x4 o = *(const f32x4*)(pp + t * 256);
+          const int cb = t == 0 ? rb0 : t == 1 ? rb1 : rb2;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int row = rb0 * 16 + kq * 4 + r, col = cb * 16 + r16;
+            const bf16_t v = f32_to_bf16(acc[t][r] + o[r]);
+            *(bf16_t*)(As + row * ap + col * 2) = v;
+            if (t > 0) *(bf16_t*)(As + col * ap + row * 2) = v;
+          }
         }
+      }
     }
     __syncthreads();
     // ---- B = c A A + b A + a I  (A symmetric: rows of A serve both operands)
@@ -303,19 +338,19 @@ bool ns_small_fits(int rows, int cols) {
   const int m = rows < cols ? rows : cols, n = rows < cols ? cols : rows;
   if (m > 64) return false;
   const int n_pad = (n + 63) / 64 * 64;
-  const size_t bytes = (size_t)64 * (n_pad * 2 + 16) + 2 * 64 * (64 * 2 + 16);
-  return bytes <= 150 * 1024;
+  const size_t bytes = (size_t)64 * (n_pad * 2 + 16) + 2 * 64 * (64 * 2 + 16) + kPartialBytes;
+  return bytes <= kMaxLds;
 }
 
 hipError_t launch_ns_small(const void* in, int in_dtype, bf16_t* out, int batch, int rows, int cols,
                            const NsCoeffs& co, float norm_scale, float eps, hipStream_t st) {
   const int n = rows < cols ? cols : rows;
   const int n_pad = (n + 63) / 64 * 64;
-  const size_t bytes = (size_t)64 * (n_pad * 2 + 16) + 2 * 64 * (64 * 2 + 16);
+  const size_t bytes = (size_t)64 * (n_pad * 2 + 16) + 2 * 64 * (64 * 2 + 16) + kPartialBytes;
   static std::atomic<uint64_t> done_bf16{0}, done_f32{0};
-  if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<bf16_t>, 150 * 1024, done_bf16))
+  if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<bf16_t>, kMaxLds, done_bf16))
     return e;
-  if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<float>, 150 * 1024, done_f32))
+  if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<float>, kMaxLds, done_f32))
     return e;
   if (in_dtype == 0)
     hipLaunchKernelGGL(ns_small_kernel<bf16_t>, dim3(batch), dim3(kThreads), bytes, st, (const bf16_t*)in, out, rows,
