@@ -12,7 +12,7 @@ NS5.  The bars:
   * Polar-Express, KJ: no further from either reference path than REL x the distance between the
     reference's two paths on that input (REL = 1.25 towards the eager path, 1.0 towards the
     compiled one: the compiled path shares some roundings with the eager one, the HIP path none).
-The measured distances are printed (pytest -s) and recorded in DESIGN.md."""
+The measured distances are printed (pytest -s)."""
 import os
 
 import numpy as np
