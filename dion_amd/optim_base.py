@@ -303,12 +303,18 @@ class OrthoOptimizer(Optimizer):
         mats = len(params) * (params[0].numel() // (r * c))
         return mats * 5.0 * (4.0 * m * m * n + 2.0 * m ** 3)
 
+    # One pool per device for the whole process, shared by every optimizer instance: the runtime maps streams
+    # onto a handful of hardware queues in creation order, and two streams created by a later instance can
+    # land on one queue, where they run in sequence (measured: the step of a second optimizer in the same
+    # process at the sequential figure, 2.1 instead of 1.8 ms for GPT-small).
+    _side_pools: dict = {}
+
     def _side_pool(self, device) -> List["torch.cuda.Stream"]:
-        streams = self.__dict__.setdefault("_side_streams", {})
-        pool = streams.get(device)
+        key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+        pool = OrthoOptimizer._side_pools.get(key)
         if pool is None:
             pool = [torch.cuda.Stream(device=device) for _ in range(self._N_SIDE_STREAMS)]
-            streams[device] = pool
+            OrthoOptimizer._side_pools[key] = pool
         return pool
 
     def _run_shape_groups(self, work: List[Tuple[dict, List[Tensor]]]) -> None:
