@@ -637,8 +637,284 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 }
 
 // ---------------------------------------------------------------------------------------------
+// X' = P Q with Q stored [K][N] (the dominant launch of the iteration), one workgroup per CU walking a
+// list of output tiles.  What the one-tile-per-workgroup kernel above pays at every tile boundary --
+// the store acknowledgements a wavefront waits for before it may end, the dispatch of the next
+// workgroup, and the latency of its first operand loads, together 5-8 us per 256x256 tile with the
+// MFMA pipes idle -- is overlapped here:
+//   * the operand ring runs on across tiles: the refills issued during the last two slabs of a tile
+//     fetch the first two slabs of the workgroup's next tile, so the next tile's first MFMAs issue right
+//     after this tile's epilogue;
+//   * the epilogue goes through a private 4 KB LDS slice per wavefront next to the ring (not over
+//     it: the ring is already receiving the next tile) and leaves as sixteen 16-byte stores per
+//     lane, each instruction writing whole 128-byte lines.  Sixteen outstanding stores also stay countable
+//     next to the ring's loads (the wait counter has six bits), and their acknowledgements come back
+//     under the next tile's first slab.
+// OUT_T false stores C[row][col]: the MFMA operands are swapped, so that a lane's four consecutive
+// accumulator registers are four consecutive columns of one output row (8 bytes of a C row).
+// OUT_T true stores Ct[col][row] (the product of a tall input, kept in the wide layout): operands
+// in the usual order, four consecutive registers are four consecutive rows = 8 bytes of a Ct row.
+// Either way a staged chunk is 32 lines x 128 bytes from two 32x32 accumulator tiles.
+template <class Cfg, bool OUT_T>
+__global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams p, const int total_tiles) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, KK = Cfg::KK, NSTAGE = Cfg::NSTAGE;
+  constexpr int NM = TM * TN, NR = TM + TN, LPS = Cfg::LOADS_PER_STAGE;
+  constexpr int RPM = (NR + NM - 1) / NM, LPM = (LPS + NM - 1) / NM;
+  static_assert(NSTAGE == 2 && TM == 4 && TN == 2 && KK % 2 == 0, "written for 128x64 wavefront tiles, two-slot ring");
+  constexpr int STG_WAVE = 32 * 128;  // staging bytes per wavefront: 32 lines of 128 bytes
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int tilesM = p.M / BM, tilesN = p.N / BN;
+  const int tiles_per_mat = tilesM * tilesN;
+  const int KT = p.K / BK;
+
+  // Tile number `pid` of the launch -> (batch, tile row, tile column): the same map as the kernel above
+  // uses for its workgroup index, so consecutive workgroups (= XCDs) share operand panels the same way.
+  auto tile_of = [&](int pid, int& b, int& ti, int& tj) {
+    int lt;
+    if (p.xcd_interleave && pid < (total_tiles & ~255)) {
+      const int j = pid & 255;
+      lt = (pid & ~255) + (j & 7) * 32 + (j >> 3);
+    } else if (p.xcd_interleave) {
+      lt = pid;
+    } else {
+      const int xcd = pid & 7, loc = pid >> 3;
+      const int q = total_tiles >> 3, r = total_tiles & 7;
+      lt = xcd * q + (xcd < r ? xcd : r) + loc;
+    }
+    b = lt / tiles_per_mat;
+    const int t = lt - b * tiles_per_mat;
+    constexpr int GM = 8;
+    const int per_group = GM * tilesN;
+    const int g = t / per_group;
+    const int first = g * GM;
+    const int gsz = (tilesM - first) < GM ? (tilesM - first) : GM;
+    const int tg = t - g * per_group;
+    ti = first + tg % gsz;
+    tj = tg / gsz;
+  };
+
+  // ---- global -> LDS addressing (see the kernel above): per-lane offsets are the same for every tile,
+  // the tile only moves the wave-uniform base pointers.
+  const int ld_row = tid / Cfg::CPR;
+  const int ld_phys = tid % Cfg::CPR;
+  const int ld_chunk = ld_phys ^ ((ld_row / Cfg::SWZ_DIV) % Cfg::CPR);
+  constexpr int QCPR = BN / 8;
+  constexpr int QROWS_PER_LOAD = Cfg::NT / QCPR;
+  static_assert(BK % QROWS_PER_LOAD == 0 && QROWS_PER_LOAD % 4 == 0, "K-major tile/threads");
+  const int qk_row = tid / QCPR;
+  const int qk_chunk = ((((tid % QCPR) >> 2) ^ (qk_row & 3)) << 2) | (tid & 3);
+  const uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
+  const uint32_t offQ = (uint32_t)(qk_row * p.ldq + qk_chunk * 8) * 2u;
+  const uint32_t stepP = (uint32_t)(Cfg::ROWS_PER_LOAD * p.ldp) * 2u;
+  const uint32_t stepQ = (uint32_t)(QROWS_PER_LOAD * p.ldq) * 2u;
+  const int64_t slabQ = (int64_t)BK * p.ldq * 2;
+
+  int b_c, ti_c, tj_c, b_n, ti_n, tj_n;
+  int pid = blockIdx.x;
+  tile_of(pid, b_c, ti_c, tj_c);
+  auto base_p = [&](int b, int ti) { return (const char*)(p.P + (int64_t)b * p.strideP + (int64_t)(ti * BM) * p.ldp); };
+  auto base_q = [&](int b, int tj) { return (const char*)(p.Q + (int64_t)b * p.strideQ + tj * BN); };
+  const char* gP_c = base_p(b_c, ti_c);
+  const char* gQ_c = base_q(b_c, tj_c);
+  const char *gP_n = gP_c, *gQ_n = gQ_c;
+  auto look_ahead = [&]() {
+    // the tile after the current one; past the end of the list the current tile stands in (its slabs are
+    // fetched again and never read, which keeps the load count per slab fixed)
+    const int np = pid + (int)gridDim.x;
+    if (np < total_tiles) {
+      tile_of(np, b_n, ti_n, tj_n);
+      gP_n = base_p(b_n, ti_n);
+      gQ_n = base_q(b_n, tj_n);
+    } else {
+      b_n = b_c; ti_n = ti_c; tj_n = tj_c;
+      gP_n = gP_c; gQ_n = gQ_c;
+    }
+  };
+  look_ahead();
+
+  // slab kt of the current tile, or slab kt - KT of the next one, into ring slot buf (load j of LPS)
+  auto issue_load = [&](int kt, int buf, int j) {
+    const bool nx = kt >= KT;
+    const int k = nx ? kt - KT : kt;
+    char* l = lds + buf * Cfg::STAGE_BYTES + wave * (64 * 16);
+    if (j < Cfg::P_LOADS) {
+      const char* src = (nx ? gP_n : gP_c) + (int64_t)k * (BK * 2) + (offP + j * stepP);
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
+    } else {
+      const int jq = j - Cfg::P_LOADS;
+      const char* src = (nx ? gQ_n : gQ_c) + k * slabQ + (offQ + jq * stepQ);
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + Cfg::P_BYTES + jq * (Cfg::NT * 16)), 16, 0, 0);
+    }
+  };
+
+  // ---- LDS -> register fragments (see the kernel above)
+  const int frow = lane & 31;
+  const int fhalf = lane >> 5;
+  const int fswz = (frow / Cfg::SWZ_DIV) % Cfg::CPR;
+  uint32_t aoff[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk)
+    aoff[kk] = (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + ((kk * 2 + fhalf) ^ fswz) * 16);
+  uint32_t qoff[TN];
+  {
+    const int g16 = lane >> 4, t16 = lane & 15;
+#pragma unroll
+    for (int r = 0; r < TN; ++r)
+      qoff[r] = (uint32_t)(Cfg::P_BYTES + (8 * (g16 >> 1) + (t16 >> 2)) * (BN * 2) +
+                           ((((wn * Cfg::WTN + r * 32) >> 5) ^ (t16 >> 2)) << 6) + (g16 & 1) * 32 + (t16 & 3) * 8);
+  }
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+  bf16x8 fa[2][TM], fb[2][TN];
+  // The transposing reads are assembly the compiler cannot see in flight; this wait takes the fragments it
+  // guards as read-write operands, so no use of them is scheduled ahead of it (see the kernel above).
+  auto qk_wait = [&](int f) { asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(fb[f][0]), "+v"(fb[f][1]) : "n"(TM - 1)); };
+  auto read_frag = [&](int buf, int kk, int f, int r) {
+    const char* st = lds + buf * Cfg::STAGE_BYTES;
+    if (r == 0 || r > TN) {
+      const int i = r == 0 ? 0 : r - TN;
+      fa[f][i] = *(const bf16x8*)(st + aoff[kk] + i * (32 * BK * 2));
+    } else {
+      const int j = r - 1;
+      const uint32_t a = lds_base + (uint32_t)(buf * Cfg::STAGE_BYTES) + qoff[j] + (uint32_t)(kk * (16 * BN * 2));
+      typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+      u32x2 lo, hi;
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(a));
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(a), "n"(4 * BN * 2));
+      typedef __attribute__((ext_vector_type(4))) unsigned u32x4f;
+      const u32x4f v = {lo[0], lo[1], hi[0], hi[1]};
+      fb[f][j] = __builtin_bit_cast(bf16x8, v);
+    }
+  };
+
+  f32x16 acc[TM][TN];
+  auto clear_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  };
+  clear_acc();
+
+  // ---- epilogue addressing: lane = (line wl, half wh) when staging, (line rl, 16-byte piece rq) when storing
+  char* stg = lds + Cfg::RING_BYTES + wave * STG_WAVE;
+  const int wl = lane & 31, wh = lane >> 5;
+  const int rl = lane >> 3, rq = lane & 7;
+  const int ld_out = OUT_T ? p.ldct : p.ldc;
+
+  auto store_tile = [&](int b, int ti, int tj) {
+    const int row_base = ti * BM + wm * Cfg::WTM;
+    const int col_base = tj * BN + wn * Cfg::WTN;
+    bf16_t* out = OUT_T ? p.Ct + (int64_t)b * p.strideCt + (int64_t)col_base * ld_out + row_base
+                        : p.C + (int64_t)b * p.strideC + (int64_t)row_base * ld_out + col_base;
+    const __amdgpu_buffer_rsrc_t rs = bx_resource(out);
+    const int lane_bytes = (rl * ld_out + rq * 8) * 2;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      // chunk c: accumulator tiles t2 = 0, 1 side by side along the 128-byte lines
+      const int line0 = OUT_T ? (c >> 1) * 32 : c * 32;   // first output line of the chunk (relative)
+      const int run0 = OUT_T ? (c & 1) * 64 : 0;          // first element of the chunk within a line
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        const f32x16& a = OUT_T ? acc[(c & 1) * 2 + t2][c >> 1] : acc[c][t2];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          uint2 pk;
+          pk.x = pack_bf16x2(a[g * 4 + 0], a[g * 4 + 1]);
+          pk.y = pack_bf16x2(a[g * 4 + 2], a[g * 4 + 3]);
+          // 8-byte piece t2*8 + 2g + wh of line wl; XOR with the line pair number spreads the 32 lines of
+          // a half wavefront over all 64 banks
+          *(uint2*)(stg + wl * 128 + (((t2 * 8 + 2 * g + wh) ^ ((wl >> 1) & 15)) << 3)) = pk;
+        }
+      }
+      asm volatile("" ::: "memory");
+      uint2 lo[4], hi[4];
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int line = rl + 8 * it;
+        const int sw = (line >> 1) & 15;
+        lo[it] = *(const uint2*)(stg + line * 128 + (((2 * rq) ^ sw) << 3));
+        hi[it] = *(const uint2*)(stg + line * 128 + (((2 * rq + 1) ^ sw) << 3));
+      }
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const bx_u32x4 o = {lo[it].x, lo[it].y, hi[it].x, hi[it].y};
+        __builtin_amdgcn_raw_buffer_store_b128(o, rs, lane_bytes, ((line0 + 8 * it) * ld_out + run0) * 2, 0);
+      }
+    }
+  };
+
+  // ---- prologue: slab 0 of the first tile, its first fragments, slab 1
+#pragma unroll
+  for (int j = 0; j < LPS; ++j) issue_load(0, 0, j);
+  pipeline_barrier<0>();
+#pragma unroll
+  for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
+#pragma unroll
+  for (int j = 0; j < LPS; ++j) issue_load(1, 1, j);
+  __builtin_amdgcn_sched_barrier(0);
+
+  for (;;) {
+    // ---- one tile: the main loop of the kernel above; refills past the tile's last slab fetch the next tile
+    for (int kt0 = 0; kt0 < KT; kt0 += NSTAGE) {
+#pragma unroll
+      for (int s = 0; s < NSTAGE; ++s) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          const int cur = kk & 1, nxt = cur ^ 1;
+          const bool last = (kk == KK - 1);
+          if (last) pipeline_barrier<0>();
+          qk_wait(cur);
+#pragma unroll
+          for (int q = 0; q < NM; ++q) {
+            if constexpr (OUT_T)
+              acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][q / TN], fb[cur][q % TN],
+                                                                            acc[q / TN][q % TN], 0, 0, 0);
+            else
+              acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][q % TN], fa[cur][q / TN],
+                                                                            acc[q / TN][q % TN], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = q * RPM; r < (q + 1) * RPM && r < NR; ++r) {
+              if (last) read_frag((s + 1) % NSTAGE, 0, nxt, r);
+              else read_frag(s, kk + 1, nxt, r);
+            }
+            if (last) {
+#pragma unroll
+              for (int j = q * LPM; j < (q + 1) * LPM && j < LPS; ++j) issue_load(kt0 + s + NSTAGE, s, j);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      }
+    }
+    // The first fragments of the next tile are on their way into set 0.  Let them land before the epilogue:
+    // its register traffic must not meet a transposing read still in flight.
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fb[0][0]), "+v"(fb[0][1]));
+    store_tile(b_c, ti_c, tj_c);
+    pid += (int)gridDim.x;
+    if (pid >= total_tiles) break;
+    clear_acc();
+    b_c = b_n; ti_c = ti_n; tj_c = tj_n;
+    gP_c = gP_n; gQ_c = gQ_n;
+    look_ahead();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  wait_vmcnt<0>();  // the stand-in refills of the last tile must land before the LDS is given back
+}
+
+// ---------------------------------------------------------------------------------------------
 typedef TileCfg<128, 128, 64, 2, 2, 2> Cfg128;     // 4 wavefronts, 64x64 each; two workgroups per CU
 typedef TileCfg<256, 256, 64, 2, 4, 2> Cfg256w8;   // 8 wavefronts, 128x64 each: two per SIMD, one workgroup per CU
+constexpr int kWalkMaxK = 2048;                    // longest reduction the tile-walking kernel is used for
 
 // Tile list dealt to the XCDs in interleaved 32-tile chunks (see the kernel) when the first operand of
 // one matrix is at least 16 MB; below that a contiguous run per XCD keeps whole matrices in one L2.
@@ -661,6 +937,34 @@ static hipError_t launch_epi(const GemmParams& p, hipStream_t stream,
   return hipGetLastError();
 }
 
+// One workgroup per CU, each walking its share of the tile list.
+template <class Cfg, bool OUT_T>
+static hipError_t launch_walk(const GemmParams& p, hipStream_t stream) {
+  static std::atomic<uint64_t> attr_done{0};
+  constexpr int kLds = Cfg::RING_BYTES + Cfg::WM * Cfg::WN * 32 * 128;
+  auto kern = gemm_qk_walk_kernel<Cfg, OUT_T>;
+  if (hipError_t e = set_max_dynamic_lds_once((const void*)kern, kLds, attr_done)) return e;
+  const int64_t total = (int64_t)(p.M / Cfg::BM) * (p.N / Cfg::BN) * p.batch;
+  if (total <= 0) return hipSuccess;
+  if (total > 0x7fffffff) return hipErrorInvalidValue;
+  // a wavefront's output tile is addressed with 32-bit byte offsets from its first element
+  if ((int64_t)(OUT_T ? p.ldct : p.ldc) * 129 * 2 > 0x7fffffffLL) return hipErrorInvalidValue;
+  static std::atomic<int> cu_count[64];
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  int cus = cu_count[dev & 63].load(std::memory_order_relaxed);
+  if (cus == 0) {
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) return e;
+    if (cus <= 0) return hipErrorInvalidValue;
+    cu_count[dev & 63].store(cus, std::memory_order_relaxed);
+  }
+  GemmParams pp = p;
+  pp.xcd_interleave = xcd_interleave_pays(p) ? 1 : 0;
+  const unsigned grid = (unsigned)(total < cus ? total : cus);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::NT), kLds, stream, pp, (int)total);
+  return hipGetLastError();
+}
+
 // The operand / result combinations the Newton-Schulz drivers use.
 template <class Cfg>
 static hipError_t launch_cfg(const GemmParams& p, hipStream_t stream) {
@@ -668,6 +972,14 @@ static hipError_t launch_cfg(const GemmParams& p, hipStream_t stream) {
   const bool d = p.D != nullptr, c = p.C != nullptr, ct = p.Ct != nullptr;
   if (p.q_kmajor) {
     if (p.tri) return hipErrorInvalidValue;
+    if constexpr (Cfg::BM == 256) {
+      // Short reductions go to the tile-walking kernel: what it saves is a fixed cost per tile, 13 % of the
+      // launch at 32 slabs and nothing at 64 (where its static tile order costs as much as it saves).
+      if (p.K <= kWalkMaxK && p.alpha == 1.0f) {  // (the drivers' X' products are unscaled)
+        if (!d && c && !ct) return launch_walk<Cfg, false>(p, stream);  // X' = B X
+        if (!d && !c && ct) return launch_walk<Cfg, true>(p, stream);   // (B X)^T only
+      }
+    }
     if (!d && c && !ct) return launch_epi<Cfg, false, true, false, true>(p, stream);  // X' = B X
     if (!d && !c && ct) return launch_epi<Cfg, false, false, true, true>(p, stream);  // (B X)^T only
     if (d && c && !ct) return launch_epi<Cfg, true, true, false, true>(p, stream);    // a X + B X

@@ -113,10 +113,12 @@ def test_line_3_short_reduction_many_launches(batch, m, n):
 
 
 @pytest.mark.parametrize("batch,m,n", [(24, 512, 8192), (5, 1024, 14336), (3, 2304, 10240), (2, 4096, 8192),
-                                       (33, 768, 4096)])
+                                       (33, 768, 4096), (4, 768, 8192), (3, 1280, 7168), (7, 2048, 3584)])
 def test_line_3_thousand_tile_launches(batch, m, n):
-    """X' = B X over a thousand or more 256-wide tiles (tile counts that are and are not multiples of the CU
-    count; both tile orders): the product, and the same bits on every launch."""
+    """X' = B X over hundreds to thousands of 256-wide tiles (tile counts that are and are not multiples of the
+    CU count, so that workgroups of the tile-walking kernel -- reductions up to 2048 -- take unequal numbers
+    of tiles; both tile orders; longer reductions on the one-tile-per-workgroup kernel): the product, and
+    the same bits on every launch."""
     lib, check = _lib()
     torch.manual_seed(batch + m + n)
     X = torch.randn(batch, m, n, device=DEV).to(torch.bfloat16)
@@ -134,6 +136,15 @@ def test_line_3_thousand_tile_launches(batch, m, n):
         check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), C.data_ptr(), batch, m, n, ctypes.c_float(0.0), st),
               "line_3")
         assert torch.equal(C, first), rep
+    if m <= 2048:
+        # the transposed-output form (last product of a tall orthogonalization) of the same launches
+        from dion_amd import zeropower_via_newtonschulz5
+
+        del first, C
+        wide = zeropower_via_newtonschulz5(X)
+        tall_in = X.mT.contiguous()
+        for _ in range(2):
+            assert torch.equal(zeropower_via_newtonschulz5(tall_in), wide.mT)
 
 
 def test_line_3_argument_errors():

@@ -2,7 +2,7 @@
 know that the results are still on their way when the statement has executed: it may hand a destination register
 it considers dead to something else, and a read that lands late then overwrites that value (once: the lane index
 ahead of the epilogue's address arithmetic, a GPU memory fault).  This test compiles gemm_nt.hip to gfx950 assembly
-and walks every kernel that contains such reads in program order (each loop back-edge taken once), modelling the
+and walks every kernel that contains such reads (gemm_nt_kernel, gemm_qk_walk_kernel) in program order (each loop back-edge taken once), modelling the
 LDS return queue (in-order; s_waitcnt lgkmcnt(N) retires all but the newest N entries): no instruction may read or
 write a register while a transposing read into it is in flight.  Needs hipcc, no GPU."""
 import os
@@ -86,13 +86,14 @@ def test_no_kernel_touches_a_register_a_transposing_read_is_in_flight_to(tmp_pat
     kernels, name, body = {}, None, []
     for line in out.read_text().split("\n"):
         if name is None:
-            if re.match(r"_ZN4dion14gemm_nt_kernel\S*:", line):
+            if re.match(r"_ZN4dion\d+gemm_(nt|qk_walk)_kernel\S*:", line):
                 name, body = line.split(":")[0], []
         else:
             body.append(line)
             if "s_endpgm" in line:
                 kernels[name], name = body, None
-    assert len(kernels) >= 20, "expected every gemm_nt_kernel instantiation in the assembly"
+    assert len(kernels) >= 22, "expected every gemm_nt_kernel / gemm_qk_walk_kernel instantiation in the assembly"
+    assert sum("gemm_qk_walk_kernel" in k for k in kernels) == 2
     with_tr = 0
     for kname, kbody in kernels.items():
         n_tr, hazards = walk(kbody)
