@@ -147,6 +147,33 @@ def test_line_3_thousand_tile_launches(batch, m, n):
             assert torch.equal(zeropower_via_newtonschulz5(tall_in), wide.mT)
 
 
+def test_line_3_seeded_sweep_of_walked_tile_lists():
+    """Twenty seeded (batch, m, n) with 256-wide tiles, reductions of 256..2048 and 384..1500 tiles: lists whose
+    length is anything modulo the CU count, matrices that end in the middle of a workgroup's share."""
+    lib, check = _lib()
+    rng = np.random.default_rng(20240607)
+    st = _stream()
+    done = 0
+    while done < 20:
+        m = 256 * int(rng.integers(1, 9))
+        n = 256 * int(rng.integers(1, 33))
+        batch = int(rng.integers(1, 41))
+        tiles = (m // 256) * (n // 256) * batch
+        if not 384 <= tiles <= 1500:
+            continue
+        done += 1
+        torch.manual_seed(done)
+        X = torch.randn(batch, m, n, device=DEV).to(torch.bfloat16)
+        Bm = torch.randn(batch, m, m, device=DEV)
+        Bm = ((Bm + Bm.mT) / 2).to(torch.bfloat16)
+        C = torch.full_like(X, float("nan"))
+        check(lib.dion_ns_line_3(Bm.data_ptr(), X.data_ptr(), C.data_ptr(), batch, m, n, ctypes.c_float(0.0), st),
+              "line_3")
+        ref = torch.bmm(Bm.float(), X.float())
+        err = float((C.float() - ref).norm() / ref.norm())
+        assert err <= 4e-3, (batch, m, n, tiles, err)
+
+
 def test_line_3_argument_errors():
     lib, check = _lib()
     from dion_amd._lib import DionHipError
