@@ -52,7 +52,26 @@ def build(verbose: bool = True) -> str:
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
+    build_c_caller(verbose)
     return LIB_PATH
+
+
+C_CALLER_SRC = os.path.join(os.path.dirname(HERE), "tests", "c_caller", "ns_caller.c")
+C_CALLER_BIN = os.path.join(os.path.dirname(HERE), "tests", "c_caller", "ns_caller")
+
+
+def build_c_caller(verbose: bool = True) -> str:
+    """The C program under tests/c_caller (a caller of the library with no Python or C++ in it), compiled
+    with the host C compiler against include/dion_hip.h and linked to the library just built."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["gcc", "-std=c11", "-Wall", "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include",
+           "-I" + os.path.join(os.path.dirname(HERE), "include"), C_CALLER_SRC, "-o", C_CALLER_BIN,
+           "-L" + HERE, "-ldion_hip", f"-L{rocm}/lib", "-lamdhip64", "-lm",
+           "-Wl,-rpath,$ORIGIN/../../dion_amd", f"-Wl,-rpath,{rocm}/lib"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return C_CALLER_BIN
 
 
 if __name__ == "__main__":
