@@ -418,6 +418,14 @@ def main() -> int:
             "pct_of_bf16_peak": round(100.0 * ns_tf / PEAK_BF16_TFLOPS, 2),
         }
         del X
+        if args.workload == "gpt_small_heads":
+            # the per-head group on its own: 36 heads x 12 layers of 64 x 768, one LDS-resident launch
+            Xh = (torch.randn(432, 64, 768, device=dev) * 0.01).to(torch.bfloat16)
+            ms_h = time_kernel(lambda: fn(Xh, 1e-8), iters=20)
+            h_tf = 432 * ns_flops(64, 768) / (ms_h * 1e-3) * 1e-12
+            result["ns_per_head"] = {"shape": "432x(64x768)", "us": round(ms_h * 1e3, 1), "tflops": round(h_tf, 1),
+                                     "pct_of_bf16_peak": round(100.0 * h_tf / PEAK_BF16_TFLOPS, 2)}
+            del Xh
         torch.cuda.empty_cache()
 
     if args.stream_compare:
