@@ -52,7 +52,6 @@ def build(verbose: bool = True) -> str:
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    build_c_caller(verbose)
     return LIB_PATH
 
 
@@ -75,6 +74,15 @@ def build_c_caller(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
+    # `--c-caller` builds only the C test program (needs gcc and a built library); the default builds the
+    # library (needs hipcc only) and, when gcc is there, the C test program as well.
+    import shutil
+
+    if "--c-caller" in sys.argv[1:]:
+        print(build_c_caller())
+        sys.exit(0)
     build()
     print(LIB_PATH)
+    if shutil.which("gcc") is not None:
+        print(build_c_caller())
     sys.exit(0)

@@ -15,7 +15,7 @@ DION_BF16 = 0
 DION_F32 = 1
 DION_NS_GRAM = 1
 DION_NS_STATIC_SCRATCH_BYTES = 64 << 20
-ABI_VERSION = 11  # dion_abi_version() of the library these signatures describe
+ABI_VERSION = 12  # dion_abi_version() of the library these signatures describe
 
 _u64p = ctypes.POINTER(ctypes.c_uint64)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -38,6 +38,20 @@ SIGNATURES = {
     "dion_ns_orthogonalize_update": (c_int, [c_void_p, c_int, _u64p, c_int, c_int, c_int, c_int, c_int, _f32p,
                                              c_int, c_float, c_float, c_int, c_int, c_void_p, c_float, c_void_p,
                                              c_float, c_int, c_void_p, c_size_t, c_void_p]),
+    "dion_ns_accepts_prepared": (c_int, [c_int, c_int, c_int, c_int, c_int]),
+    "dion_ns_orthogonalize_prepared": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, _f32p,
+                                               c_int, c_float, c_float, c_int, c_int, c_void_p, c_size_t,
+                                               c_void_p]),
+    "dion_ns_orthogonalize_update_prepared": (c_int, [c_void_p, c_void_p, c_int, _u64p, c_int, c_int, c_int, c_int,
+                                                      c_int, _f32p, c_int, c_float, c_float, c_int, c_int, c_void_p,
+                                                      c_float, c_void_p, c_float, c_int, c_void_p, c_size_t,
+                                                      c_void_p]),
+    "dion_ns_plan_audit_prepared": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                            c_size_t]),
+    "dion_gemm_tile_edge": (c_int, [c_int, c_int, c_int, c_int]),
+    "dion_muon_pre_sumsq_blocks": (c_int, [c_int, c_int]),
+    "dion_muon_pre_prepared": (c_int, [_u64p, c_int, _u64p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                       c_float, c_int, c_void_p]),
     "dion_muon_pre": (c_int, [_u64p, c_int, _u64p, c_int, c_void_p, c_int, c_int64, c_float, c_int, c_void_p]),
     "dion_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_void_p]),
     "dion_muon_post": (c_int, [_u64p, c_int, c_void_p, c_int, c_int, c_int64, c_int, c_void_p, c_void_p, c_void_p,

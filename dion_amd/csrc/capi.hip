@@ -37,7 +37,7 @@ static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 extern "C" const char* dion_last_error(void) { return g_err; }
-extern "C" int dion_abi_version(void) { return 11; }
+extern "C" int dion_abi_version(void) { return 12; }
 
 // ---------------------------------------------------------------------------------------------
 // Kernel-level GEMMs
@@ -212,15 +212,27 @@ bool ns_update_fuses(int batch, int rows, int cols, int flags, int n_iters) {
   return pl.mp == pl.m && pl.np == pl.n;
 }
 
+// A prepared input (short side along rows, unnormalised, with partial sums of squares) is taken when
+// the matrices fill whole tiles -- no padding, so the input can be the first GEMMs' operand as it lies --
+// outside the LDS-resident kernel and with at least one iteration to carry the normalisation.
+bool ns_accepts_prepared(int batch, int rows, int cols, int flags, int n_iters) {
+  if (batch <= 0 || batch > 65535 || rows <= 0 || cols <= 0 || n_iters <= 0) return false;
+  if (ns_small_path(rows, cols, flags, n_iters)) return false;
+  if (((int64_t)rows * cols) % 4096) return false;
+  const NsPlan pl = make_plan(batch, rows, cols, flags);
+  return pl.mp == pl.m && pl.np == pl.n;
+}
+
 // One kernel launch of a planned call.
 struct NsStep {
-  enum Kind { kNorm, kPrepare, kGemm, kGemmUpdate, kUnpad, kSmall } kind;
+  enum Kind { kNorm, kNormFinalize, kPrepare, kGemm, kGemmUpdate, kUnpad, kSmall } kind;
   const char* what;
   GemmParams g;    // kGemm, kGemmUpdate
-  FusedPost fp;    // kGemmUpdate
+  // kGemmUpdate: the launch updates parameters ptr0 .. ptr0 + n_ptr - 1 of the call's table
+  int ptr0, n_ptr;
   int x_code;      // kGemmUpdate: 0 bf16, 1 fp32 parameters
   bool transposed; // kGemmUpdate: the product updates X[col][row]
-  // kNorm, kPrepare, kSmall: the caller's input
+  // kNorm, kPrepare, kSmall: the caller's input; kNormFinalize: `partial` is read, not written
   const void* in;
   int in_dtype, batch, R, C;
   float norm_scale, eps;
@@ -242,10 +254,20 @@ struct NsStep {
   NsCoeffs co;  // kSmall
 };
 
+// The launch list of one call.  Fixed capacity and no heap: planning a call allocates nothing, on
+// the host or on the device.  A standard iteration is three launches, a Gram iteration at most five.
+constexpr int kMaxSteps = 160;
 struct NsCall {
-  std::vector<NsStep> steps;
-  // what the call may read and write: [lo, hi) byte ranges
-  const char *in_lo, *in_hi, *out_lo, *out_hi, *ws_lo, *ws_hi;
+  NsStep steps[kMaxSteps];
+  int n_steps;
+  bool overflow;
+  void push(const NsStep& s) {
+    if (n_steps < kMaxSteps) steps[n_steps++] = s;
+    else overflow = true;
+  }
+  const PostSpec* post;  // the update a kGemmUpdate step applies
+  // what the call may read and write: [lo, hi) byte ranges (sq: the caller's norm partials, read only)
+  const char *in_lo, *in_hi, *out_lo, *out_hi, *ws_lo, *ws_hi, *sq_lo, *sq_hi;
   // parameters updated in place by a fused update: n_ptrs ranges of x_bytes each
   const uint64_t* X_ptrs;
   int n_ptrs;
@@ -262,11 +284,18 @@ NsStep blank_step(NsStep::Kind kind, const char* what) {
 
 // Builds the launch list of one orthogonalization (no HIP call is made).  With `post` (only when
 // ns_update_fuses) the last GEMM applies the update to the parameters and `out` is not written.
+// With `sumsq` the input is "prepared": bf16 [batch, m, n] with the short side along rows (the transpose
+// of a tall caller matrix), not normalised, and sumsq [batch, sumsq_blocks] holds partial sums of its
+// squares per matrix.  The normalisation is then folded into the first two GEMMs as a per-matrix factor
+// and neither the norm pass nor the prepare pass runs (only when ns_accepts_prepared).
 int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int cols, const float* coeffs,
              int n_iters, float norm_scale, float eps, int flags, int gram_reset, void* workspace,
-             size_t workspace_bytes, const PostSpec* post, NsCall& call) {
-  call.steps.clear();
-  call.in_lo = call.in_hi = call.out_lo = call.out_hi = call.ws_lo = call.ws_hi = nullptr;
+             size_t workspace_bytes, const PostSpec* post, NsCall& call, const float* sumsq = nullptr,
+             int sumsq_blocks = 0) {
+  call.n_steps = 0;
+  call.overflow = false;
+  call.post = post;
+  call.in_lo = call.in_hi = call.out_lo = call.out_hi = call.ws_lo = call.ws_hi = call.sq_lo = call.sq_hi = nullptr;
   call.X_ptrs = nullptr;
   call.n_ptrs = 0;
   call.x_bytes = 0;
@@ -290,6 +319,16 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
     call.n_ptrs = post->n_ptrs;
     call.x_bytes = (size_t)post->mats_per_ptr * mat_elems * (post->x_dtype == DION_BF16 ? 2 : 4);
   }
+  if (sumsq) {
+    if (!ns_accepts_prepared(batch, rows, cols, flags, n_iters) || in_dtype != DION_BF16 || sumsq_blocks <= 0)
+      return fail(DION_E_INVALID,
+                  "dion_ns_orthogonalize_prepared: %d x (%d x %d), %d iterations does not take a prepared input "
+                  "(see dion_ns_accepts_prepared)", batch, rows, cols, n_iters);
+    if (!aligned16((uint64_t)(uintptr_t)in))
+      return fail(DION_E_INVALID, "dion_ns_orthogonalize_prepared: in is not 16-byte aligned");
+    call.sq_lo = (const char*)sumsq;
+    call.sq_hi = call.sq_lo + (size_t)batch * sumsq_blocks * 4;
+  }
   if (ns_small_path(rows, cols, flags, n_iters)) {
     NsStep s = blank_step(NsStep::kSmall, "small-matrix Newton-Schulz");
     s.in = in;
@@ -302,7 +341,7 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
     s.eps = eps;
     s.co.n = n_iters;
     for (int i = 0; i < n_iters * 3; ++i) s.co.c[i / 3][i % 3] = coeffs[i];
-    call.steps.push_back(s);
+    call.push(s);
     return DION_OK;
   }
   // the last GEMM stores into the caller's buffer 16 bytes per lane
@@ -337,7 +376,16 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
 
   const int mp = pl.mp, np = pl.np;
   const int64_t sX = (int64_t)mp * np, sA = (int64_t)mp * mp;
-  {
+  if (sumsq) {
+    NsStep s = blank_step(NsStep::kNormFinalize, "frobenius norm from the caller's partial sums");
+    s.batch = batch;
+    s.norm_scale = norm_scale;
+    s.eps = eps;
+    s.partial = const_cast<float*>(sumsq);
+    s.nblk = sumsq_blocks;
+    s.inv = inv;
+    call.push(s);
+  } else {
     NsStep s = blank_step(NsStep::kNorm, "frobenius norm");
     s.in = in;
     s.in_dtype = in_dtype;
@@ -349,9 +397,9 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
     s.partial = partial;
     s.nblk = pl.nblk;
     s.inv = inv;
-    call.steps.push_back(s);
+    call.push(s);
   }
-  {
+  if (!sumsq) {
     // Only X (short side along rows) is carried between iterations: X' = B X reads X with the
     // reduction index along rows.  With no iteration at all the result is the prepared input, and
     // the output copy of a tall input reads X^T: prepare that layout instead.
@@ -378,7 +426,7 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
       s.ld_same = np;
       s.stride_same = sX;
     }
-    call.steps.push_back(s);
+    call.push(s);
   }
 
   const bool direct = (mp == pl.m && np == pl.n);
@@ -406,12 +454,22 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
     p.alpha = alpha;
     p.beta = beta;
     p.diag = diag;
-    call.steps.push_back(s);
+    call.push(s);
+  };
+  // A prepared input is the unnormalised X_0: every GEMM that reads it carries the factor 1/(||X_0|| s + eps)
+  // (squared for X_0 X_0^T); products of these GEMMs are normalised, and so is every later X.
+  const bf16_t* const x_raw = sumsq ? (const bf16_t*)in : nullptr;
+  auto scaled = [&](GemmParams& p, const bf16_t* Xc, int pow) {
+    if (x_raw && Xc == x_raw) {
+      p.scale_vec = inv;
+      p.scale_pow = pow;
+    }
   };
   // gram(Xc -> R): R = Xc Xc^T
   auto gram = [&](const char* what, const bf16_t* Xc, bf16_t* R) {
     NsStep s = blank_step(NsStep::kGemm, what);
     GemmParams& p = s.g;
+    scaled(p, Xc, 2);
     p.P = p.Q = Xc;
     p.C = p.Ct = R;
     p.strideP = p.strideQ = sX;
@@ -423,7 +481,7 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
     p.batch = batch;
     p.tri = 1;
     p.alpha = 1.0f;
-    call.steps.push_back(s);
+    call.push(s);
   };
   // apply(S, Xc -> Xn | Xt | out | parameters): X' = S X (S symmetric m x m).  The last product of a
   // tall input is written transposed (the caller's orientation); when no padding is in the way
@@ -443,6 +501,7 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
     p.K = mp;
     p.batch = batch;
     p.alpha = 1.0f;
+    scaled(p, Xc, 1);
     if (final_direct && post) {
       // the product is consumed by the update: one launch per kMaxPtrs parameters
       const int mpp = post->mats_per_ptr;
@@ -460,18 +519,13 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
         s.g = p;
         s.g.P = p.P + b0 * p.strideP;
         s.g.Q = p.Q + b0 * p.strideQ;
+        if (s.g.scale_vec) s.g.scale_vec += b0;
         s.g.batch = c * mpp;
-        memcpy(s.fp.X.p, post->X_ptrs + c0, (size_t)c * sizeof(uint64_t));
-        s.fp.mats_per_ptr = mpp;
-        s.fp.vec_ok = table_aligned(post->X_ptrs + c0, c) ? 1 : 0;
-        s.fp.lr_dev = post->lr_dev;
-        s.fp.wd_dev = post->wd_dev;
-        s.fp.wd_host = post->wd_host;
-        s.fp.adj_ratio = post->adj_ratio;
-        s.fp.cautious = post->cautious;
+        s.ptr0 = c0;
+        s.n_ptr = c;
         s.x_code = dt(post->x_dtype);
         s.transposed = pl.tall != 0;
-        call.steps.push_back(s);
+        call.push(s);
       }
       return;
     }
@@ -496,21 +550,25 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
     }
     NsStep s = blank_step(NsStep::kGemm, what);
     s.g = p;
-    call.steps.push_back(s);
+    call.push(s);
   };
 
   int cur = 0;
   bool wrote_out = false;
+  // the matrix the next GEMM reads as X: the caller's prepared input until the first X' is written
+  bool x_written = false;
+  auto xc = [&]() -> const bf16_t* { return (x_raw && !x_written) ? x_raw : X[cur]; };
   if (!pl.gram) {
     for (int it = 0; it < n_iters; ++it) {
       const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
-      gram("A = X X^T", X[cur], sq[0]);
+      gram("A = X X^T", xc(), sq[0]);
       // a*I folded into B: the next GEMM needs no addend (one fewer pass over X)
       sym("B = c A A + b A + a I", sq[0], sq[0], sq[0], sq[1], c, b, a);
       const bool fin = (it == n_iters - 1) && direct;
-      apply("X = B X", sq[1], X[cur], X[cur ^ 1], it == n_iters - 1, fin);
+      apply("X = B X", sq[1], xc(), X[cur ^ 1], it == n_iters - 1, fin);
       wrote_out = fin;
       cur ^= 1;
+      x_written = true;
     }
   } else {
     // Gram recurrence: R = X X^T and Q with X_t = Q X_0 live in m x m; per iteration
@@ -527,15 +585,16 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
       return -1;
     };
     int r = take(), q = -1;
-    gram("R = X X^T", X[cur], sq[r]);
+    gram("R = X X^T", xc(), sq[r]);
     for (int it = 0; it < n_iters; ++it) {
       const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
       if (it == gram_reset && it > 0 && q >= 0) {
-        apply("X = Q X (restart)", sq[q], X[cur], X[cur ^ 1], false, false);
+        apply("X = Q X (restart)", sq[q], xc(), X[cur ^ 1], false, false);
         cur ^= 1;
+        x_written = true;
         used[q] = false;
         q = -1;
-        gram("R = X X^T (restart)", X[cur], sq[r]);
+        gram("R = X X^T (restart)", xc(), sq[r]);
       }
       const int z = take();
       sym("Z = a I + b R + c R R", sq[r], sq[r], sq[r], sq[z], c, b, a);
@@ -560,9 +619,10 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
       }
     }
     if (q >= 0) {
-      apply("X = Q X", sq[q], X[cur], X[cur ^ 1], true, direct);
+      apply("X = Q X", sq[q], xc(), X[cur ^ 1], true, direct);
       wrote_out = direct;
       cur ^= 1;
+      x_written = true;
     }
   }
   if (!wrote_out) {
@@ -577,8 +637,11 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
     s.batch = batch;
     s.R = rows;
     s.C = cols;
-    call.steps.push_back(s);
+    call.push(s);
   }
+  if (call.overflow)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize: more than %d kernel launches in one call (%d iterations, %d "
+                "parameters): split the call", kMaxSteps, n_iters, post ? post->n_ptrs : 0);
   return DION_OK;
 }
 
@@ -603,10 +666,14 @@ int ns_audit(const NsCall& call) {
   auto wr = [&](const void* p, size_t bytes) {
     return inside(p, bytes, call.ws_lo, call.ws_hi) || inside(p, bytes, call.out_lo, call.out_hi);
   };
-  int idx = 0;
-  for (const NsStep& s : call.steps) {
+  for (int idx = 0; idx < call.n_steps; ++idx) {
+    const NsStep& s = call.steps[idx];
     const char* bad = nullptr;
     switch (s.kind) {
+      case NsStep::kNormFinalize:
+        if (s.nblk <= 0 || !inside(s.partial, (size_t)s.batch * s.nblk * 4, call.sq_lo, call.sq_hi)) bad = "norm partials";
+        else if (!wr(s.inv, (size_t)s.batch * 4)) bad = "reciprocal norms";
+        break;
       case NsStep::kNorm: {
         const size_t es = s.in_dtype == DION_BF16 ? 2 : 4;
         if (!rd(s.in, (size_t)s.batch * s.R * s.C * es)) bad = "input";
@@ -635,20 +702,25 @@ int ns_audit(const NsCall& call) {
                               : rd(p.Q, span_bytes(p.batch, p.strideQ, p.N, p.ldq, p.K, 2))))
           bad = "second operand";
         else if (p.D && !rd(p.D, span_bytes(p.batch, p.strideD, p.M, p.ldd, p.N, 2))) bad = "addend";
+        else if (p.scale_vec && (!inside(p.scale_vec, (size_t)p.batch * 4, call.ws_lo, call.ws_hi) ||
+                                 (p.scale_pow != 1 && p.scale_pow != 2)))
+          bad = "per-matrix factors";
         else if (p.C && !wr(p.C, span_bytes(p.batch, p.strideC, p.M, p.ldc, p.N, 2))) bad = "product";
         else if (p.Ct && !wr(p.Ct, span_bytes(p.batch, p.strideCt, p.N, p.ldct, p.M, 2))) bad = "transposed product";
         else if (s.kind == NsStep::kGemm && !p.C && !p.Ct) bad = "no destination";
         else if (s.kind == NsStep::kGemmUpdate) {
           // matrix b updates parameter b / mats_per_ptr at matrix offset b % mats_per_ptr
           const int es = s.x_code == 0 ? 2 : 4;
-          const int mpp = s.fp.mats_per_ptr;
+          const int mpp = call.post ? call.post->mats_per_ptr : 0;
           const size_t one = s.transposed ? span_bytes(1, 0, p.N, p.ldct, p.M, es) : span_bytes(1, 0, p.M, p.ldc, p.N, es);
           const size_t stride = (size_t)(s.transposed ? p.strideCt : p.strideC) * es;
-          if (mpp <= 0 || p.batch > kMaxPtrs * mpp || p.C || p.Ct) bad = "update batch";
+          if (mpp <= 0 || s.n_ptr <= 0 || s.n_ptr > kMaxPtrs || p.batch != s.n_ptr * mpp || s.ptr0 < 0 ||
+              s.ptr0 + s.n_ptr > call.n_ptrs || p.C || p.Ct)
+            bad = "update batch";
           else if ((size_t)(mpp - 1) * stride + one > call.x_bytes) bad = "parameter extent";
           else
-            for (int i = 0; i < (p.batch + mpp - 1) / mpp && !bad; ++i)
-              if (!s.fp.X.p[i]) bad = "null parameter";
+            for (int i = 0; i < s.n_ptr && !bad; ++i)
+              if (!call.X_ptrs[s.ptr0 + i]) bad = "null parameter";
         }
         break;
       }
@@ -666,15 +738,18 @@ int ns_audit(const NsCall& call) {
     if (bad)
       return fail(DION_E_INVALID, "dion_ns_orthogonalize: launch %d (%s) would access its %s outside the call's buffers",
                   idx, s.what, bad);
-    ++idx;
   }
   return DION_OK;
 }
 
 int ns_execute(const NsCall& call, hipStream_t st) {
-  for (const NsStep& s : call.steps) {
+  for (int idx = 0; idx < call.n_steps; ++idx) {
+    const NsStep& s = call.steps[idx];
     hipError_t e = hipSuccess;
     switch (s.kind) {
+      case NsStep::kNormFinalize:
+        e = launch_norm_finalize(s.partial, s.nblk, s.batch, s.norm_scale, s.eps, s.inv, st);
+        break;
       case NsStep::kNorm:
         e = launch_frobenius_inv(s.in, s.in_dtype, s.batch, (int64_t)s.R * s.C, s.norm_scale, s.eps, s.partial,
                                  s.nblk, s.inv, st);
@@ -686,9 +761,21 @@ int ns_execute(const NsCall& call, hipStream_t st) {
       case NsStep::kGemm:
         e = launch_gemm_nt(s.g, st);
         break;
-      case NsStep::kGemmUpdate:
-        e = launch_gemm_nt_post(s.g, s.fp, s.x_code, s.transposed, st);
+      case NsStep::kGemmUpdate: {
+        const PostSpec& ps = *call.post;
+        FusedPost fp;
+        memset((void*)&fp, 0, sizeof(fp));
+        memcpy(fp.X.p, ps.X_ptrs + s.ptr0, (size_t)s.n_ptr * sizeof(uint64_t));
+        fp.mats_per_ptr = ps.mats_per_ptr;
+        fp.vec_ok = table_aligned(ps.X_ptrs + s.ptr0, s.n_ptr) ? 1 : 0;
+        fp.lr_dev = ps.lr_dev;
+        fp.wd_dev = ps.wd_dev;
+        fp.wd_host = ps.wd_host;
+        fp.adj_ratio = ps.adj_ratio;
+        fp.cautious = ps.cautious;
+        e = launch_gemm_nt_post(s.g, fp, s.x_code, s.transposed, st);
         break;
+      }
       case NsStep::kUnpad:
         e = launch_unpad(s.src, s.src_stride, s.ld, s.dst, s.batch, s.R, s.C, st);
         break;
@@ -703,10 +790,11 @@ int ns_execute(const NsCall& call, hipStream_t st) {
 
 int ns_run(const void* in, int in_dtype, void* out, int batch, int rows, int cols, const float* coeffs,
            int n_iters, float norm_scale, float eps, int flags, int gram_reset, void* workspace,
-           size_t workspace_bytes, void* stream, const PostSpec* post) {
-  NsCall call;
+           size_t workspace_bytes, void* stream, const PostSpec* post, const float* sumsq = nullptr,
+           int sumsq_blocks = 0) {
+  NsCall call;  // on the stack: planning allocates nothing
   if (int rc = ns_build(in, in_dtype, out, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
-                        workspace, workspace_bytes, post, call))
+                        workspace, workspace_bytes, post, call, sumsq, sumsq_blocks))
     return rc;
   if (int rc = ns_audit(call)) return rc;
   return ns_execute(call, (hipStream_t)stream);
@@ -826,14 +914,64 @@ extern "C" int dion_ns_orthogonalize_update(const void* in, int in_dtype, const 
                         nullptr, lr_dev, nullptr, adj_ratio, wd_dev, wd_host, cautious, stream);
 }
 
+extern "C" int dion_ns_accepts_prepared(int batch, int rows, int cols, int flags, int n_iters) {
+  if (flags & ~DION_NS_GRAM) return 0;
+  return ns_accepts_prepared(batch, rows, cols, flags, n_iters) ? 1 : 0;
+}
+
+extern "C" int dion_ns_orthogonalize_prepared(const void* in, const float* sumsq, int sumsq_blocks, void* out,
+                                              int batch, int rows, int cols, const float* coeffs, int n_iters,
+                                              float norm_scale, float eps, int flags, int gram_reset,
+                                              void* workspace, size_t workspace_bytes, void* stream) {
+  if (batch == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!sumsq) return fail(DION_E_INVALID, "dion_ns_orthogonalize_prepared: sumsq is null");
+  return ns_run(in, DION_BF16, out, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
+                workspace, workspace_bytes, stream, nullptr, sumsq, sumsq_blocks);
+}
+
+extern "C" int dion_ns_orthogonalize_update_prepared(const void* in, const float* sumsq, int sumsq_blocks,
+                                                     const uint64_t* X_ptrs, int x_dtype, int n_ptrs,
+                                                     int mats_per_ptr, int rows, int cols, const float* coeffs,
+                                                     int n_iters, float norm_scale, float eps, int flags,
+                                                     int gram_reset, const float* lr_dev, float adj_ratio,
+                                                     const float* wd_dev, float wd_host, int cautious,
+                                                     void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = check_state_dtype("dion_ns_orthogonalize_update_prepared", "x_dtype", x_dtype)) return rc;
+  if (n_ptrs < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || n_iters < 0)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize_update_prepared: bad size");
+  if ((int64_t)n_ptrs * mats_per_ptr > 0x7fffffff)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize_update_prepared: too many matrices");
+  const int batch = n_ptrs * mats_per_ptr;
+  if (batch == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!X_ptrs || !lr_dev || !sumsq)
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize_update_prepared: null argument");
+  for (int i = 0; i < n_ptrs; ++i)
+    if (!X_ptrs[i]) return fail(DION_E_INVALID, "dion_ns_orthogonalize_update_prepared: parameter %d is null", i);
+  if (!ns_update_fuses(batch, rows, cols, flags, n_iters))
+    return fail(DION_E_INVALID, "dion_ns_orthogonalize_update_prepared: %d x (%d x %d) does not take a prepared input "
+                "(see dion_ns_accepts_prepared)", batch, rows, cols);
+  const PostSpec ps = {X_ptrs, x_dtype, n_ptrs, mats_per_ptr, lr_dev, adj_ratio, wd_dev, wd_host, cautious};
+  return ns_run(in, DION_BF16, nullptr, batch, rows, cols, coeffs, n_iters, norm_scale, eps, flags, gram_reset,
+                workspace, workspace_bytes, stream, &ps, sumsq, sumsq_blocks);
+}
+
+extern "C" int dion_gemm_tile_edge(int batch, int m, int n, int symmetric) {
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.M = m;
+  p.N = symmetric ? m : n;
+  p.batch = batch;
+  p.tri = symmetric ? 1 : 0;
+  return gemm_tile_edge(p);
+}
+
 // Host-only check of the planning code: builds the launch list of dion_ns_orthogonalize
 // (with_update == 0) or of the fused form of dion_ns_orthogonalize_update (with_update != 0, when
 // the shape fuses) over synthetic, never dereferenced addresses and checks it as every real call
 // is checked before its first launch.  audit_ws_bytes > 0 checks against a workspace of that size
 // instead of the size the plan was laid out for.
-extern "C" int dion_ns_plan_audit(int batch, int rows, int cols, int in_dtype, int n_iters, int flags,
-                                  int gram_reset, int with_update, int x_dtype, int mats_per_ptr,
-                                  size_t audit_ws_bytes) {
+static int plan_audit(int batch, int rows, int cols, int in_dtype, int n_iters, int flags, int gram_reset,
+                      int with_update, int x_dtype, int mats_per_ptr, size_t audit_ws_bytes, bool prepared) {
   if (batch <= 0 || rows <= 0 || cols <= 0 || n_iters < 0 || n_iters > 16 || mats_per_ptr <= 0)
     return fail(DION_E_INVALID, "dion_ns_plan_audit: bad size");
   if (int rc = check_state_dtype("dion_ns_plan_audit", "x_dtype", x_dtype)) return rc;
@@ -847,6 +985,8 @@ extern "C" int dion_ns_plan_audit(int batch, int rows, int cols, int in_dtype, i
   void* in = base;
   void* out = base + gap;
   void* ws = base + 2 * gap;
+  const float* sumsq = prepared ? (const float*)(base + 3 * gap + (gap >> 1)) : nullptr;
+  const int sumsq_blocks = prepared ? (int)((int64_t)rows * cols / 4096) : 0;
   NsCall call;
   std::vector<uint64_t> xp;
   PostSpec ps;
@@ -860,11 +1000,26 @@ extern "C" int dion_ns_plan_audit(int batch, int rows, int cols, int in_dtype, i
     ps = {xp.data(), x_dtype, n_ptrs, mats_per_ptr, (const float*)(base + 3 * gap), 1.0f, nullptr, 0.0f, 0};
   }
   if (int rc = ns_build(in, in_dtype, fused ? nullptr : out, batch, rows, cols, coeffs, n_iters, 1.0f, 0.0f, flags,
-                        gram_reset, small ? nullptr : ws, ws_bytes, fused ? &ps : nullptr, call))
+                        gram_reset, small ? nullptr : ws, ws_bytes, fused ? &ps : nullptr, call, sumsq,
+                        sumsq_blocks))
     return rc;
   if (audit_ws_bytes > 0 && call.ws_lo) call.ws_hi = call.ws_lo + audit_ws_bytes;
   if (int rc = ns_audit(call)) return rc;
-  return (int)call.steps.size();
+  return call.n_steps;
+}
+
+extern "C" int dion_ns_plan_audit(int batch, int rows, int cols, int in_dtype, int n_iters, int flags,
+                                  int gram_reset, int with_update, int x_dtype, int mats_per_ptr,
+                                  size_t audit_ws_bytes) {
+  return plan_audit(batch, rows, cols, in_dtype, n_iters, flags, gram_reset, with_update, x_dtype, mats_per_ptr,
+                    audit_ws_bytes, false);
+}
+
+extern "C" int dion_ns_plan_audit_prepared(int batch, int rows, int cols, int n_iters, int flags, int gram_reset,
+                                           int with_update, int x_dtype, int mats_per_ptr,
+                                           size_t audit_ws_bytes) {
+  return plan_audit(batch, rows, cols, DION_BF16, n_iters, flags, gram_reset, with_update, x_dtype, mats_per_ptr,
+                    audit_ws_bytes, true);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -906,6 +1061,45 @@ extern "C" int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t
     HIP_TRY(launch_muon_pre(g, dt(g_dtype), m, dt(m_dtype), (bf16_t*)U + (int64_t)i0 * numel, c, numel, mu,
                             nesterov, vec, (hipStream_t)stream),
             "dion_muon_pre");
+  }
+  return DION_OK;
+}
+
+extern "C" int dion_muon_pre_sumsq_blocks(int rows, int cols) {
+  if (rows <= 0 || cols <= 0 || ((int64_t)rows * cols) % 4096 || rows % 64 || cols % 64) return 0;
+  const int64_t b = (int64_t)rows * cols / 4096;
+  return b > 0x7fffffff ? 0 : (int)b;
+}
+
+extern "C" int dion_muon_pre_prepared(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int m_dtype,
+                                      void* U, float* sumsq, int n, int mats_per_ptr, int rows, int cols, float mu,
+                                      int nesterov, void* stream) {
+  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0)
+    return fail(DION_E_INVALID, "dion_muon_pre_prepared: bad size");
+  if (int rc = check_state_dtype("dion_muon_pre_prepared", "m_dtype", m_dtype)) return rc;
+  if (g_dtype != DION_BF16 && g_dtype != DION_F32) return fail(DION_E_INVALID, "dion_muon_pre_prepared: g_dtype");
+  if (n == 0 || rows == 0 || cols == 0) return DION_OK;
+  if (!G_ptrs || !M_ptrs || !U || !sumsq) return fail(DION_E_INVALID, "dion_muon_pre_prepared: null argument");
+  const int blocks = dion_muon_pre_sumsq_blocks(rows, cols);
+  if (blocks == 0)
+    return fail(DION_E_INVALID, "dion_muon_pre_prepared: rows and cols (%d, %d) must be multiples of 64", rows, cols);
+  const int64_t mat = (int64_t)rows * cols;
+  if ((int64_t)mats_per_ptr * blocks > 0x7fffffff || (int64_t)n * mats_per_ptr > 0x7fffffff)
+    return fail(DION_E_INVALID, "dion_muon_pre_prepared: too many matrices per parameter");
+  if (!table_aligned(G_ptrs, n) || !table_aligned(M_ptrs, n) || !aligned16((uint64_t)U))
+    return fail(DION_E_INVALID, "dion_muon_pre_prepared: pointers must be 16-byte aligned");
+  const int chunk = ptr_chunk(mats_per_ptr);
+  if (chunk == 0) return fail(DION_E_INVALID, "dion_muon_pre_prepared: mats_per_ptr %d > 65535", mats_per_ptr);
+  for (int c0 = 0; c0 < n; c0 += chunk) {
+    const int c = (n - c0) < chunk ? (n - c0) : chunk;
+    PtrTab G, M;
+    fill_tab(G, G_ptrs + c0, c);
+    fill_tab(M, M_ptrs + c0, c);
+    const int64_t first = (int64_t)c0 * mats_per_ptr;
+    HIP_TRY(launch_muon_pre_prepared(G, dt(g_dtype), M, dt(m_dtype), (bf16_t*)U + first * mat,
+                                     sumsq + first * blocks, c, mats_per_ptr, rows, cols, mu, nesterov,
+                                     (hipStream_t)stream),
+            "dion_muon_pre_prepared");
   }
   return DION_OK;
 }

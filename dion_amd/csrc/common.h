@@ -189,7 +189,20 @@ struct GemmParams {
   int xcd_interleave;  // set by the launcher: tile list dealt to the XCDs in interleaved 32-tile chunks
   float alpha, beta;
   float diag;        // added to C[i][i] (global diagonal); used with tri to fold a*I into B
+  // Optional per-matrix factor of the product, read on the device: matrix b is scaled by
+  // alpha * scale_vec[b] (scale_pow == 1) or alpha * scale_vec[b]^2 (scale_pow == 2).  This is how the
+  // Frobenius normalisation of an orthogonalization input is folded into its first two GEMMs
+  // (A = s^2 U U^T, X' = s B U) instead of being a pass over U.
+  const float* scale_vec;
+  int scale_pow;
 };
+
+// alpha of matrix b of a launch (see GemmParams::scale_vec)
+__device__ __forceinline__ float gemm_alpha(const GemmParams& p, int b) {
+  if (!p.scale_vec) return p.alpha;
+  const float s = p.scale_vec[b];
+  return p.alpha * (p.scale_pow == 2 ? s * s : s);
+}
 
 // Returns hipSuccess or the launch error; the tile configuration is picked by shape.
 hipError_t launch_gemm_nt(const GemmParams& p, hipStream_t stream);

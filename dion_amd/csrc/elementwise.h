@@ -20,6 +20,9 @@ hipError_t launch_ns_small(const void* in, int in_dtype, bf16_t* out, int batch,
 hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t numel,
                                 float norm_scale, float eps, float* partial, int nblk,
                                 float* inv_norm, hipStream_t st);
+// inv_norm[b] = 1 / (sqrt(sum of partial[b][0..nblk)) * norm_scale + eps), fixed summation order.
+hipError_t launch_norm_finalize(const float* partial, int nblk, int batch, float norm_scale, float eps,
+                                float* inv_norm, hipStream_t st);
 hipError_t launch_ns_prepare(const void* in, int in_dtype, int batch, int R, int C,
                              const float* inv_norm, bf16_t* same, int Rp, int Cp, int ld_same,
                              int64_t stride_same, bf16_t* trans, int ld_trans, int64_t stride_trans,
@@ -30,6 +33,13 @@ hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* d
 // 1 = fp32, like the gradient / update dtypes.
 hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, bf16_t* U, int n,
                            int64_t numel, float mu, int nesterov, bool vec, hipStream_t st);
+// muon_pre for matrices that go to the orthogonalization as they are written: U [n * mats][min][max] with
+// the short side along rows (a tall matrix is written transposed) plus sumsq [n * mats][rows * cols / 4096]
+// partial sums of squares.  rows, cols multiples of 64, rows * cols of 4096, all pointers 16-byte aligned,
+// numel / 4096 <= 2^31 - 1 and n * mats <= 65535 (checked by the caller).
+hipError_t launch_muon_pre_prepared(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, bf16_t* U,
+                                    float* sumsq, int n, int mats, int rows, int cols, float mu,
+                                    int nesterov, hipStream_t st);
 hipError_t launch_muon_post(const PtrTab& X, int x_dtype, const void* U, int u_dtype, int n, int64_t numel,
                             int cols, const float* row_scale, const float* lr_dev, const float* adj_lr_dev,
                             float adj_ratio, const float* wd_dev, float wd_host, int cautious, bool vec,

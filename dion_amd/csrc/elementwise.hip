@@ -90,13 +90,22 @@ __global__ __launch_bounds__(256) void sumsq_partial_kernel(const T* __restrict_
   if (threadIdx.x == 0) partial[(int64_t)b * nblk + blockIdx.x] = s;
 }
 
-__global__ __launch_bounds__(64) void norm_finalize_kernel(const float* __restrict__ partial, int nblk,
-                                                           float norm_scale, float eps,
-                                                           float* __restrict__ inv_norm) {
+__global__ __launch_bounds__(256) void norm_finalize_kernel(const float* __restrict__ partial, int nblk,
+                                                            float norm_scale, float eps,
+                                                            float* __restrict__ inv_norm) {
+  // Fixed summation order: thread t adds partials t, t + 256, ... (four independent running sums,
+  // so four loads are in flight), then the block sum.
+  __shared__ float red[16];
   const int b = blockIdx.x;
-  float s = 0.f;
-  for (int i = threadIdx.x; i < nblk; i += 64) s += partial[(int64_t)b * nblk + i];
-  s = wave_sum(s);
+  const float* src = partial + (int64_t)b * nblk;
+  float s4[4] = {0.f, 0.f, 0.f, 0.f};
+  int i = threadIdx.x;
+  for (; i + 3 * 256 < nblk; i += 4 * 256) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s4[j] += src[i + j * 256];
+  }
+  for (int j = 0; i < nblk; i += 256, ++j) s4[j] += src[i];
+  const float s = block_sum((s4[0] + s4[1]) + (s4[2] + s4[3]), red);
   if (threadIdx.x == 0) inv_norm[b] = 1.0f / (sqrtf(s) * norm_scale + eps);
 }
 
@@ -204,8 +213,13 @@ hipError_t launch_frobenius_inv(const void* in, int in_dtype, int batch, int64_t
     if (vec) SUMSQ_LAUNCH(float, true); else SUMSQ_LAUNCH(float, false);
   }
 #undef SUMSQ_LAUNCH
-  hipLaunchKernelGGL(norm_finalize_kernel, dim3(batch), dim3(64), 0, st, partial, nblk, norm_scale,
-                     eps, inv_norm);
+  return launch_norm_finalize(partial, nblk, batch, norm_scale, eps, inv_norm, st);
+}
+
+hipError_t launch_norm_finalize(const float* partial, int nblk, int batch, float norm_scale, float eps,
+                                float* inv_norm, hipStream_t st) {
+  hipLaunchKernelGGL(norm_finalize_kernel, dim3(batch), dim3(256), 0, st, partial, nblk, norm_scale, eps,
+                     inv_norm);
   return hipGetLastError();
 }
 
@@ -247,9 +261,15 @@ hipError_t launch_unpad(const bf16_t* src, int64_t src_stride, int ld, bf16_t* d
 // ------------------------------------------------------------------------------------------
 // Muon pre: momentum + Nesterov + bf16 cast, list-of-parameters in, one arena out.
 // ------------------------------------------------------------------------------------------
-template <typename GT, typename MT, bool VEC>
+// SUMSQ (VEC only, one tile per workgroup): the workgroup also writes the sum of squares of the 4096
+// bf16 values it stored, sumsq[p * gridDim.x + blockIdx.x] -- partial sums of ||U||_F^2 per matrix when
+// a matrix is a whole number of tiles.
+template <typename GT, typename MT, bool VEC, bool SUMSQ = false>
 __global__ __launch_bounds__(256) void muon_pre_kernel(PtrTab G, PtrTab M, bf16_t* __restrict__ U,
-                                                       int64_t numel, float mu, int nesterov) {
+                                                       int64_t numel, float mu, int nesterov,
+                                                       float* __restrict__ sumsq = nullptr) {
+  __shared__ float red[16];
+  float ss = 0.f;
   const int p = blockIdx.y;
   const GT* __restrict__ g = (const GT*)G.p[p];
   MT* __restrict__ m = (MT*)M.p[p];
@@ -281,7 +301,18 @@ __global__ __launch_bounds__(256) void muon_pre_kernel(PtrTab G, PtrTab M, bf16_
         }
         st_store8<MT>(m, i, mv[c]);
         st_store8<bf16_t>(u, i, uv);
+        if (SUMSQ) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float r = st_round<bf16_t>(uv[e]);
+            ss += r * r;
+          }
+        }
       }
+    }
+    if (SUMSQ) {
+      ss = block_sum(ss, red);
+      if (threadIdx.x == 0) sumsq[(int64_t)p * gridDim.x + blockIdx.x] = ss;
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
@@ -290,6 +321,70 @@ __global__ __launch_bounds__(256) void muon_pre_kernel(PtrTab G, PtrTab M, bf16_
       st_store<MT>(m, i, mv);
       u[i] = f32_to_bf16(nesterov ? __fadd_rn(__fmul_rn(mv, mu), gv) : mv);
     }
+  }
+}
+
+// The same update for tall matrices (rows > cols) whose orthogonalization input is wanted with the short
+// side along rows: U[p][mat] is written transposed, [cols][rows].  One 64 x 64 tile per workgroup, staged
+// through LDS so that G / M rows are read and U^T rows written as whole 128-byte (bf16) runs; every thread
+// handles two 8-element chunks, like the flat kernel.  sumsq[(p * mats + mat) * tiles + tile]: sum of
+// squares of the tile's bf16 values, tile = (row tile) * (cols / 64) + column tile.
+// Needs rows % 64 == 0, cols % 64 == 0, 16-byte aligned pointers.
+template <typename GT, typename MT>
+__global__ __launch_bounds__(256) void muon_pre_transposed_kernel(PtrTab G, PtrTab M, bf16_t* __restrict__ U,
+                                                                  int mats, int rows, int cols, float mu,
+                                                                  int nesterov, float* __restrict__ sumsq) {
+  __shared__ __attribute__((aligned(16))) bf16_t tile[64][72];
+  __shared__ float red[16];
+  const int p = blockIdx.z / mats, mat = blockIdx.z - p * mats;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int64_t mat_off = (int64_t)mat * rows * cols;
+  const GT* __restrict__ g = (const GT*)G.p[p] + mat_off;
+  MT* __restrict__ m = (MT*)M.p[p] + mat_off;
+  bf16_t* __restrict__ ut = U + ((int64_t)p * mats + mat) * rows * cols;
+  const int chunk = threadIdx.x & 7, rr = threadIdx.x >> 3;  // 8 chunks x 32 rows per pass
+  float gv[2][8], mv[2][8];
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int64_t i8 = ((int64_t)(r0 + rr + pass * 32) * cols + c0 + chunk * 8) >> 3;
+    st_load8<GT>(g, i8, gv[pass]);
+    st_load8<MT>(m, i8, mv[pass]);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int64_t i8 = ((int64_t)(r0 + rr + pass * 32) * cols + c0 + chunk * 8) >> 3;
+    float uv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      mv[pass][e] = __fadd_rn(__fmul_rn(mv[pass][e], mu), gv[pass][e]);
+      uv[e] = nesterov ? __fadd_rn(__fmul_rn(mv[pass][e], mu), gv[pass][e]) : mv[pass][e];
+    }
+    st_store8<MT>(m, i8, mv[pass]);
+    uint4 o;
+    o.x = pack_bf16x2(uv[0], uv[1]);
+    o.y = pack_bf16x2(uv[2], uv[3]);
+    o.z = pack_bf16x2(uv[4], uv[5]);
+    o.w = pack_bf16x2(uv[6], uv[7]);
+    *(uint4*)&tile[rr + pass * 32][chunk * 8] = o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float r = st_round<bf16_t>(uv[e]);
+      ss += r * r;
+    }
+  }
+  ss = block_sum(ss, red);  // (its barriers also order the tile writes before the reads below)
+  if (threadIdx.x == 0)
+    sumsq[((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x] = ss;
+  // transposed: thread -> (U^T row = column rr + 32 * pass of the tile, 8 consecutive source rows)
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int col = rr + pass * 32;
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      w[e] = (uint32_t)tile[chunk * 8 + 2 * e][col] | ((uint32_t)tile[chunk * 8 + 2 * e + 1][col] << 16);
+    *(uint4*)(ut + (int64_t)(c0 + col) * rows + r0 + chunk * 8) = make_uint4(w[0], w[1], w[2], w[3]);
   }
 }
 
@@ -322,6 +417,37 @@ hipError_t launch_muon_pre(const PtrTab& G, int g_dtype, const PtrTab& M, int m_
   }
 #undef PRE_LAUNCH_M
 #undef PRE_LAUNCH
+  return hipGetLastError();
+}
+
+hipError_t launch_muon_pre_prepared(const PtrTab& G, int g_dtype, const PtrTab& M, int m_dtype, bf16_t* U,
+                                    float* sumsq, int n, int mats, int rows, int cols, float mu,
+                                    int nesterov, hipStream_t st) {
+  if (rows > cols) {
+    dim3 grid(cols / 64, rows / 64, n * mats);
+#define PRET_LAUNCH(GT, MT)                                                                            \
+  hipLaunchKernelGGL((muon_pre_transposed_kernel<GT, MT>), grid, dim3(256), 0, st, G, M, U, mats, rows, cols, \
+                     mu, nesterov, sumsq)
+    if (g_dtype == 0) {
+      if (m_dtype == 0) PRET_LAUNCH(bf16_t, bf16_t); else PRET_LAUNCH(bf16_t, float);
+    } else {
+      if (m_dtype == 0) PRET_LAUNCH(float, bf16_t); else PRET_LAUNCH(float, float);
+    }
+#undef PRET_LAUNCH
+    return hipGetLastError();
+  }
+  // one 4096-element tile per workgroup, so that blockIdx.x is the tile number within the parameter
+  const int64_t numel = (int64_t)mats * rows * cols;
+  dim3 grid((unsigned)(numel / 4096), n);
+#define PRES_LAUNCH(GT, MT)                                                                             \
+  hipLaunchKernelGGL((muon_pre_kernel<GT, MT, true, true>), grid, dim3(256), 0, st, G, M, U, numel, mu, \
+                     nesterov, sumsq)
+  if (g_dtype == 0) {
+    if (m_dtype == 0) PRES_LAUNCH(bf16_t, bf16_t); else PRES_LAUNCH(bf16_t, float);
+  } else {
+    if (m_dtype == 0) PRES_LAUNCH(float, bf16_t); else PRES_LAUNCH(float, float);
+  }
+#undef PRES_LAUNCH
   return hipGetLastError();
 }
 

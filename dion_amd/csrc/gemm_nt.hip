@@ -434,7 +434,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   // copy would be 8-byte pieces scattered over 32 rows per instruction, so it is staged through
   // LDS ([column][row], this wavefront's private slice) and stored as 16 bytes per lane with
   // 256-byte runs per row.
-  const float alpha = p.alpha, beta = p.beta;
+  const float alpha = gemm_alpha(p, b), beta = p.beta;
   const int row_base = ti * BM + wm * Cfg::WTM;
   const int col_base = tj * BN + wn * Cfg::WTN;
   const bool mirror = HAS_CT && !(p.tri && ti == tj);  // a diagonal tile is its own mirror
@@ -816,6 +816,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
                         : p.C + (int64_t)b * p.strideC + (int64_t)row_base * ld_out + col_base;
     const __amdgpu_buffer_rsrc_t rs = bx_resource(out);
     const int lane_bytes = (rl * ld_out + rq * 8) * 2;
+    const float alpha = gemm_alpha(p, b);  // 1 unless a per-matrix factor rides on this launch
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       // chunk c: accumulator tiles t2 = 0, 1 side by side along the 128-byte lines
@@ -827,8 +828,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           uint2 pk;
-          pk.x = pack_bf16x2(a[g * 4 + 0], a[g * 4 + 1]);
-          pk.y = pack_bf16x2(a[g * 4 + 2], a[g * 4 + 3]);
+          pk.x = pack_bf16x2(alpha * a[g * 4 + 0], alpha * a[g * 4 + 1]);
+          pk.y = pack_bf16x2(alpha * a[g * 4 + 2], alpha * a[g * 4 + 3]);
           // 8-byte piece t2*8 + 2g + wh of line wl; XOR with the line pair number spreads the 32 lines of
           // a half wavefront over all 64 banks
           *(uint2*)(stg + wl * 128 + (((t2 * 8 + 2 * g + wh) ^ ((wl >> 1) & 15)) << 3)) = pk;

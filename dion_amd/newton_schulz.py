@@ -91,6 +91,37 @@ def orthogonalize_update(func, G: Tensor, epsilon, X, lr: Tensor, adj_ratio: flo
                                 gram=gram, gram_reset=reset)
 
 
+def _schedule_args(func, epsilon):
+    coeffs, norm_scale, default_eps, gram, reset = SCHEDULES[func]
+    eps = 0.0 if default_eps is None else _eps(epsilon, default_eps)
+    return coeffs, norm_scale, eps, gram, reset
+
+
+def accepts_prepared(func, batch: int, rows: int, cols: int) -> bool:
+    """True when the built-in operator ``func`` takes ``batch`` matrices of ``rows x cols`` in the prepared
+    form (``ops.muon_pre_prepared``)."""
+    if func not in SCHEDULES:
+        return False
+    coeffs, _s, _e, gram, _r = SCHEDULES[func]
+    return ops.ns_accepts_prepared(batch, rows, cols, len(coeffs), gram)
+
+
+@torch.no_grad()
+def orthogonalize_prepared(func, U: Tensor, sumsq: Tensor, rows: int, cols: int, epsilon) -> Tensor:
+    """``func(G, epsilon)`` for a built-in ``func`` on the prepared form of ``G``."""
+    coeffs, norm_scale, eps, gram, reset = _schedule_args(func, epsilon)
+    return ops.ns_orthogonalize_prepared(U, sumsq, rows, cols, coeffs, norm_scale, eps, gram=gram, gram_reset=reset)
+
+
+@torch.no_grad()
+def orthogonalize_update_prepared(func, U: Tensor, sumsq: Tensor, rows: int, cols: int, epsilon, X, lr: Tensor,
+                                  adj_ratio: float, weight_decay, cautious_wd: bool = False) -> None:
+    """``orthogonalize_update`` on the prepared form of ``G``."""
+    coeffs, norm_scale, eps, gram, reset = _schedule_args(func, epsilon)
+    ops.ns_orthogonalize_update_prepared(U, sumsq, rows, cols, X, coeffs, norm_scale, eps, lr, adj_ratio,
+                                         weight_decay, cautious_wd, gram=gram, gram_reset=reset)
+
+
 # The reference exposes Triton-backed twins of the two schedules; here there is one
 # implementation, so the names resolve to it.
 newton_schulz_triton = zeropower_via_newtonschulz5

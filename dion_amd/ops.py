@@ -248,6 +248,69 @@ def ns_orthogonalize_update(G: Tensor, X: List[Tensor], coeffs: Sequence[Sequenc
                                            _stream_handle(G.device)), "ns_orthogonalize_update")
 
 
+def ns_accepts_prepared(batch: int, rows: int, cols: int, n_iters: int, gram: bool = False) -> bool:
+    """True when ``batch`` matrices of ``rows x cols`` can go to the orthogonalization as ``muon_pre_prepared``
+    writes them (whole GEMM tiles, not the small-matrix kernel, at least one iteration)."""
+    lib = _lib.load()
+    return bool(lib.dion_ns_accepts_prepared(int(batch), int(rows), int(cols), DION_NS_GRAM if gram else 0,
+                                             int(n_iters)))
+
+
+def _check_prepared(U: Tensor, sumsq: Tensor, rows: int, cols: int) -> Tuple[int, int]:
+    _check_bf16(U, "U")
+    m, n = min(rows, cols), max(rows, cols)
+    if U.ndim != 3 or U.shape[1] != m or U.shape[2] != n or not U.is_contiguous():
+        raise ValueError(f"a prepared input of {rows} x {cols} matrices is a contiguous [batch, {m}, {n}] tensor, "
+                         f"got {tuple(U.shape)}")
+    batch = U.shape[0]
+    if (sumsq.dtype != torch.float32 or sumsq.ndim != 2 or sumsq.shape[0] != batch or not sumsq.is_contiguous()
+            or sumsq.device != U.device):
+        raise ValueError("sumsq must be a contiguous float32 [batch, blocks] tensor on the device of U")
+    return batch, sumsq.shape[1]
+
+
+def ns_orthogonalize_prepared(U: Tensor, sumsq: Tensor, rows: int, cols: int, coeffs, norm_scale: float,
+                              epsilon: float, gram: bool = False, gram_reset: int = 0) -> Tensor:
+    """``ns_orthogonalize`` of the matrices ``muon_pre_prepared`` wrote: ``U [batch, min, max]`` holds them
+    with the short side along rows and unnormalised, ``sumsq [batch, blocks]`` partial sums of their squares.
+    Returns ``[batch, rows, cols]`` bf16.  The Frobenius normalisation rides on the first two GEMMs."""
+    batch, blocks = _check_prepared(U, sumsq, rows, cols)
+    out = torch.empty(batch, rows, cols, dtype=torch.bfloat16, device=U.device)
+    carr, n_iters = _flat_coeffs(coeffs)
+    flags = DION_NS_GRAM if gram else 0
+    lib = _lib.load()
+    ws = _workspace(U.device, lib.dion_ns_workspace_bytes(batch, rows, cols, flags))
+    check(lib.dion_ns_orthogonalize_prepared(U.data_ptr(), sumsq.data_ptr(), blocks, out.data_ptr(), batch, rows,
+                                             cols, carr, n_iters, float(norm_scale), float(epsilon), flags,
+                                             int(gram_reset), ws.data_ptr(), ws.numel(), _stream_handle(U.device)),
+          "ns_orthogonalize_prepared")
+    return out
+
+
+def ns_orthogonalize_update_prepared(U: Tensor, sumsq: Tensor, rows: int, cols: int, X: List[Tensor], coeffs,
+                                     norm_scale: float, epsilon: float, lr: Tensor, adj_ratio: float, weight_decay,
+                                     cautious_wd: bool = False, gram: bool = False, gram_reset: int = 0) -> None:
+    """``ns_orthogonalize_update`` on a prepared input (see ``ns_orthogonalize_prepared``): the update of
+    every ``X[i]`` (``[mats, rows, cols]``) rides on the last GEMM."""
+    batch, blocks = _check_prepared(U, sumsq, rows, cols)
+    n = len(X)
+    if n == 0 or batch % n:
+        raise ValueError(f"{batch} matrices do not divide over {n} parameters")
+    mats_per_ptr = batch // n
+    xp, xcode = _state_ptrs(X, "X", mats_per_ptr * rows * cols)
+    lr_p, wd_p, wd_h = _scalar_args(lr, weight_decay, U.device)
+    carr, n_iters = _flat_coeffs(coeffs)
+    flags = DION_NS_GRAM if gram else 0
+    lib = _lib.load()
+    ws = _workspace(U.device, lib.dion_ns_update_workspace_bytes(batch, rows, cols, flags, n_iters))
+    check(lib.dion_ns_orthogonalize_update_prepared(U.data_ptr(), sumsq.data_ptr(), blocks, xp, xcode, n,
+                                                    mats_per_ptr, rows, cols, carr, n_iters, float(norm_scale),
+                                                    float(epsilon), flags, int(gram_reset), lr_p,
+                                                    float(adj_ratio), wd_p, wd_h, int(bool(cautious_wd)),
+                                                    ws.data_ptr(), ws.numel(), _stream_handle(U.device)),
+          "ns_orthogonalize_update_prepared")
+
+
 # ---------------------------------------------------------------------------------------------
 # optimizer-step kernels on lists of same-shape parameters
 # ---------------------------------------------------------------------------------------------
@@ -295,6 +358,32 @@ def muon_pre(G: List[Tensor], M: List[Tensor], momentum: float, nesterov: bool) 
     check(lib.dion_muon_pre(gp, _dtype_code(G[0], "G"), mp, mcode, U.data_ptr(), n, numel, float(momentum),
                             int(bool(nesterov)), _stream_handle(U.device)), "muon_pre")
     return U
+
+
+def muon_pre_prepared(G: List[Tensor], M: List[Tensor], momentum: float, nesterov: bool, mats: int, rows: int,
+                      cols: int) -> Tuple[Tensor, Tensor]:
+    """``muon_pre`` for parameters made of ``mats`` matrices of ``rows x cols`` each, writing the
+    orthogonalization input the way the iteration carries it: returns ``(U, sumsq)`` with ``U [N * mats,
+    min(rows, cols), max(rows, cols)]`` bf16 (a tall matrix transposed) and ``sumsq [N * mats, blocks]`` fp32
+    partial sums of squares of each matrix.  ``M`` is updated exactly as by ``muon_pre``."""
+    n = len(G)
+    assert n == len(M) and n > 0
+    numel = M[0].numel()
+    if numel != mats * rows * cols:
+        raise ValueError(f"parameters of {numel} elements are not {mats} matrices of {rows} x {cols}")
+    gp = _list_ptrs(G, "G", G[0].dtype, numel)
+    mp, mcode = _state_ptrs(M, "M", numel)
+    lib = _lib.load()
+    blocks = lib.dion_muon_pre_sumsq_blocks(rows, cols)
+    if blocks == 0:
+        raise ValueError(f"muon_pre_prepared: {rows} x {cols} matrices are not whole 64 x 64 tiles")
+    dev = M[0].device
+    U = torch.empty((n * mats, min(rows, cols), max(rows, cols)), dtype=torch.bfloat16, device=dev)
+    sumsq = torch.empty((n * mats, blocks), dtype=torch.float32, device=dev)
+    check(lib.dion_muon_pre_prepared(gp, _dtype_code(G[0], "G"), mp, mcode, U.data_ptr(), sumsq.data_ptr(), n, mats,
+                                     rows, cols, float(momentum), int(bool(nesterov)), _stream_handle(dev)),
+          "muon_pre_prepared")
+    return U, sumsq
 
 
 def muon_post(X: List[Tensor], U: Tensor, lr: Tensor, adj_ratio: float, weight_decay, cautious_wd: bool = False,

@@ -18,6 +18,7 @@ import torch
 from torch import Tensor
 
 from . import global_scope, ops
+from . import newton_schulz as ns
 from .optim_base import OrthoOptimizer, adjust_lr_ratio, split_lr_scales
 
 
@@ -55,6 +56,9 @@ class _MomentumOrtho(OrthoOptimizer):
     _normalize = False
     # Muon only: run orthogonalization and update as one library call (False: the two-call sequence)
     fused_update = True
+    # hand the orthogonalization its input as the momentum kernel writes it (False: the arena in the
+    # parameters' layout, normalised and transposed by passes of the orthogonalization call)
+    prepared_input = True
 
     def _shape_group_phases(self, group: dict, params: List[Tensor]):
         """Generator: [momentum / cast] yield [orthogonalization GEMMs] yield [normalise / update]."""
@@ -81,11 +85,35 @@ class _MomentumOrtho(OrthoOptimizer):
         M = [s["momentum"] for s in states]
         eps = float(group["epsilon"])
 
+        ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
+        # Matrices that fill whole GEMM tiles reach the orthogonalization as the momentum kernel writes them:
+        # short side along rows, unnormalised, with the partial sums of the Frobenius norm from the same pass
+        # (no separate norm / scale / transpose pass over the arena; the factor rides on the first two GEMMs).
+        flat3d = flatten and len(shape) >= 3
+        prepared = (self.prepared_input and split_sizes is None and not flat3d and not self._custom_ns
+                    and ns.accepts_prepared(self._newton_schulz_func, n * mats, rows, cols)
+                    and all(t.data_ptr() % 16 == 0 for t in G + M))
+        if prepared:
+            U, sumsq = ops.muon_pre_prepared(G, M, group["mu"], group["nesterov"], mats, rows, cols)
+            yield
+            _note_stream(U)
+            _note_stream(sumsq)
+            func = self._newton_schulz_func
+            if not self._normalize and self.fused_update:
+                ns.orthogonalize_update_prepared(func, U, sumsq, rows, cols, eps, X, group["lr"], ratio,
+                                                 group["weight_decay"], group["cautious_wd"])
+                return
+            O = ns.orthogonalize_prepared(func, U, sumsq, rows, cols, eps)
+            del U, sumsq
+            yield
+            _note_stream(O)
+            self._normalize_and_update(group, X, states, O, n, mats, rows, cols, ratio, None)
+            return
+
         U = ops.muon_pre(G, M, group["mu"], group["nesterov"])  # [n, *shape] bf16
         yield
         _note_stream(U)
 
-        ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
         if not self._normalize and split_sizes is None and self.fused_update:
             # Muon proper: the update consumes the orthogonalized matrices where the last GEMM
             # produces them (same result as the two calls below, bit for bit)
@@ -105,7 +133,10 @@ class _MomentumOrtho(OrthoOptimizer):
         del U
         yield
         _note_stream(O)
+        self._normalize_and_update(group, X, states, O, n, mats, rows, cols, ratio, split_sizes)
 
+    def _normalize_and_update(self, group, X, states, O, n, mats, rows, cols, ratio, split_sizes) -> None:
+        """NorMuon's neuron-wise normalisation (when this class normalises) and the update pass."""
         row_scale = None
         if self._normalize:
             V = [s["variance_neuron"] for s in states]

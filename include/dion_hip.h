@@ -131,6 +131,46 @@ int dion_ns_orthogonalize_update(const void* in, int in_dtype, const uint64_t* X
                                  void* workspace, size_t workspace_bytes, void* stream);
 
 /* --------------------------------------------------------------------------------------------
+ * Orthogonalization of a "prepared" input: the producer of the input (dion_muon_pre_prepared) has
+ * already written it in the layout the iteration carries -- bf16 [batch, min(rows, cols),
+ * max(rows, cols)], short side along rows, i.e. a tall matrix transposed -- and has left partial
+ * sums of its squares per matrix.  The Frobenius normalisation X0 = in / (||in||_F * norm_scale + eps)
+ * (dion/polar_express.py:30-35, dion/newton_schulz_triton.py:508-513) then needs no pass over the
+ * input: the factor rides on the first two GEMMs (A = s^2 in in^T, X' = s B in), computed on the
+ * device from the partial sums.  rows / cols describe the caller's matrices (`out`, the
+ * parameters), as in dion_ns_orthogonalize; all other arguments as there.
+ *   in     bf16 [batch, m, n], m = min(rows, cols), n = max(rows, cols), 16-byte aligned
+ *   sumsq  fp32 [batch, sumsq_blocks]; the sum of row b is ||in[b]||_F^2
+ * Taken only when dion_ns_accepts_prepared() returns 1: rows and cols multiples of the GEMM tile
+ * (no padding), rows * cols a multiple of 4096, at least one iteration, more than 64 rows or columns
+ * on the short side, at most 65535 matrices; DION_E_INVALID otherwise (use dion_ns_orthogonalize).
+ * Results differ from dion_ns_orthogonalize in the last bf16 bit (X0 is not rounded to bf16 once
+ * more before the first products).
+ * ------------------------------------------------------------------------------------------ */
+int dion_ns_accepts_prepared(int batch, int rows, int cols, int flags, int n_iters);
+int dion_ns_orthogonalize_prepared(const void* in, const float* sumsq, int sumsq_blocks, void* out, int batch,
+                                   int rows, int cols, const float* coeffs, int n_iters, float norm_scale,
+                                   float eps, int flags, int gram_reset, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+/* dion_ns_orthogonalize_update on a prepared input (the update always rides on the last GEMM:
+ * every shape that takes a prepared input fuses).  Workspace from dion_ns_update_workspace_bytes. */
+int dion_ns_orthogonalize_update_prepared(const void* in, const float* sumsq, int sumsq_blocks,
+                                          const uint64_t* X_ptrs, int x_dtype, int n_ptrs, int mats_per_ptr,
+                                          int rows, int cols, const float* coeffs, int n_iters,
+                                          float norm_scale, float eps, int flags, int gram_reset,
+                                          const float* lr_dev, float adj_ratio, const float* wd_dev,
+                                          float wd_host, int cautious, void* workspace,
+                                          size_t workspace_bytes, void* stream);
+/* dion_ns_plan_audit for the prepared form (host only, no device work). */
+int dion_ns_plan_audit_prepared(int batch, int rows, int cols, int n_iters, int flags, int gram_reset,
+                                int with_update, int x_dtype, int mats_per_ptr, size_t audit_ws_bytes);
+
+/* Tile edge (128 or 256) the GEMM launcher picks for `batch` products of an m x n result
+ * (symmetric != 0: an m x m symmetric product, upper tiles only).  Lets a benchmark count executed
+ * FLOP with the library's own rule.  No counterpart in the reference. */
+int dion_gemm_tile_edge(int batch, int m, int n, int symmetric);
+
+/* --------------------------------------------------------------------------------------------
  * Memory-bound fused kernels of the optimizer step.
  * Optimizer state -- parameters X, momentum M, second moments V -- is fp32 or bf16 in memory, as the
  * reference keeps it in the parameter's dtype (dion/megabatch_base.py:198-203, dion/normuon.py:122):
@@ -146,6 +186,24 @@ int dion_ns_orthogonalize_update(const void* in, int in_dtype, const uint64_t* X
  * dion/megabatch_base.py:872. */
 int dion_muon_pre(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int m_dtype, void* U,
                   int n, int64_t numel, float mu, int nesterov, void* stream);
+
+/* dion_muon_pre for matrices that take a prepared orthogonalization input: same momentum update,
+ * but U is written in the layout the iteration carries and the Frobenius norm's partial sums come
+ * out of the same pass (they are in registers anyway).
+ *   G_ptrs / M_ptrs: n pointers, each to mats_per_ptr dense [rows, cols] matrices
+ *   U      bf16 [n * mats_per_ptr, min(rows, cols), max(rows, cols)]: matrix as it lies when
+ *          rows <= cols, transposed when rows > cols
+ *   sumsq  fp32 [n * mats_per_ptr, dion_muon_pre_sumsq_blocks(rows, cols)]: sums of squares of the bf16
+ *          values written, over 4096-element pieces of each matrix, in a fixed order
+ * rows and cols multiples of 64, all pointers 16-byte aligned (DION_E_INVALID otherwise).
+ * M is bit-identical to dion_muon_pre's, U holds the same values.
+ * Replaces muon_update_pre_orthogonalize (dion/muon.py:284-311), the torch.stack of
+ * dion/megabatch_base.py:872, the transposition of tall inputs and the norm of
+ * dion/newton_schulz_triton.py:508-513 / dion/polar_express.py:30-35. */
+int dion_muon_pre_sumsq_blocks(int rows, int cols);
+int dion_muon_pre_prepared(const uint64_t* G_ptrs, int g_dtype, const uint64_t* M_ptrs, int m_dtype, void* U,
+                           float* sumsq, int n, int mats_per_ptr, int rows, int cols, float mu, int nesterov,
+                           void* stream);
 
 /* Weight decay + update for one shape group.
  *   X_i = (1 - lr wd) X_i - lr adj_ratio U[i]            (cautious == 0)

@@ -101,13 +101,6 @@ int main(void) {
       }
   }
   printf("O O^T - I: worst diagonal %.3e, worst off-diagonal %.3e\n", worst_diag, worst_off);
-  /* a refused call reports what was wrong instead of touching the device */
-  if (dion_ns_orthogonalize(d_in, DION_BF16, (char*)d_out + 2, BATCH, ROWS, COLS, pe, 5, 1.02f, 1e-6f, 0, 0, d_ws,
-                            ws_bytes, NULL) != DION_E_INVALID) {
-    fprintf(stderr, "a misaligned output pointer was not refused\n");
-    return 5;
-  }
-  printf("refused as expected: %s\n", dion_last_error());
   CHECK_HIP(hipFree(d_in));
   CHECK_HIP(hipFree(d_out));
   CHECK_HIP(hipFree(d_ws));

@@ -1,7 +1,7 @@
-"""The library called from a C program (tests/c_caller/ns_caller.c, built by dion_amd._build next to the
-library): dion_ns_orthogonalize and dion_ns_orthogonalize_static through nothing but the C header, the result
-checked in the program itself (rows orthonormal to the accuracy of five bf16 Polar-Express iterations, the two
-entry points bit-identical, a misaligned output refused).  The program runs as a child process."""
+"""The library called from a C program (tests/c_caller/ns_caller.c, built with the host C compiler by
+`python -m dion_amd._build --c-caller`): dion_ns_orthogonalize and dion_ns_orthogonalize_static through nothing
+but the C header, the result checked in the program itself (rows orthonormal to the accuracy of five bf16
+Polar-Express iterations, the two entry points bit-identical).  The program runs as a child process."""
 import os
 import subprocess
 
@@ -14,11 +14,16 @@ BIN = os.path.join(HERE, "c_caller", "ns_caller")
 @pytest.mark.gpu
 def test_c_program_orthogonalizes_through_the_c_abi():
     if not os.path.exists(BIN):
-        pytest.fail("tests/c_caller/ns_caller is not built: run python -m dion_amd._build")
+        import shutil
+
+        if shutil.which("gcc") is None:
+            pytest.skip("tests/c_caller/ns_caller is not built and gcc is not installed")
+        from dion_amd import _build
+
+        _build.build_c_caller(verbose=False)
     run = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
     print(run.stdout, run.stderr)
     assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
-    assert "refused as expected" in run.stdout and "16-byte" in run.stdout
 
 
 def test_header_is_valid_c11(tmp_path):

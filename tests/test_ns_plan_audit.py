@@ -106,3 +106,37 @@ def test_static_scratch_limit_is_checked_before_any_device_work():
     assert rc == -2
     msg = lib.dion_last_error().decode()
     assert str(_lib.DION_NS_STATIC_SCRATCH_BYTES) in msg and "caller workspace" in msg
+
+
+def _audit_prepared(lib, shape, n_iters=5, flags=0, with_update=0, x_dtype=F32, mats_per_ptr=1, ws=0, reset=2):
+    b, r, c = shape
+    return lib.dion_ns_plan_audit_prepared(b, r, c, n_iters, flags, reset, with_update, x_dtype, mats_per_ptr, ws)
+
+
+@pytest.mark.parametrize("shape", CONFIG_SHAPES + RAGGED_SHAPES)
+def test_prepared_input_plans(shape):
+    """The prepared form (input in the iteration's layout, norm partials from the caller): taken exactly by
+    the shapes that fill whole tiles, two launches shorter than the plain form (no norm pass over the input,
+    no prepare pass; one small launch turns the partial sums into the per-matrix factor), every launch
+    inside the call's buffers, the fused update included."""
+    lib = _lib.load()
+    b, r, c = shape
+    for flags in (0, GRAM):
+        takes = bool(lib.dion_ns_accepts_prepared(b, r, c, flags, 5))
+        whole = min(r, c) > 64 and r % 128 == 0 and c % 128 == 0
+        if takes:
+            assert whole, shape
+        if not whole:
+            assert not takes, shape
+        n = _audit_prepared(lib, shape, 5, flags)
+        if not takes:
+            assert n == -1 and "does not take a prepared input" in lib.dion_last_error().decode(), shape
+            continue
+        plain = _audit(lib, shape, 5, flags)
+        assert n == plain - 1, (shape, flags, n, plain)
+        assert _audit_prepared(lib, shape, 0, flags) == -1  # no iteration to carry the normalisation
+        for x_dtype in (F32, BF16):
+            assert _audit_prepared(lib, shape, 5, flags, with_update=1, x_dtype=x_dtype) > 0, \
+                (shape, lib.dion_last_error().decode())
+        # a workspace cut short is caught for this form too
+        assert _audit_prepared(lib, shape, 5, flags, ws=4096) == -1

@@ -86,3 +86,33 @@ def test_static_scratch_refuses_what_does_not_fit():
     assert "fixed" in msg and str(_lib.DION_NS_STATIC_SCRATCH_BYTES) in msg
     torch.cuda.synchronize()
     assert bool((out == 7.0).all()), "a refused call must not touch the output"
+
+
+@pytest.mark.gpu
+def test_static_entry_point_allocates_no_device_memory():
+    """Free device memory as the driver reports it (hipMemGetInfo) is the same before and after warm calls of
+    the entry point: nothing is allocated or freed, on any of the three kernel routes (tiled, padded,
+    LDS-resident).  Outputs are allocated before the reading is taken."""
+    lib = _lib.load()
+    torch.manual_seed(5)
+    cases = [(2, 256, 512), (1, 200, 136), (5, 64, 768)]
+    Gs = [torch.randn(shape, device=DEV).to(torch.bfloat16) for shape in cases]
+    outs = [torch.empty_like(G) for G in Gs]
+    carr, n = _coeffs(NS5_COEFFS)
+    st = torch.cuda.current_stream().cuda_stream
+
+    def call(G, out):
+        b, r, c = G.shape
+        _lib.check(lib.dion_ns_orthogonalize_static(G.data_ptr(), _lib.DION_BF16, out.data_ptr(), b, r, c, carr, n,
+                                                    1.0, 1e-7, 0, 0, st), "dion_ns_orthogonalize_static")
+
+    for G, out in zip(Gs, outs):  # warm: code objects loaded, the array's address resolved
+        call(G, out)
+    torch.cuda.synchronize()
+    free_before, _total = torch.cuda.mem_get_info()
+    for _ in range(3):
+        for G, out in zip(Gs, outs):
+            call(G, out)
+    torch.cuda.synchronize()
+    free_after, _total = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
