@@ -190,6 +190,7 @@ def test_custom_orthogonalization_keeps_the_two_call_sequence():
     pb = torch.nn.Parameter(pa.data.clone())
     oa = dion.Muon([pa], lr=0.02, newton_schulz_func=my_ns)
     ob = dion.Muon([pb], lr=0.02, use_polar_express=False)
+    ob.prepared_input = False  # the built-in operator on the arena in the parameters' layout, as my_ns gets it
     g = torch.randn(256, 512, device=DEV)
     pa.grad, pb.grad = g.clone(), g.clone()
     oa.step()
