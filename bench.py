@@ -357,8 +357,8 @@ def main() -> int:
         # the launch stream.  "executed" counts the MFMA work actually issued (upper-triangle tiles only
         # for the two symmetric products), "algorithmic" the full product.
         A = torch.empty(B, m, m, device=dev, dtype=torch.bfloat16)
-        tile = 256 if (m % 256 == 0 and n % 256 == 0) else 128
-        T = m // tile
+        # executed share of a symmetric product: upper tiles only, with the tile edge the library picks
+        T = m // lib.dion_gemm_tile_edge(B, m, m, 1)
         tri = (T + 1) / (2.0 * T)
         ms1 = time_kernel(lambda: lib.dion_ns_line_1(X.data_ptr(), A.data_ptr(), B, m, n, st))
         ms2 = time_kernel(lambda: lib.dion_ns_line_2(Bm.data_ptr(), A.data_ptr(), B, m, 1.0, 1.0, st))

@@ -66,6 +66,9 @@ SIGNATURES = {
     "dion_dion2_topk": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "dion_dion2_gather": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
                                   c_void_p, c_void_p]),
+    "dion_dion2_gather_sumsq_blocks": (c_int, [c_int, c_int, c_int, c_int]),
+    "dion_dion2_gather_prepared": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
+                                           c_void_p, c_void_p, c_void_p]),
     "dion_dion2_post": (c_int, [_u64p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float, c_void_p]),
     "dion_dion2_index_map": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),

@@ -1272,6 +1272,49 @@ extern "C" int dion_dion2_gather(const uint64_t* M_ptrs, int m_dtype, int n, int
   return DION_OK;
 }
 
+extern "C" int dion_dion2_gather_sumsq_blocks(int rows, int cols, int select_dim, int k) {
+  if (rows <= 0 || cols <= 0 || k <= 0 || (select_dim != -2 && select_dim != -1)) return 0;
+  if (select_dim == -2) return (k <= rows && k <= cols) ? k : 0;  // [k, cols] as it lies; a tall block is not taken
+  if (k > cols) return 0;
+  if (rows <= k) return rows;                                      // [rows, k] as it lies
+  if (rows % 64 || k % 64) return 0;
+  const int64_t b = (int64_t)(rows / 64) * (k / 64);              // [k, rows], transposed through 64 x 64 tiles
+  return b > 0x7fffffff ? 0 : (int)b;
+}
+
+extern "C" int dion_dion2_gather_prepared(const uint64_t* M_ptrs, int m_dtype, int n, int mats_per_ptr, int rows,
+                                          int cols, int select_dim, const int32_t* idx, int k, float ef_decay,
+                                          void* U_sel, float* sumsq, void* stream) {
+  if (int rc = check_select_dim("dion_dion2_gather_prepared", select_dim)) return rc;
+  if (int rc = check_state_dtype("dion_dion2_gather_prepared", "m_dtype", m_dtype)) return rc;
+  if (n < 0 || mats_per_ptr <= 0 || rows < 0 || cols < 0 || k < 0)
+    return fail(DION_E_INVALID, "dion_dion2_gather_prepared: bad size");
+  if (n == 0 || rows == 0 || cols == 0 || k == 0) return DION_OK;
+  if (!M_ptrs || !idx || !U_sel || !sumsq) return fail(DION_E_INVALID, "dion_dion2_gather_prepared: null argument");
+  const int blocks = dion_dion2_gather_sumsq_blocks(rows, cols, select_dim, k);
+  if (blocks == 0)
+    return fail(DION_E_INVALID, "dion_dion2_gather_prepared: %d of %d x %d along dim %d has no prepared form "
+                "(see dion_dion2_gather_sumsq_blocks)", k, rows, cols, select_dim);
+  if (!aligned16((uint64_t)U_sel))
+    return fail(DION_E_INVALID, "dion_dion2_gather_prepared: U_sel is not 16-byte aligned");
+  const int64_t sel_numel = select_dim == -2 ? (int64_t)k * cols : (int64_t)rows * k;
+  const bool vec4 = (cols % 4 == 0) && table_aligned(M_ptrs, n);
+  const int cmax = ptr_chunk(mats_per_ptr);
+  if (cmax == 0) return fail(DION_E_INVALID, "more than 65535 matrices behind one pointer");
+  for (int i0 = 0; i0 < n; i0 += cmax) {
+    const int c = (n - i0) < cmax ? (n - i0) : cmax;
+    PtrTab m;
+    fill_tab(m, M_ptrs + i0, c);
+    const int64_t mat0 = (int64_t)i0 * mats_per_ptr;
+    HIP_TRY(launch_dion2_gather_prepared(m, dt(m_dtype), c * mats_per_ptr, mats_per_ptr, rows, cols,
+                                         select_dim == -2, idx + mat0 * k, k, ef_decay,
+                                         (bf16_t*)U_sel + mat0 * sel_numel, sumsq + mat0 * blocks, vec4,
+                                         (hipStream_t)stream),
+            "dion_dion2_gather_prepared");
+  }
+  return DION_OK;
+}
+
 extern "C" int dion_dion2_post(const uint64_t* X_ptrs, int x_dtype, int n, int mats_per_ptr, int rows, int cols,
                                int select_dim, const void* U_sel, int u_dtype, int k, const int32_t* map,
                                const float* row_scale, const float* lr_dev, const float* adj_lr_dev,

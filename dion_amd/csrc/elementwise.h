@@ -60,6 +60,13 @@ hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int3
 hipError_t launch_dion2_gather(const PtrTab& M, int m_dtype, int n_mat, int mats_per_ptr, int rows, int cols,
                                int select_rows, const int32_t* idx, int k, float ef_decay, bf16_t* U,
                                bool vec4, hipStream_t st);
+// dion2 gather writing the orthogonalization input in the iteration's layout plus partial sums of squares:
+// rows selected (k <= cols): U [n_mat, k, cols], one partial per selected row; columns selected: U [n_mat, rows, k]
+// with one partial per row when rows <= k, else U^T [n_mat, k, rows] with one partial per 64 x 64 tile
+// (rows % 64 == 0 and k % 64 == 0).
+hipError_t launch_dion2_gather_prepared(const PtrTab& M, int m_dtype, int n_mat, int mats_per_ptr, int rows,
+                                        int cols, int select_rows, const int32_t* idx, int k, float ef_decay,
+                                        bf16_t* U, float* sumsq, bool vec4, hipStream_t st);
 hipError_t launch_dion2_post(const PtrTab& X, int x_dtype, int n_mat, int mats_per_ptr, int rows, int cols,
                              int select_rows, const void* U, int u_dtype, int k, const int32_t* map,
                              const float* row_scale, const float* lr_dev, const float* adj_lr_dev,

@@ -916,11 +916,16 @@ hipError_t launch_dion2_topk(const float* norms, int n_mat, int dim, int k, int3
 // U_sel = bf16(M[sel]); M[sel] *= ef_decay.
 // rows selected: block (j, mat) copies row idx[j]; columns selected: block (row, mat) gathers the k
 // selected columns (ascending, so the reads walk the row forwards).
-template <typename MT, bool VEC>
+// SUMSQ: the block also writes the sum of squares of the bf16 values of its slice of U, sumsq[mat * gridDim.x +
+// blockIdx.x] -- one partial sum of ||U_mat||_F^2 per selected row (rows selected) or per row (columns).
+template <typename MT, bool VEC, bool SUMSQ = false>
 __global__ __launch_bounds__(256) void dion2_gather_kernel(PtrTab M, int mats_per_ptr, int rows,
                                                            int cols, int select_rows,
                                                            const int32_t* __restrict__ idx, int k,
-                                                           float ef_decay, bf16_t* __restrict__ U) {
+                                                           float ef_decay, bf16_t* __restrict__ U,
+                                                           float* __restrict__ sumsq = nullptr) {
+  __shared__ float red[16];
+  float ss = 0.f;
   const int mat = blockIdx.y;
   MT* m = (MT*)M.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
   const int32_t* id = idx + (int64_t)mat * k;
@@ -934,13 +939,23 @@ __global__ __launch_bounds__(256) void dion2_gather_kernel(PtrTab M, int mats_pe
         st_load4<MT>(src, c4, v);
         st_store4<bf16_t>(u, c4, v);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], ef_decay);
+        for (int e = 0; e < 4; ++e) {
+          if (SUMSQ) {
+            const float r = st_round<bf16_t>(v[e]);
+            ss += r * r;
+          }
+          v[e] = __fmul_rn(v[e], ef_decay);
+        }
         st_store4<MT>(src, c4, v);
       }
     } else {
       for (int c = threadIdx.x; c < cols; c += 256) {
         const float v = st_load<MT>(src, c);
         u[c] = f32_to_bf16(v);
+        if (SUMSQ) {
+          const float r = st_round<bf16_t>(v);
+          ss += r * r;
+        }
         st_store<MT>(src, c, __fmul_rn(v, ef_decay));
       }
     }
@@ -952,8 +967,61 @@ __global__ __launch_bounds__(256) void dion2_gather_kernel(PtrTab M, int mats_pe
       const int c = id[j];
       const float v = st_load<MT>(src, c);
       u[j] = f32_to_bf16(v);
+      if (SUMSQ) {
+        const float q = st_round<bf16_t>(v);
+        ss += q * q;
+      }
       st_store<MT>(src, c, __fmul_rn(v, ef_decay));
     }
+  }
+  if (SUMSQ) {
+    ss = block_sum(ss, red);
+    if (threadIdx.x == 0) sumsq[(int64_t)mat * gridDim.x + blockIdx.x] = ss;
+  }
+}
+
+// Columns selected from tall matrices, U written transposed ([k][rows]: the short side along rows, the
+// layout the orthogonalization carries): one tile of 64 rows x 64 selected columns per workgroup, staged
+// through LDS so that U^T rows leave as whole 128-byte runs.  sumsq[(mat * row_tiles + row tile) * (k / 64) +
+// column tile]: sum of squares of the tile's bf16 values.  rows % 64 == 0, k % 64 == 0.
+template <typename MT>
+__global__ __launch_bounds__(256) void dion2_gather_cols_transposed_kernel(PtrTab M, int mats_per_ptr, int rows,
+                                                                           int cols,
+                                                                           const int32_t* __restrict__ idx, int k,
+                                                                           float ef_decay, bf16_t* __restrict__ U,
+                                                                           float* __restrict__ sumsq) {
+  __shared__ __attribute__((aligned(16))) bf16_t tile[64][72];
+  __shared__ float red[16];
+  const int mat = blockIdx.z;
+  MT* m = (MT*)M.p[mat / mats_per_ptr] + (int64_t)(mat % mats_per_ptr) * rows * cols;
+  const int r0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
+  const int j = threadIdx.x & 63, rsub = threadIdx.x >> 6;
+  const int c = idx[(int64_t)mat * k + j0 + j];
+  float ss = 0.f;
+  float v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) v[i] = st_load<MT>(m, (int64_t)(r0 + rsub + 4 * i) * cols + c);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const bf16_t b = f32_to_bf16(v[i]);
+    tile[rsub + 4 * i][j] = b;
+    const float q = bf16_to_f32(b);
+    ss += q * q;
+    st_store<MT>(m, (int64_t)(r0 + rsub + 4 * i) * cols + c, __fmul_rn(v[i], ef_decay));
+  }
+  ss = block_sum(ss, red);  // (its barriers also order the tile writes before the reads below)
+  if (threadIdx.x == 0)
+    sumsq[((int64_t)mat * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x] = ss;
+  bf16_t* ut = U + (int64_t)mat * k * rows;
+  const int chunk = threadIdx.x & 7, rr = threadIdx.x >> 3;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int col = rr + pass * 32;
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      w[e] = (uint32_t)tile[chunk * 8 + 2 * e][col] | ((uint32_t)tile[chunk * 8 + 2 * e + 1][col] << 16);
+    *(uint4*)(ut + (int64_t)(j0 + col) * rows + r0 + chunk * 8) = make_uint4(w[0], w[1], w[2], w[3]);
   }
 }
 
@@ -970,6 +1038,32 @@ hipError_t launch_dion2_gather(const PtrTab& M, int m_dtype, int n_mat, int mats
     if (vec4) GATHER_LAUNCH(float, true); else GATHER_LAUNCH(float, false);
   }
 #undef GATHER_LAUNCH
+  return hipGetLastError();
+}
+
+hipError_t launch_dion2_gather_prepared(const PtrTab& M, int m_dtype, int n_mat, int mats_per_ptr, int rows,
+                                        int cols, int select_rows, const int32_t* idx, int k, float ef_decay,
+                                        bf16_t* U, float* sumsq, bool vec4, hipStream_t st) {
+  if (!select_rows && rows > k) {
+    dim3 grid(k / 64, rows / 64, n_mat);
+    if (m_dtype == 0)
+      hipLaunchKernelGGL(dion2_gather_cols_transposed_kernel<bf16_t>, grid, dim3(256), 0, st, M, mats_per_ptr, rows,
+                         cols, idx, k, ef_decay, U, sumsq);
+    else
+      hipLaunchKernelGGL(dion2_gather_cols_transposed_kernel<float>, grid, dim3(256), 0, st, M, mats_per_ptr, rows,
+                         cols, idx, k, ef_decay, U, sumsq);
+    return hipGetLastError();
+  }
+  dim3 grid(select_rows ? k : rows, n_mat);
+#define GATHERS_LAUNCH(MT, V)                                                                               \
+  hipLaunchKernelGGL((dion2_gather_kernel<MT, V, true>), grid, dim3(256), 0, st, M, mats_per_ptr, rows, cols, \
+                     select_rows, idx, k, ef_decay, U, sumsq)
+  if (m_dtype == 0) {
+    if (vec4) GATHERS_LAUNCH(bf16_t, true); else GATHERS_LAUNCH(bf16_t, false);
+  } else {
+    if (vec4) GATHERS_LAUNCH(float, true); else GATHERS_LAUNCH(float, false);
+  }
+#undef GATHERS_LAUNCH
   return hipGetLastError();
 }
 

@@ -474,10 +474,21 @@ def normuon_stats_selected(U: Tensor, V: List[Tensor], idx: Tensor, beta2: float
     return scale
 
 
-def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_decay: float):
+def dion2_prepared_blocks(rows: int, cols: int, select_dim: int, k: int) -> int:
+    """Partial sums per matrix that ``dion2_select(..., prepared=True)`` writes for ``k`` slices of a
+    ``rows x cols`` matrix along ``select_dim``; 0 when the selected block has no prepared form."""
+    return int(_lib.load().dion_dion2_gather_sumsq_blocks(int(rows), int(cols), int(select_dim), int(k)))
+
+
+def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_decay: float, prepared: bool = False):
     """``M += G``; pick the ``k`` slices of largest L1 norm along ``select_dim`` of every matrix; return
     (U_sel bf16 arena, idx int32 [n_mat, k] ascending, map int32 [n_mat, dim]) and decay the selected
-    slices of ``M`` by ``ef_decay``.  Mirrors ``dion2_pre_orthogonalize`` (dion/dion2.py:439-547)."""
+    slices of ``M`` by ``ef_decay``.  Mirrors ``dion2_pre_orthogonalize`` (dion/dion2.py:439-547).
+
+    ``prepared=True`` (only where ``dion2_prepared_blocks`` is not 0): the selected blocks are written as a
+    prepared orthogonalization input -- ``U_sel [n_mat, min, max]`` with the short side of the block along rows
+    (a tall block transposed) -- and a fourth result ``sumsq [n_mat, blocks]`` holds partial sums of their
+    squares."""
     if select_dim not in (-2, -1):
         raise ValueError(f"select_dim must be -2 or -1, got {select_dim}")
     n = len(G)
@@ -505,6 +516,17 @@ def dion2_select(G: List[Tensor], M: List[Tensor], k: int, select_dim: int, ef_d
           "dion2_accumulate")
     check(lib.dion_dion2_topk(norms.data_ptr(), n_mat, dim, k, idx.data_ptr(), imap.data_ptr(), st),
           "dion2_topk")
+    if prepared:
+        blocks = dion2_prepared_blocks(rows, cols, select_dim, k)
+        if blocks == 0:
+            raise ValueError(f"dion2_select: {k} slices of {rows} x {cols} along dim {select_dim} have no prepared form")
+        sr, sc = (k, cols) if select_dim == -2 else (rows, k)
+        U = U.view(n_mat, min(sr, sc), max(sr, sc))
+        sumsq = torch.empty(n_mat, blocks, dtype=torch.float32, device=dev)
+        check(lib.dion_dion2_gather_prepared(mp, mcode, n, mats_per_ptr, rows, cols, select_dim, idx.data_ptr(), k,
+                                             float(ef_decay), U.data_ptr(), sumsq.data_ptr(), st),
+              "dion2_gather_prepared")
+        return U, idx, imap, sumsq
     check(lib.dion_dion2_gather(mp, mcode, n, mats_per_ptr, rows, cols, select_dim, idx.data_ptr(), k,
                                 float(ef_decay), U.data_ptr(), st), "dion2_gather")
     return U, idx, imap

@@ -15,7 +15,7 @@ from torch import Tensor
 from torch.optim.optimizer import Optimizer
 
 from . import newton_schulz as ns
-from . import scalar_opts
+from . import ops, scalar_opts
 
 
 class LiveScalars:
@@ -357,6 +357,22 @@ class OrthoOptimizer(Optimizer):
         if self._custom_ns:
             out = out.reshape(U.shape).to(torch.bfloat16).contiguous()
         return out
+
+    # hand the orthogonalization its input as the producing kernel writes it (False: the arena in the
+    # parameters' layout, normalised and transposed by passes of the orthogonalization call)
+    prepared_input = True
+
+    def _takes_prepared(self, n_mat: int, rows: int, cols: int, select_dim: int, k: int, flat3d: bool,
+                        M: List[Tensor]) -> bool:
+        """Dion2 / NorDion2: whether the ``k`` slices selected along ``select_dim`` of ``n_mat`` matrices of
+        ``rows x cols`` go to a built-in orthogonalization as the gather kernel writes them."""
+        if not self.prepared_input or flat3d or self._custom_ns:
+            return False
+        if ops.dion2_prepared_blocks(rows, cols, select_dim, k) == 0:
+            return False
+        sr, sc = (k, cols) if select_dim == -2 else (rows, k)
+        return ns.accepts_prepared(self._newton_schulz_func, n_mat, sr, sc) and \
+            all(m.data_ptr() % 16 == 0 for m in M)
 
     def _orthogonalize_update(self, U: Tensor, epsilon: float, X: List[Tensor], lr: Tensor, adj_ratio: float,
                               weight_decay, cautious_wd: bool) -> bool:

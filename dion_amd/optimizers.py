@@ -56,9 +56,6 @@ class _MomentumOrtho(OrthoOptimizer):
     _normalize = False
     # Muon only: run orthogonalization and update as one library call (False: the two-call sequence)
     fused_update = True
-    # hand the orthogonalization its input as the momentum kernel writes it (False: the arena in the
-    # parameters' layout, normalised and transposed by passes of the orthogonalization call)
-    prepared_input = True
 
     def _shape_group_phases(self, group: dict, params: List[Tensor]):
         """Generator: [momentum / cast] yield [orthogonalization GEMMs] yield [normalise / update]."""
@@ -305,11 +302,26 @@ class Dion2(OrthoOptimizer):
                                                          group["weight_decay"], group["ef_decay"], select_dim)
             return
 
+        eps = float(group["epsilon"])
+        sel_rows, sel_cols = (k, cols) if select_dim == -2 else (rows, k)
+        if self._takes_prepared(n * mats, rows, cols, select_dim, k, flatten and len(shape) >= 3, M):
+            # the gather writes the selected blocks the way the iteration carries them, with the partial sums
+            # of their Frobenius norms (no norm / scale / transpose pass inside the orthogonalization call)
+            U_sel, _idx, imap, sumsq = ops.dion2_select(G, M, k, select_dim, group["ef_decay"], prepared=True)
+            yield
+            _note_stream(U_sel)
+            _note_stream(sumsq)
+            O = ns.orthogonalize_prepared(self._newton_schulz_func, U_sel, sumsq, sel_rows, sel_cols, eps)
+            del U_sel, sumsq
+            yield
+            _note_stream(O)
+            ratio = adjust_lr_ratio(ratio_shape, group["adjust_lr"], flatten)
+            ops.dion2_post(X, O.view(n, mats, sel_rows, sel_cols), imap, group["lr"], ratio,
+                           group["weight_decay"], select_dim)
+            return
         U_sel, _idx, imap = ops.dion2_select(G, M, k, select_dim, group["ef_decay"])
-        sel_rows, sel_cols = U_sel.shape[-2], U_sel.shape[-1]
         yield
         _note_stream(U_sel)
-        eps = float(group["epsilon"])
         if flatten and len(shape) >= 3:
             # leading dim stays, the rest of the selected block is one long row
             # (dion/megabatch_base.py:903-904)
@@ -418,15 +430,25 @@ class NorDion2(OrthoOptimizer):
             return
 
         # error-feedback decay of the selected rows is the momentum factor (dion/nordion2.py:352-359)
-        U_sel, idx, imap = ops.dion2_select(G, M, k, select_dim, group["mu"])
-        yield
-        _note_stream(U_sel)
-        if flatten and len(shape) >= 3:
-            # leading dim stays, the selected rows of all the other dims form one long row (per parameter,
-            # as in Muon and Dion2 here; dion/megabatch_base.py:903-904 flattens the stack instead)
-            O = self._orthogonalize(U_sel.view(n, shape[0], -1), float(group["epsilon"]))
+        eps = float(group["epsilon"])
+        flat3d = flatten and len(shape) >= 3
+        if self._takes_prepared(n * mats, rows, cols, select_dim, k, flat3d, M):
+            U_sel, idx, imap, sumsq = ops.dion2_select(G, M, k, select_dim, group["mu"], prepared=True)
+            yield
+            _note_stream(U_sel)
+            _note_stream(sumsq)
+            O = ns.orthogonalize_prepared(self._newton_schulz_func, U_sel, sumsq, k, cols, eps)
+            del sumsq
         else:
-            O = self._orthogonalize(U_sel.view(n * mats, k, cols), float(group["epsilon"]))
+            U_sel, idx, imap = ops.dion2_select(G, M, k, select_dim, group["mu"])
+            yield
+            _note_stream(U_sel)
+            if flat3d:
+                # leading dim stays, the selected rows of all the other dims form one long row (per parameter,
+                # as in Muon and Dion2 here; dion/megabatch_base.py:903-904 flattens the stack instead)
+                O = self._orthogonalize(U_sel.view(n, shape[0], -1), eps)
+            else:
+                O = self._orthogonalize(U_sel.view(n * mats, k, cols), eps)
         del U_sel
         yield
         _note_stream(O)

@@ -279,6 +279,22 @@ int dion_dion2_gather(const uint64_t* M_ptrs, int m_dtype, int n, int mats_per_p
                       int select_dim, const int32_t* idx, int k, float ef_decay, void* U_sel,
                       void* stream);
 
+/* dion_dion2_gather writing U_sel as a prepared orthogonalization input (see
+ * dion_ns_orthogonalize_prepared): the selected block with its short side along rows, plus partial sums
+ * of squares of each block.  dion_dion2_gather_sumsq_blocks gives the partial sums per matrix, or 0 when
+ * the block has no prepared form (then use dion_dion2_gather):
+ *   select_dim -2, k <= cols:          U_sel [n_mat, k, cols] as dion_dion2_gather writes it, k sums
+ *   select_dim -1, rows <= k:          U_sel [n_mat, rows, k] likewise, `rows` sums
+ *   select_dim -1, rows > k:           U_sel [n_mat, k, rows], the block transposed; rows and k multiples
+ *                                      of 64, (rows / 64) * (k / 64) sums
+ * M is updated exactly as by dion_dion2_gather.  U_sel 16-byte aligned.
+ * Replaces dion/dion2.py:519-545 together with the transposition and norm of
+ * dion/newton_schulz_triton.py:508-513 / dion/polar_express.py:30-35. */
+int dion_dion2_gather_sumsq_blocks(int rows, int cols, int select_dim, int k);
+int dion_dion2_gather_prepared(const uint64_t* M_ptrs, int m_dtype, int n, int mats_per_ptr, int rows, int cols,
+                               int select_dim, const int32_t* idx, int k, float ef_decay, void* U_sel,
+                               float* sumsq, void* stream);
+
 /* Dion2 fused weight decay + selective update, single rounding:
  *   x = (1 - lr wd) x - b u[map]   on selected slices,  x = (1 - lr wd) x elsewhere
  *   b = lr * adj_ratio, or (*adj_lr_dev) * adj_ratio when adj_lr_dev (nullable, device fp32 scalar:

@@ -341,6 +341,7 @@ def test_nordion2_step_vs_oracle(shape):
         g = (torch.randn(shape) * 0.02).to(torch.bfloat16)
         p.grad = g.to(DEV)
         opt.step()
+        x_old = x
         x, M, V_ref, idx = oracle.nordion2_step(x, g, M, V, 0.02, 0.25, 0.95, 0.95, 0.01, "spectral_norm")
         assert _rel(opt.state[p]["momentum"], M) <= 1e-6
         v_gpu = opt.state[p]["variance_neuron"].cpu()
@@ -348,7 +349,10 @@ def test_nordion2_step_vs_oracle(shape):
         mask[idx] = False
         assert torch.equal(v_gpu[mask], V[mask])  # unselected neurons keep their second moment
         assert _rel(v_gpu, V_ref) <= 3e-2
-        assert _rel(p.data, x) <= 1e-3
+        # the orthogonalized update within 2e-2 of the oracle's: in units of the parameters, 2e-2 of what
+        # the update term moves them
+        moved = _rel(x - x_old * (1 - 0.02 * 0.01), x)
+        assert _rel(p.data, x) <= 2e-2 * moved
         x = p.data.cpu().clone()
         V = v_gpu.clone()
 

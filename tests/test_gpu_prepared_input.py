@@ -143,3 +143,73 @@ def test_step_with_and_without_prepared_input(cls_name, shape):
         assert _rel(a.data, b.data) <= 2e-2 * moved  # the two paths agree to a fraction of that
         if cls_name == "NorMuon":
             assert _rel(oa.state[a]["variance_neuron"], ob.state[b]["variance_neuron"]) <= 2e-2
+
+
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols,select_dim,k", [(256, 1024, -2, 128), (1024, 256, -1, 128), (384, 256, -1, 256),
+                                                    (512, 512, -2, 256), (256, 1024, -2, 64), (130, 520, -2, 33)])
+def test_prepared_dion2_gather_vs_plain(rows, cols, select_dim, k, mdtype):
+    """dion2_select with prepared=True against the plain call: same indices, same momentum bit for bit, the
+    same bf16 block (transposed when it is tall), partial sums = the float64 sum of squares of the block."""
+    from dion_amd import ops
+
+    gen = torch.Generator().manual_seed(rows + 3 * cols + k)
+    n, mats = 2, 2
+    G = [(torch.randn(mats, rows, cols, generator=gen) * 0.02).to(torch.bfloat16).to(DEV) for _ in range(n)]
+    M0 = [(torch.randn(mats, rows, cols, generator=gen) * 0.02).to(mdtype).to(DEV) for _ in range(n)]
+    assert ops.dion2_prepared_blocks(rows, cols, select_dim, k) > 0
+    Ma = [m.clone() for m in M0]
+    Mb = [m.clone() for m in M0]
+    U_plain, idx_a, map_a = ops.dion2_select(G, Ma, k, select_dim, 0.9)
+    U, idx_b, map_b, sumsq = ops.dion2_select(G, Mb, k, select_dim, 0.9, prepared=True)
+    torch.cuda.synchronize()
+    assert torch.equal(idx_a, idx_b) and torch.equal(map_a, map_b)
+    for a, b in zip(Ma, Mb):
+        assert torch.equal(a, b)
+    sr, sc = (k, cols) if select_dim == -2 else (rows, k)
+    want = U_plain.reshape(n * mats, sr, sc)
+    if sr > sc:
+        want = want.mT
+    assert U.shape == (n * mats, min(sr, sc), max(sr, sc))
+    assert torch.equal(U, want.contiguous())
+    exact = U.double().pow(2).sum(dim=(1, 2))
+    assert sumsq.shape == (n * mats, ops.dion2_prepared_blocks(rows, cols, select_dim, k))
+    assert float(((sumsq.double().sum(dim=1) - exact).abs() / exact).max()) <= 1e-6
+
+
+def test_dion2_blocks_without_a_prepared_form():
+    from dion_amd import ops
+
+    assert ops.dion2_prepared_blocks(1024, 256, -2, 512) == 0   # rows selected, block taller than wide
+    assert ops.dion2_prepared_blocks(1000, 256, -1, 64) == 0    # transposed form needs whole 64 x 64 tiles
+    assert ops.dion2_prepared_blocks(1024, 256, -1, 64) == 16 * 1
+
+
+@pytest.mark.parametrize("cls_name", ["Dion2", "NorDion2"])
+@pytest.mark.parametrize("shape", [(512, 1024), (1024, 512), (2, 512, 512)])
+def test_dion2_step_with_and_without_prepared_input(cls_name, shape):
+    import dion
+
+    cls = getattr(dion, cls_name)
+    gen = torch.Generator().manual_seed(12)
+    X = [torch.randn(shape, generator=gen) * 0.02 for _ in range(3)]
+    G = [(torch.randn(shape, generator=gen) * 0.02).to(torch.bfloat16) for _ in range(3)]
+
+    def run(prepared):
+        ps = [torch.nn.Parameter(x.clone().to(DEV)) for x in X]
+        for p, g in zip(ps, G):
+            p.grad_dtype = None
+            p.grad = g.to(DEV)
+        opt = cls(ps, lr=0.02, fraction=0.25, weight_decay=0.01)
+        opt.prepared_input = prepared
+        opt.step()
+        opt.step()
+        torch.cuda.synchronize()
+        return ps, opt
+
+    pa, oa = run(True)
+    pb, ob = run(False)
+    for a, b, x in zip(pa, pb, X):
+        assert torch.equal(oa.state[a]["momentum"], ob.state[b]["momentum"])
+        moved = _rel(b.data - x.to(DEV) * (1 - 0.02 * 0.01) ** 2, x)   # what the selected updates add up to
+        assert _rel(a.data, b.data) <= 2e-2 * max(moved, 1e-6)
