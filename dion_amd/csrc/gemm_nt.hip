@@ -66,6 +66,69 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
 }
 
+// Compile-time loop: f(std::integral_constant<int, I>()) for I in [I0, N).
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>());
+    static_for<I + 1, N>(f);
+  }
+}
+
+// The fragment reads of a 16-wide k slice are issued, one behind each MFMA of the slice before, in the
+// order the MFMAs (row-major over the TM x TN accumulator tiles) first need them: A0, B0..B(TN-1),
+// A1..A(TM-1).  Every read is an assembly statement and so is every wait: the LDS returns in order, so
+// "all but the newest N LDS instructions have returned" is exactly "the fragments MFMA q needs are in
+// their registers", with N counted here from the issue order -- the reads of the slice issued after the
+// later of the two fragments q needs, plus the reads of the next slice issued ahead of q.  (Left to the
+// compiler, every slice starts with a wait for all six reads, the last of which was issued two MFMAs
+// earlier.)  A K-major fragment is two transposing reads.
+template <int TM, int TN, bool QK>
+struct FragSched {
+  static constexpr int NR = TM + TN, NM = TM * TN;
+  static constexpr int RPM = (NR + NM - 1) / NM;  // reads slotted behind each MFMA
+  static constexpr int instrs(int r) { return (QK && r >= 1 && r <= TN) ? 2 : 1; }
+  static constexpr int pos_a(int i) { return i == 0 ? 0 : TN + i; }
+  static constexpr int pos_b(int j) { return 1 + j; }
+  // LDS instructions that may still be outstanding when MFMA q of a slice issues
+  static constexpr int allowed(int q) {
+    const int i = q / TN, j = q % TN;
+    const int need = pos_a(i) > pos_b(j) ? pos_a(i) : pos_b(j);
+    int n = 0;
+    for (int r = need + 1; r < NR; ++r) n += instrs(r);
+    const int issued = q * RPM < NR ? q * RPM : NR;
+    for (int r = 0; r < issued; ++r) n += instrs(r);
+    return n;
+  }
+  static_assert(allowed(NM - 1) < 16, "lgkmcnt is a four-bit field");
+};
+
+// Fragment wait: an asm statement that takes the fragments it guards as read-write operands, so that to
+// the compiler they are (re)defined here and no use of them can be scheduled ahead of the wait.
+template <int N>
+__device__ __forceinline__ void frag_wait(bf16x8& a, bf16x8& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+// 16-byte LDS read at addr + OFF, issued from assembly (the compiler does not know it is in flight: the
+// matching frag_wait is what its consumers wait on).
+template <int OFF>
+__device__ __forceinline__ void lds_read16(bf16x8& dst, uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "ds offset field");
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+// K-major fragment: two transposing reads, rows k..k+3 and k+4..k+7 of the tile (HI bytes apart)
+template <int OFF, int HI>
+__device__ __forceinline__ void lds_read_tr(bf16x8& dst, uint32_t addr) {
+  static_assert(OFF >= 0 && OFF + HI < 65536, "ds offset field");
+  typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+  typedef __attribute__((ext_vector_type(4))) unsigned u32x4f;
+  u32x2 lo, hi;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(addr), "n"(OFF));
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "n"(OFF + HI));
+  const u32x4f v = {lo[0], lo[1], hi[0], hi[1]};
+  dst = __builtin_bit_cast(bf16x8, v);
+}
+
 // Enumeration of the upper triangle (ti <= tj) of a T x T tile grid in super-blocks of SB x SB
 // tiles, so that the ~32 workgroups an XCD runs side by side touch as few distinct operand row
 // blocks as possible (their L2 is what feeds the LDS): a diagonal super-block has SB(SB+1)/2
@@ -280,22 +343,27 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   // tile, not two: Q's loads are skipped and its fragments are read from P's half of the slot.  (With a
   // two-slot ring the barrier waits for every outstanding load, so the load count per slab is free to vary.)
   const bool one_operand = !QK && p.tri && ti == tj && p.P == p.Q && p.ldp == p.ldq && p.strideP == p.strideQ;
+  // LDS layout of the ring: [P slot 0][P slot 1][Q slot 0][Q slot 1].  With the two slots of an operand
+  // side by side, slot, wavefront-tile row block and k slice all fit the offset field of the LDS read
+  // instructions: the per-lane address registers below are all the address arithmetic the loop needs.
+  static_assert(Cfg::P_BYTES == Cfg::Q_BYTES, "square tiles: a one-operand tile reads Q's fragments from P's slots");
   auto issue_load = [&](int kt, int buf, int j) {
     if (one_operand && j >= Cfg::P_LOADS) return;
     const int k = kt < KT ? kt : KT - 1;
-    char* l = lds + buf * Cfg::STAGE_BYTES + wave * (64 * 16);
+    char* l = lds + buf * Cfg::P_BYTES + wave * (64 * 16);
     if (j < Cfg::P_LOADS) {
       const char* src = gP + (int64_t)k * (BK * 2) + (offP + j * stepP);
       __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
     } else {
       const int jq = j - Cfg::P_LOADS;
       const char* src = gQ + k * slabQ + (offQ + jq * stepQ);
-      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + Cfg::P_BYTES + jq * (Cfg::NT * 16)),
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + NSTAGE * Cfg::P_BYTES + jq * (Cfg::NT * 16)),
                                        16, 0, 0);
     }
   };
 
   // ---- LDS -> register fragment addressing (per lane, per 16-wide k slice).
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
   const int frow = lane & 31;
   const int fhalf = lane >> 5;
   const int fswz = (frow / Cfg::SWZ_DIV) % Cfg::CPR;
@@ -303,8 +371,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
     const int chunk = ((kk * 2 + fhalf) ^ fswz) * 16;
-    aoff[kk] = (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + chunk);
-    boff[kk] = (uint32_t)((one_operand ? 0 : Cfg::P_BYTES) + (wn * Cfg::WTN + frow) * (BK * 2) + chunk);
+    aoff[kk] = lds_base + (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + chunk);
+    boff[kk] = lds_base + (uint32_t)((one_operand ? 0 : NSTAGE * Cfg::P_BYTES) + (wn * Cfg::WTN + frow) * (BK * 2) + chunk);
   }
 
   // QK fragments: within a 16-lane group, lane 4r+q addresses row r / 4-element piece q of a 4x16
@@ -315,49 +383,30 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
     const int g16 = lane >> 4, t16 = lane & 15;
 #pragma unroll
     for (int r = 0; r < TN; ++r)
-      qoff[r] = (uint32_t)(Cfg::P_BYTES + (8 * (g16 >> 1) + (t16 >> 2)) * (BN * 2) +
-                           ((((wn * Cfg::WTN + r * 32) >> 5) ^ (t16 >> 2)) << 6) + (g16 & 1) * 32 +
-                           (t16 & 3) * 8);
+      qoff[r] = lds_base + (uint32_t)(NSTAGE * Cfg::P_BYTES + (8 * (g16 >> 1) + (t16 >> 2)) * (BN * 2) +
+                                      ((((wn * Cfg::WTN + r * 32) >> 5) ^ (t16 >> 2)) << 6) + (g16 & 1) * 32 +
+                                      (t16 & 3) * 8);
   }
 
-  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
-  // Fragment reads of a slice go out in the order A0, B0..B(TN-1), A1..A(TM-1); LDS returns in order, so once
-  // at most the TM-1 reads issued after the last B fragment are outstanding, every B fragment has arrived.
-  // The wait is an asm statement that takes the fragments it guards as read-write operands: to the compiler
-  // they are (re)defined here, so no use of them can be scheduled ahead of the wait.
+  typedef FragSched<TM, TN, QK> FS;
   bf16x8 fa[2][TM], fb[2][TN];
-  auto qk_wait = [&](int f) {
-    if constexpr (QK) {
-      static_assert(TN == 2, "operand list of the wait below");
-      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(fb[f][0]), "+v"(fb[f][1]) : "n"(TM - 1));
-    }
-  };
-  // Fragment read r (0..NR-1) of slice kk of ring slot buf into fragment set f, in the order the
-  // MFMAs (row-major over the TM x TN accumulators) first need them: A0, B0..B(TN-1), A1..A(TM-1).
-  auto read_frag = [&](int buf, int kk, int f, int r) {
-    const char* st = lds + buf * Cfg::STAGE_BYTES;
-    if (r == 0 || r > TN) {
-      const int i = r == 0 ? 0 : r - TN;
-      fa[f][i] = *(const bf16x8*)(st + aoff[kk] + i * (32 * BK * 2));
-    } else if (QK) {
-      // The transposing reads are written as assembly: through the builtin the
-      // compiler makes each of them wait for every outstanding direct-to-LDS load (it cannot tell that they
-      // read another ring slot), which exposes the whole load latency once per slab.  The compiler does not
-      // know these reads are in flight: qk_wait() below is the wait their consumers need.
-      const int j = r - 1;
-      const uint32_t a = lds_base + (uint32_t)(buf * Cfg::STAGE_BYTES) + qoff[j] + (uint32_t)(kk * (16 * BN * 2));
-      typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
-      u32x2 lo, hi;
-      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(a));
-      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(a), "n"(4 * BN * 2));
-      typedef __attribute__((ext_vector_type(4))) unsigned u32x4f;
-      const u32x4f v = {lo[0], lo[1], hi[0], hi[1]};
-      fb[f][j] = __builtin_bit_cast(bf16x8, v);
+  // Fragment read r (0..NR-1, order A0, B0..B(TN-1), A1..A(TM-1)) of slice kk of ring slot buf into
+  // fragment set f; all four are compile-time constants and end up in the instruction's offset field.
+  auto read_frag = [&](auto bufc, auto kkc, auto fc, auto rc) {
+    constexpr int buf = decltype(bufc)::value, kk = decltype(kkc)::value, f = decltype(fc)::value,
+                  r = decltype(rc)::value;
+    if constexpr (r == 0 || r > TN) {
+      constexpr int i = r == 0 ? 0 : r - TN;
+      lds_read16<buf * Cfg::P_BYTES + i * (32 * BK * 2)>(fa[f][i], aoff[kk]);
+    } else if constexpr (QK) {
+      constexpr int j = r - 1;
+      lds_read_tr<buf * Cfg::Q_BYTES + kk * (16 * BN * 2), 4 * BN * 2>(fb[f][j], qoff[j]);
     } else {
-      const int j = r - 1;
-      fb[f][j] = *(const bf16x8*)(st + boff[kk] + j * (32 * BK * 2));
+      constexpr int j = r - 1;
+      lds_read16<buf * Cfg::Q_BYTES + j * (32 * BK * 2)>(fb[f][j], boff[kk]);
     }
   };
+  typedef std::integral_constant<int, 0> ic0;
 
   f32x16 acc[TM][TN];
 #pragma unroll
@@ -374,8 +423,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 #pragma unroll
     for (int j = 0; j < LPS; ++j) issue_load(s, s, j);
   pipeline_barrier<(NSTAGE - 2) * LPS>();
-#pragma unroll
-  for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
+  static_for<0, NR>([&](auto rc) { read_frag(ic0(), ic0(), ic0(), rc); });
 #pragma unroll
   for (int j = 0; j < LPS; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
   __builtin_amdgcn_sched_barrier(0);
@@ -385,47 +433,45 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   // the slot that slab occupied) are slotted one behind each MFMA.  sched_barrier pins that order.
   // KT is a multiple of NSTAGE (launcher checks) so ring slots are compile-time constants.
   for (int kt0 = 0; kt0 < KT; kt0 += NSTAGE) {
+    static_for<0, NSTAGE * KK>([&](auto skc) {
+      constexpr int s = decltype(skc)::value / KK, kk = decltype(skc)::value % KK;
+      constexpr int cur = kk & 1, nxt = cur ^ 1;
+      constexpr bool last = (kk == KK - 1);
+      // slab kt+1 landed, slab kt fully read
+      if constexpr (last) pipeline_barrier<(NSTAGE - 2) * LPS>();
+      static_for<0, NM>([&](auto qc) {
+        constexpr int q = decltype(qc)::value, i = q / TN, j = q % TN;
+        frag_wait<FS::allowed(q)>(fa[cur][i], fb[cur][j]);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<q * RPM, ((q + 1) * RPM < NR ? (q + 1) * RPM : NR)>([&](auto rc) {
+          if constexpr (last)
+            read_frag(std::integral_constant<int, (s + 1) % NSTAGE>(), ic0(), std::integral_constant<int, nxt>(), rc);
+          else
+            read_frag(std::integral_constant<int, s>(), std::integral_constant<int, kk + 1>(),
+                      std::integral_constant<int, nxt>(), rc);
+        });
+        if constexpr (last) {
 #pragma unroll
-    for (int s = 0; s < NSTAGE; ++s) {
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        const int cur = kk & 1, nxt = cur ^ 1;
-        const bool last = (kk == KK - 1);
-        // slab kt+1 landed, slab kt fully read
-        if (last) pipeline_barrier<(NSTAGE - 2) * LPS>();
-        qk_wait(cur);
-#pragma unroll
-        for (int q = 0; q < NM; ++q) {
-          acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              fa[cur][q / TN], fb[cur][q % TN], acc[q / TN][q % TN], 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int r = q * RPM; r < (q + 1) * RPM && r < NR; ++r) {
-            if (last) read_frag((s + 1) % NSTAGE, 0, nxt, r);
-            else read_frag(s, kk + 1, nxt, r);
-          }
-          if (last) {
-#pragma unroll
-            for (int j = q * LPM; j < (q + 1) * LPM && j < LPS; ++j)
-              issue_load(kt0 + s + NSTAGE, s, j);
-          }
-          __builtin_amdgcn_sched_barrier(0);
+          for (int jl = q * LPM; jl < (q + 1) * LPM && jl < LPS; ++jl) issue_load(kt0 + s + NSTAGE, s, jl);
         }
-      }
-    }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
   }
   wait_vmcnt<0>();  // drain the redundant tail refills before LDS is reused / the wave exits
-  if (QK) {
-    // The read-ahead of the last slice issued transposing reads whose results nobody uses.  The compiler
-    // does not know they are in flight; were their destination registers dead here, it would hand them
-    // to whatever comes next (the lane index, store addresses) and a read landing late would overwrite
-    // that.  So: wait for the LDS queue to drain, and only then let go of the fragment registers -- the
-    // empty asm statements below are their last use and sit behind the wait.
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+  // The read-ahead of the last slice issued reads whose results nobody uses.  The compiler does not know
+  // they are in flight; were their destination registers dead here, it would hand them to whatever comes
+  // next (the lane index, store addresses) and a read landing late would overwrite that.  So: wait for the
+  // LDS queue to drain, and only then let go of the fragment registers -- the empty asm statements below
+  // are their last use and sit behind the wait.
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
+  for (int f = 0; f < 2; ++f) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) asm volatile("" ::"v"(fb[f][j]));
+    for (int i = 0; i < TM; ++i) asm volatile("" ::"v"(fa[f][i]));
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" ::"v"(fb[f][j]));
   }
 
   // ---- epilogue.  Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4,
@@ -738,59 +784,54 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
   };
   look_ahead();
 
-  // slab kt of the current tile, or slab kt - KT of the next one, into ring slot buf (load j of LPS)
+  // slab kt of the current tile, or slab kt - KT of the next one, into ring slot buf (load j of LPS);
+  // ring layout [P slot 0][P slot 1][Q slot 0][Q slot 1] as in the kernel above
   auto issue_load = [&](int kt, int buf, int j) {
     const bool nx = kt >= KT;
     const int k = nx ? kt - KT : kt;
-    char* l = lds + buf * Cfg::STAGE_BYTES + wave * (64 * 16);
+    char* l = lds + buf * Cfg::P_BYTES + wave * (64 * 16);
     if (j < Cfg::P_LOADS) {
       const char* src = (nx ? gP_n : gP_c) + (int64_t)k * (BK * 2) + (offP + j * stepP);
       __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
     } else {
       const int jq = j - Cfg::P_LOADS;
       const char* src = (nx ? gQ_n : gQ_c) + k * slabQ + (offQ + jq * stepQ);
-      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + Cfg::P_BYTES + jq * (Cfg::NT * 16)), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + NSTAGE * Cfg::P_BYTES + jq * (Cfg::NT * 16)), 16, 0, 0);
     }
   };
 
   // ---- LDS -> register fragments (see the kernel above)
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
   const int frow = lane & 31;
   const int fhalf = lane >> 5;
   const int fswz = (frow / Cfg::SWZ_DIV) % Cfg::CPR;
   uint32_t aoff[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk)
-    aoff[kk] = (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + ((kk * 2 + fhalf) ^ fswz) * 16);
+    aoff[kk] = lds_base + (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + ((kk * 2 + fhalf) ^ fswz) * 16);
   uint32_t qoff[TN];
   {
     const int g16 = lane >> 4, t16 = lane & 15;
 #pragma unroll
     for (int r = 0; r < TN; ++r)
-      qoff[r] = (uint32_t)(Cfg::P_BYTES + (8 * (g16 >> 1) + (t16 >> 2)) * (BN * 2) +
-                           ((((wn * Cfg::WTN + r * 32) >> 5) ^ (t16 >> 2)) << 6) + (g16 & 1) * 32 + (t16 & 3) * 8);
+      qoff[r] = lds_base + (uint32_t)(NSTAGE * Cfg::P_BYTES + (8 * (g16 >> 1) + (t16 >> 2)) * (BN * 2) +
+                                      ((((wn * Cfg::WTN + r * 32) >> 5) ^ (t16 >> 2)) << 6) + (g16 & 1) * 32 +
+                                      (t16 & 3) * 8);
   }
-  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+  typedef FragSched<TM, TN, true> FS;
   bf16x8 fa[2][TM], fb[2][TN];
-  // The transposing reads are assembly the compiler cannot see in flight; this wait takes the fragments it
-  // guards as read-write operands, so no use of them is scheduled ahead of it (see the kernel above).
-  auto qk_wait = [&](int f) { asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(fb[f][0]), "+v"(fb[f][1]) : "n"(TM - 1)); };
-  auto read_frag = [&](int buf, int kk, int f, int r) {
-    const char* st = lds + buf * Cfg::STAGE_BYTES;
-    if (r == 0 || r > TN) {
-      const int i = r == 0 ? 0 : r - TN;
-      fa[f][i] = *(const bf16x8*)(st + aoff[kk] + i * (32 * BK * 2));
+  auto read_frag = [&](auto bufc, auto kkc, auto fc, auto rc) {
+    constexpr int buf = decltype(bufc)::value, kk = decltype(kkc)::value, f = decltype(fc)::value,
+                  r = decltype(rc)::value;
+    if constexpr (r == 0 || r > TN) {
+      constexpr int i = r == 0 ? 0 : r - TN;
+      lds_read16<buf * Cfg::P_BYTES + i * (32 * BK * 2)>(fa[f][i], aoff[kk]);
     } else {
-      const int j = r - 1;
-      const uint32_t a = lds_base + (uint32_t)(buf * Cfg::STAGE_BYTES) + qoff[j] + (uint32_t)(kk * (16 * BN * 2));
-      typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
-      u32x2 lo, hi;
-      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(a));
-      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(a), "n"(4 * BN * 2));
-      typedef __attribute__((ext_vector_type(4))) unsigned u32x4f;
-      const u32x4f v = {lo[0], lo[1], hi[0], hi[1]};
-      fb[f][j] = __builtin_bit_cast(bf16x8, v);
+      constexpr int j = r - 1;
+      lds_read_tr<buf * Cfg::Q_BYTES + kk * (16 * BN * 2), 4 * BN * 2>(fb[f][j], qoff[j]);
     }
   };
+  typedef std::integral_constant<int, 0> ic0;
 
   f32x16 acc[TM][TN];
   auto clear_acc = [&]() {
@@ -857,8 +898,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
 #pragma unroll
   for (int j = 0; j < LPS; ++j) issue_load(0, 0, j);
   pipeline_barrier<0>();
-#pragma unroll
-  for (int r = 0; r < NR; ++r) read_frag(0, 0, 0, r);
+  static_for<0, NR>([&](auto rc) { read_frag(ic0(), ic0(), ic0(), rc); });
 #pragma unroll
   for (int j = 0; j < LPS; ++j) issue_load(1, 1, j);
   __builtin_amdgcn_sched_barrier(0);
@@ -866,40 +906,38 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
   for (;;) {
     // ---- one tile: the main loop of the kernel above; refills past the tile's last slab fetch the next tile
     for (int kt0 = 0; kt0 < KT; kt0 += NSTAGE) {
-#pragma unroll
-      for (int s = 0; s < NSTAGE; ++s) {
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-          const int cur = kk & 1, nxt = cur ^ 1;
-          const bool last = (kk == KK - 1);
-          if (last) pipeline_barrier<0>();
-          qk_wait(cur);
-#pragma unroll
-          for (int q = 0; q < NM; ++q) {
-            if constexpr (OUT_T)
-              acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][q / TN], fb[cur][q % TN],
-                                                                            acc[q / TN][q % TN], 0, 0, 0);
+      static_for<0, NSTAGE * KK>([&](auto skc) {
+        constexpr int s = decltype(skc)::value / KK, kk = decltype(skc)::value % KK;
+        constexpr int cur = kk & 1, nxt = cur ^ 1;
+        constexpr bool last = (kk == KK - 1);
+        if constexpr (last) pipeline_barrier<0>();
+        static_for<0, NM>([&](auto qc) {
+          constexpr int q = decltype(qc)::value, i = q / TN, j = q % TN;
+          frag_wait<FS::allowed(q)>(fa[cur][i], fb[cur][j]);
+          if constexpr (OUT_T)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+          else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          static_for<q * RPM, ((q + 1) * RPM < NR ? (q + 1) * RPM : NR)>([&](auto rc) {
+            if constexpr (last)
+              read_frag(std::integral_constant<int, (s + 1) % NSTAGE>(), ic0(), std::integral_constant<int, nxt>(), rc);
             else
-              acc[q / TN][q % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][q % TN], fa[cur][q / TN],
-                                                                            acc[q / TN][q % TN], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+              read_frag(std::integral_constant<int, s>(), std::integral_constant<int, kk + 1>(),
+                        std::integral_constant<int, nxt>(), rc);
+          });
+          if constexpr (last) {
 #pragma unroll
-            for (int r = q * RPM; r < (q + 1) * RPM && r < NR; ++r) {
-              if (last) read_frag((s + 1) % NSTAGE, 0, nxt, r);
-              else read_frag(s, kk + 1, nxt, r);
-            }
-            if (last) {
-#pragma unroll
-              for (int j = q * LPM; j < (q + 1) * LPM && j < LPS; ++j) issue_load(kt0 + s + NSTAGE, s, j);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+            for (int jl = q * LPM; jl < (q + 1) * LPM && jl < LPS; ++jl) issue_load(kt0 + s + NSTAGE, s, jl);
           }
-        }
-      }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      });
     }
     // The first fragments of the next tile are on their way into set 0.  Let them land before the epilogue:
     // its register traffic must not meet a transposing read still in flight.
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fb[0][0]), "+v"(fb[0][1]));
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]), "+v"(fb[0][0]), "+v"(fb[0][1]));
     store_tile(b_c, ti_c, tj_c);
     pid += (int)gridDim.x;
     if (pid >= total_tiles) break;

@@ -1,10 +1,12 @@
-"""The GEMM kernels issue their transposing LDS reads (ds_read_b64_tr_b16) from assembly, so the compiler does not
-know that the results are still on their way when the statement has executed: it may hand a destination register
-it considers dead to something else, and a read that lands late then overwrites that value (once: the lane index
-ahead of the epilogue's address arithmetic, a GPU memory fault).  This test compiles gemm_nt.hip to gfx950 assembly
-and walks every kernel that contains such reads (gemm_nt_kernel, gemm_qk_walk_kernel) in program order (each loop back-edge taken once), modelling the
-LDS return queue (in-order; s_waitcnt lgkmcnt(N) retires all but the newest N entries): no instruction may read or
-write a register while a transposing read into it is in flight.  Needs hipcc, no GPU."""
+"""The GEMM kernels issue the LDS reads of their MFMA fragments (ds_read_b128, ds_read_b64_tr_b16) from assembly and
+wait for them with hand-counted s_waitcnt lgkmcnt(N), so the compiler does not know that a result is still on its
+way when the statement has executed: it may hand a destination register it considers dead to something else, and a
+read that lands late then overwrites that value (once: the lane index ahead of the epilogue's address arithmetic, a
+GPU memory fault); and a wait counted one too high lets an MFMA read a fragment that has not arrived.  This test
+compiles gemm_nt.hip to gfx950 assembly and walks every kernel (gemm_nt_kernel, gemm_qk_walk_kernel) in program
+order (each loop back-edge taken once), modelling the LDS return queue (in-order; s_waitcnt lgkmcnt(N) retires all
+but the newest N entries): no instruction may read or write a register while an LDS read into it is in flight.
+Needs hipcc, no GPU."""
 import os
 import re
 import shutil
@@ -26,12 +28,17 @@ def _regs(tok):
 
 
 def walk(body):
-    """Returns (number of transposing reads seen, list of hazards) for one kernel's assembly lines."""
+    """Returns (number of LDS reads seen, list of hazards) for one kernel's assembly lines."""
     labels = {l.split(":")[0].strip(): i for i, l in enumerate(body) if re.match(r"\.L\w+:", l.strip())}
-    taken, queue, hazards = set(), [], []
+    taken, queue, vmq, hazards = set(), [], [], []
     pc = steps = n_tr = 0
+    in_asm = False
     while pc < len(body) and steps < 500000:
         steps += 1
+        if "#ASMSTART" in body[pc]:
+            in_asm = True
+        elif "#ASMEND" in body[pc]:
+            in_asm = False
         cur, s = pc, body[pc].split(";")[0].strip()
         pc += 1
         if not s or s.startswith(".") or s.endswith(":"):
@@ -51,9 +58,22 @@ def walk(body):
             m = re.search(r"lgkmcnt\((\d+)\)", s)
             if m:
                 del queue[: max(0, len(queue) - int(m.group(1)))]
+            m = re.search(r"vmcnt\((\d+)\)", s)
+            if m:
+                del vmq[: max(0, len(vmq) - int(m.group(1)))]
             continue
-        inflight = set().union(*[q for q in queue if q]) if queue else set()
-        if op.startswith("ds_read_b64_tr"):
+        inflight = set().union(*[q for q in queue + vmq if q]) if queue or vmq else set()
+        if re.match(r"(buffer|global|flat|scratch)_", op):
+            # vector memory: returns in order, counted by vmcnt.  The destination of a load issued from an
+            # assembly statement is in flight until a wait retires it (the compiler guards its own loads)
+            is_load = in_asm and "_load" in op and "_lds_" not in op and not op.endswith("_lds")
+            dest = _regs(args[0]) if is_load else set()
+            touched = set().union(*[_regs(a) for a in args]) if args else set()
+            if touched & inflight:
+                hazards.append((cur, s))
+            vmq.append(dest)
+            continue
+        if op.startswith("ds_read"):
             dest = _regs(args[0])
             n_tr += 1
             if dest & inflight:
@@ -70,11 +90,18 @@ def walk(body):
 
 def test_the_walk_flags_a_register_reused_before_the_wait():
     bad = ["ds_read_b64_tr_b16 v[10:11], v3", "v_and_b32_e32 v10, 63, v0", "s_waitcnt lgkmcnt(0)", "s_endpgm"]
-    good = ["ds_read_b64_tr_b16 v[10:11], v3", "ds_read_b128 v[20:23], v4", "s_waitcnt lgkmcnt(1)",
+    good = ["ds_read_b64_tr_b16 v[10:11], v3", "ds_read_b128 v[20:23], v4", "ds_read_b128 v[30:33], v4", "s_waitcnt lgkmcnt(1)",
             "v_mfma_f32_32x32x16_bf16 v[0:15], v[20:23], v[10:13], v[0:15]", "v_and_b32_e32 v10, 63, v0", "s_endpgm"]
-    early = ["ds_read_b64_tr_b16 v[10:11], v3", "ds_read_b128 v[20:23], v4", "s_waitcnt lgkmcnt(2)",
+    early = ["ds_read_b64_tr_b16 v[10:11], v3", "ds_read_b128 v[20:23], v4", "ds_read_b128 v[30:33], v4", "s_waitcnt lgkmcnt(2)",
              "v_mfma_f32_32x32x16_bf16 v[0:15], v[20:23], v[10:13], v[0:15]", "s_endpgm"]
-    assert walk(bad)[1] and not walk(good)[1] and walk(early)[1]
+    plain = ["ds_read_b128 v[20:23], v4", "ds_read_b128 v[24:27], v4 offset:4096", "s_waitcnt lgkmcnt(1)",
+             "v_mfma_f32_32x32x16_bf16 v[0:15], v[20:23], v[24:27], v[0:15]", "s_endpgm"]
+    two_loads = [";;#ASMSTART", "buffer_load_dwordx4 v[40:43], v1, s[4:7], s8 offen", ";;#ASMEND",
+                 ";;#ASMSTART", "buffer_load_dwordx4 v[44:47], v1, s[4:7], s9 offen", ";;#ASMEND", "s_waitcnt vmcnt(1)"]
+    staged_bad = two_loads + ["ds_write_b128 v2, v[44:47]", "s_endpgm"]
+    staged_ok = two_loads + ["ds_write_b128 v2, v[40:43]", "s_endpgm"]
+    assert walk(bad)[1] and not walk(good)[1] and walk(early)[1] and walk(plain)[1]
+    assert walk(staged_bad)[1] and not walk(staged_ok)[1]
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not on PATH")
@@ -96,8 +123,9 @@ def test_no_kernel_touches_a_register_a_transposing_read_is_in_flight_to(tmp_pat
     assert sum("gemm_qk_walk_kernel" in k for k in kernels) == 2
     with_tr = 0
     for kname, kbody in kernels.items():
-        n_tr, hazards = walk(kbody)
-        with_tr += n_tr > 0
+        n_reads, hazards = walk(kbody)
+        assert n_reads > 0, kname
+        with_tr += any("ds_read_b64_tr" in l for l in kbody)
         assert not hazards, (kname, hazards[:5])
     assert with_tr >= 8, "the K-major instantiations should contain transposing reads"
     # and nothing is spilled between the first and the last MFMA of a kernel (the software-pipelined loop)
