@@ -27,10 +27,17 @@ static __device__ __forceinline__ bf16x8 join_tr(s16x4 lo, s16x4 hi) {
   return __builtin_bit_cast(bf16x8, v);
 }
 
-template <typename T>
+// One workgroup per CU walks matrices blockIdx.x, blockIdx.x + gridDim.x, ...: while the iterations of one
+// matrix run out of LDS, the next matrix is already on its way into registers (it is read from memory once,
+// the registers hold it until the norm is known), and the stores of the last iteration are left in flight.
+// CH: 16-byte chunks of a matrix a thread holds (12 for n_pad <= 768, else kMaxChunks).  Only the small form
+// has the registers to keep the next matrix next to the live values of an iteration; the large one fetches
+// each matrix when its turn comes.
+template <typename T, int CH>
 __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict__ in, bf16_t* __restrict__ out,
-                                                       int rows, int cols, int n_pad, NsCoeffs co,
+                                                       int batch, int rows, int cols, int n_pad, NsCoeffs co,
                                                        float norm_scale, float eps) {
+  constexpr bool kPrefetch = CH <= 12;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   __shared__ float red[16];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -42,22 +49,23 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
   char* Xs = lds;
   char* As = lds + 64 * xp;
   char* Bs = As + 64 * ap;
-  const int64_t mat = blockIdx.x;
-  const T* src = in + mat * (int64_t)rows * cols;
-  bf16_t* dst = out + mat * (int64_t)rows * cols;
-
-  // ---- load (raw bf16 values), zero padding, sum of squares, scale, store to LDS
-  float ss = 0.f;
-  const bool vec = (cols % 8 == 0) && ((((uintptr_t)src) & 15) == 0) && n_pad * 8 <= kMaxChunks * kThreads;
-  if (vec) {
-    // Each thread keeps its 16-byte chunks in registers between the reduction and the scaled
-    // store, so the matrix is read from HBM once and LDS is written once.
-    const int cpr = tall ? 8 : n_pad / 8;  // chunks per 64-wide (tall) or n_pad-wide (wide) input row
-    const int nchunks = 8 * n_pad;         // 64 * n_pad / 8
-    uint4 raw[kMaxChunks];
+  const int64_t mat_elems = (int64_t)rows * cols;
+  // Each thread keeps its 16-byte chunks of a matrix in registers between the load, the reduction and the
+  // scaled store to LDS, so a matrix is read from HBM once and LDS is written once.  Matrices are whole
+  // numbers of chunks and all equally aligned, so the choice holds for every matrix of the batch.
+  const bool vec = (cols % 8 == 0) && ((((uintptr_t)in) & 15) == 0) && n_pad * 8 <= CH * kThreads;
+  const int cpr = tall ? 8 : n_pad / 8;  // chunks per 64-wide (tall) or n_pad-wide (wide) input row
+  const int nchunks = 8 * n_pad;         // 64 * n_pad / 8
+  uint4 raw[CH];
+  auto fetch = [&](int64_t mat) {
+    const T* src = in + mat * mat_elems;
+    // (the chunk coordinates are recomputed per matrix from a value the compiler cannot see through: hoisted out of
+    // the matrix loop they would sit in registers through every iteration phase)
+    int tid_l = tid;
+    asm volatile("" : "+v"(tid_l));
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
-      const int idx = tid + c * kThreads;
+    for (int c = 0; c < CH; ++c) {
+      const int idx = tid_l + c * kThreads;
       raw[c] = make_uint4(0, 0, 0, 0);
       if (idx < nchunks) {
         const int r = idx / cpr, c0 = (idx - r * cpr) * 8;  // input row, first input column
@@ -75,8 +83,19 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
         }
       }
     }
+  };
+  if (kPrefetch && vec && (int64_t)blockIdx.x < batch) fetch(blockIdx.x);
+
+  for (int64_t mat = blockIdx.x; mat < batch; mat += gridDim.x) {
+  const T* src = in + mat * mat_elems;
+  bf16_t* dst = out + mat * mat_elems;
+
+  // ---- (raw bf16 values in registers), sum of squares, scale, store to LDS
+  float ss = 0.f;
+  if (vec) {
+    if (!kPrefetch) fetch(mat);
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
+    for (int c = 0; c < CH; ++c) {
       const uint32_t w[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -91,9 +110,11 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
     __syncthreads();
     const float total = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
     const float sc = 1.0f / (sqrtf(total) * norm_scale + eps);
+    int tid_l = tid;
+    asm volatile("" : "+v"(tid_l));
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
-      const int idx = tid + c * kThreads;
+    for (int c = 0; c < CH; ++c) {
+      const int idx = tid_l + c * kThreads;
       if (idx < nchunks) {
         const int r = idx / cpr, c0 = (idx - r * cpr) * 8;
         const uint32_t w[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
@@ -116,6 +137,8 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
         }
       }
     }
+    // the registers are free again: the next matrix of this workgroup travels while this one is iterated
+    if (kPrefetch && mat + gridDim.x < batch) fetch(mat + gridDim.x);
   } else {
     for (int idx = tid; idx < 64 * n_pad; idx += kThreads) {
       const int i = idx / n_pad, j = idx - i * n_pad;  // X[i][j]
@@ -164,6 +187,9 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
   const bool three = ag < 2;
   float* Ps = (float*)(Bs + 64 * ap);  // partial sums of the odd-k wavefronts: [group][tile][lane] f32x4
 
+  // wide result with 16-byte aligned rows: written out from LDS as whole rows after the last iteration
+  const bool out_rows = !tall && (cols % 8 == 0) && ((((uintptr_t)out) & 15) == 0);
+  auto last_it = [&](int it) { return it == co.n - 1; };
   for (int it = 0; it < co.n; ++it) {
     const float a = co.c[it][0], b = co.c[it][1], c = co.c[it][2];
     // ---- A = X X^T
@@ -174,23 +200,54 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
       const char* p0 = Xs + (rb0 * 16 + r16) * xp + kq * 16;
       const char* p1 = Xs + (rb1 * 16 + r16) * xp + kq * 16;
       const char* p2 = Xs + (rb2 * 16 + r16) * xp + kq * 16;
+      // fragments of the step after next are requested before the MFMAs of this one (two register sets)
       if (three) {
-#pragma unroll 2
-        for (int s = akh; s < nstep; s += 2) {
-          const bf16x8 f0 = *(const bf16x8*)(p0 + s * 64);
-          const bf16x8 f1 = *(const bf16x8*)(p1 + s * 64);
-          const bf16x8 f2 = *(const bf16x8*)(p2 + s * 64);
-          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f0, acc[0], 0, 0, 0);
-          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f1, acc[1], 0, 0, 0);
-          acc[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f2, acc[2], 0, 0, 0);
+        bf16x8 f[2][3];
+        f[0][0] = *(const bf16x8*)(p0 + akh * 64);
+        f[0][1] = *(const bf16x8*)(p1 + akh * 64);
+        f[0][2] = *(const bf16x8*)(p2 + akh * 64);
+        int s = akh;
+        for (; s + 2 < nstep; s += 4) {
+          f[1][0] = *(const bf16x8*)(p0 + (s + 2) * 64);
+          f[1][1] = *(const bf16x8*)(p1 + (s + 2) * 64);
+          f[1][2] = *(const bf16x8*)(p2 + (s + 2) * 64);
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][0], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][1], acc[1], 0, 0, 0);
+          acc[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][2], acc[2], 0, 0, 0);
+          if (s + 4 < nstep) {
+            f[0][0] = *(const bf16x8*)(p0 + (s + 4) * 64);
+            f[0][1] = *(const bf16x8*)(p1 + (s + 4) * 64);
+            f[0][2] = *(const bf16x8*)(p2 + (s + 4) * 64);
+          }
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[1][0], f[1][0], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[1][0], f[1][1], acc[1], 0, 0, 0);
+          acc[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[1][0], f[1][2], acc[2], 0, 0, 0);
+        }
+        if (s < nstep) {  // an odd number of steps for this wavefront: the last one sits in set 0
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][0], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][1], acc[1], 0, 0, 0);
+          acc[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][2], acc[2], 0, 0, 0);
         }
       } else {
-#pragma unroll 2
-        for (int s = akh; s < nstep; s += 2) {
-          const bf16x8 f0 = *(const bf16x8*)(p0 + s * 64);
-          const bf16x8 f1 = *(const bf16x8*)(p1 + s * 64);
-          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f0, acc[0], 0, 0, 0);
-          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, f1, acc[1], 0, 0, 0);
+        bf16x8 f[2][2];
+        f[0][0] = *(const bf16x8*)(p0 + akh * 64);
+        f[0][1] = *(const bf16x8*)(p1 + akh * 64);
+        int s = akh;
+        for (; s + 2 < nstep; s += 4) {
+          f[1][0] = *(const bf16x8*)(p0 + (s + 2) * 64);
+          f[1][1] = *(const bf16x8*)(p1 + (s + 2) * 64);
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][0], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][1], acc[1], 0, 0, 0);
+          if (s + 4 < nstep) {
+            f[0][0] = *(const bf16x8*)(p0 + (s + 4) * 64);
+            f[0][1] = *(const bf16x8*)(p1 + (s + 4) * 64);
+          }
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[1][0], f[1][0], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[1][0], f[1][1], acc[1], 0, 0, 0);
+        }
+        if (s < nstep) {
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][0], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[0][0], f[0][1], acc[1], 0, 0, 0);
         }
       }
       float* pp = Ps + ((ag * 3) * 64 + lane) * 4;
@@ -258,23 +315,33 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
       // The MFMA operands are swapped (X fragment first): the accumulators then hold (B X)^T tiles, i.e.
       // lane l owns output row i*32 + l%32 and, per group of four accumulator elements, four consecutive
       // output columns -- one 8-byte store per group instead of four 2-byte ones.
-      for (int jt = wave; jt < n_pad / 32; jt += 8) {
+      const int ntile = n_pad / 32;
+      auto load_tile = [&](int jt, s16x4 (&lo)[4], s16x4 (&hi)[4]) {
+        const char* px = Xs + trow * xp + (jt * 32 + tcol) * 2;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          lo[s] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS3(px + (s * 16) * xp));
+          hi[s] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS3(px + (s * 16 + 4) * xp));
+        }
+      };
+      auto do_tile = [&](int jt, s16x4 (&clo)[4], s16x4 (&chi)[4], s16x4 (&nlo)[4], s16x4 (&nhi)[4]) {
         f32x16 acc[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
-        const char* px = Xs + trow * xp + (jt * 32 + tcol) * 2;
+        // the next column tile's fragments are requested before this tile's MFMAs and stores
+        if (jt + 8 < ntile) load_tile(jt + 8, nlo, nhi);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS3(px + (s * 16) * xp));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS3(px + (s * 16 + 4) * xp));
-          const bf16x8 fx = join_tr(lo, hi);
+          const bf16x8 fx = join_tr(clo[s], chi[s]);
           acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fx, fB[0][s], acc[0], 0, 0, 0);
           acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fx, fB[1][s], acc[1], 0, 0, 0);
         }
         const int col0 = jt * 32 + 4 * fhalf;  // + 8 * g: first of four consecutive columns
-        if (!last) {
+        // The last X' of a wide matrix goes through LDS like the others and leaves as whole rows below (16 bytes
+        // per lane): stored from the accumulators it would be 8-byte pieces 1.5 KB apart.
+        if (!last || out_rows) {
 #pragma unroll
           for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -321,9 +388,24 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
               }
           }
         }
+      };
+      s16x4 lo0[4], hi0[4], lo1[4], hi1[4];
+      if (wave < ntile) load_tile(wave, lo0, hi0);
+      for (int jt = wave; jt < ntile; jt += 16) {
+        do_tile(jt, lo0, hi0, lo1, hi1);
+        if (jt + 8 < ntile) do_tile(jt + 8, lo1, hi1, lo0, hi0);
       }
     }
     __syncthreads();
+    if (last_it(it) && out_rows) {
+      // X [m][n] in LDS -> dst [rows][cols], 16 bytes per lane, lanes side by side along a row
+      const int cpr8 = cols / 8;
+      for (int idx = tid; idx < m * cpr8; idx += kThreads) {
+        const int r = idx / cpr8, c8 = idx - r * cpr8;
+        *(uint4*)(dst + (int64_t)r * cols + c8 * 8) = *(const uint4*)(Xs + r * xp + c8 * 16);
+      }
+      __syncthreads();  // X is rewritten by the next matrix
+    }
   }
   if (co.n == 0) {  // normalisation only
     for (int idx = tid; idx < m * n; idx += kThreads) {
@@ -331,7 +413,9 @@ __global__ __launch_bounds__(kThreads) void ns_small_kernel(const T* __restrict_
       const int64_t g = tall ? (int64_t)j * cols + i : (int64_t)i * cols + j;
       dst[g] = *(const bf16_t*)(Xs + i * xp + j * 2);
     }
+    __syncthreads();  // X is rewritten by the next matrix
   }
+  }  // matrices of this workgroup
 }
 
 bool ns_small_fits(int rows, int cols) {
@@ -347,17 +431,31 @@ hipError_t launch_ns_small(const void* in, int in_dtype, bf16_t* out, int batch,
   const int n = rows < cols ? cols : rows;
   const int n_pad = (n + 63) / 64 * 64;
   const size_t bytes = (size_t)64 * (n_pad * 2 + 16) + 2 * 64 * (64 * 2 + 16) + kPartialBytes;
-  static std::atomic<uint64_t> done_bf16{0}, done_f32{0};
-  if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<bf16_t>, kMaxLds, done_bf16))
-    return e;
-  if (hipError_t e = set_max_dynamic_lds_once((const void*)ns_small_kernel<float>, kMaxLds, done_f32))
-    return e;
-  if (in_dtype == 0)
-    hipLaunchKernelGGL(ns_small_kernel<bf16_t>, dim3(batch), dim3(kThreads), bytes, st, (const bf16_t*)in, out, rows,
-                       cols, n_pad, co, norm_scale, eps);
-  else
-    hipLaunchKernelGGL(ns_small_kernel<float>, dim3(batch), dim3(kThreads), bytes, st, (const float*)in, out, rows,
-                       cols, n_pad, co, norm_scale, eps);
+  static std::atomic<uint64_t> done[4];
+  const bool small = n_pad * 8 <= 12 * kThreads;
+  const void* kern = in_dtype == 0 ? (small ? (const void*)ns_small_kernel<bf16_t, 12> : (const void*)ns_small_kernel<bf16_t, kMaxChunks>)
+                                   : (small ? (const void*)ns_small_kernel<float, 12> : (const void*)ns_small_kernel<float, kMaxChunks>);
+  if (hipError_t e = set_max_dynamic_lds_once(kern, kMaxLds, done[(in_dtype == 0 ? 0 : 2) + (small ? 0 : 1)])) return e;
+  // one workgroup per CU (the LDS footprint admits no second one), each walking its share of the batch
+  static std::atomic<int> cu_count[64];
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  int cus = cu_count[dev & 63].load(std::memory_order_relaxed);
+  if (cus == 0) {
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) return e;
+    if (cus <= 0) return hipErrorInvalidValue;
+    cu_count[dev & 63].store(cus, std::memory_order_relaxed);
+  }
+  const int grid = batch < cus ? batch : cus;
+#define SMALL_LAUNCH(T, CHN)                                                                                   \
+  hipLaunchKernelGGL((ns_small_kernel<T, CHN>), dim3(grid), dim3(kThreads), bytes, st, (const T*)in, out, batch, \
+                     rows, cols, n_pad, co, norm_scale, eps)
+  if (in_dtype == 0) {
+    if (small) SMALL_LAUNCH(bf16_t, 12); else SMALL_LAUNCH(bf16_t, kMaxChunks);
+  } else {
+    if (small) SMALL_LAUNCH(float, 12); else SMALL_LAUNCH(float, kMaxChunks);
+  }
+#undef SMALL_LAUNCH
   return hipGetLastError();
 }
 
