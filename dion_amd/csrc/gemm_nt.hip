@@ -15,8 +15,9 @@
 // dion/newton_schulz_triton.py:557-563.
 //
 // Kernel structure: one workgroup per BM x BN output tile, WM x WN wavefronts (64 lanes) each
-// owning a (BM/WM) x (BN/WN) sub-tile as 32x32 MFMA accumulators
-// (v_mfma_f32_32x32x16_bf16).  Operand tiles reach a two-slot LDS ring through direct-to-LDS
+// owning a (BM/WM) x (BN/WN) sub-tile as 16x16 MFMA accumulators (v_mfma_f32_16x16x32_bf16: per
+// FLOP half the accumulator register traffic of the 32x32x16 form, which on this power-limited part is
+// worth 5 % of clock).  Operand tiles reach a two-slot LDS ring through direct-to-LDS
 // loads (global_load_lds_dwordx4, no VGPR staging); XOR swizzles keep the LDS writes and the
 // fragment reads bank-conflict free.
 #include <type_traits>
@@ -48,8 +49,11 @@ struct TileCfg {
   static constexpr int Q_LOADS = BN / ROWS_PER_LOAD;
   static constexpr int LOADS_PER_STAGE = P_LOADS + Q_LOADS;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
-  static constexpr int TM = WTM / 32, TN = WTN / 32;
-  static constexpr int KK = BK / 16;
+  static constexpr int TM = WTM / 16, TN = WTN / 16;  // 16 x 16 accumulator tiles of a wavefront tile
+  static constexpr int ST = BK / 32;                  // 32-deep MFMA steps per slab
+  // The MFMAs of a step run in halves of sixteen: four A fragments against the four B fragments.
+  static constexpr int HALVES = TM / 4;
+  static_assert(TN == 4 && (TM == 4 || TM == 8) && ST == 2, "wavefront tiles of 64 or 128 rows by 64 columns, 64-deep slabs");
   // gfx950 LDS: 64 banks x 4 B = 256-byte bank rows, and a ds_read_b128 is served 16 lanes at a
   // time.  16 consecutive tile rows must therefore land in 16 distinct 16-byte slots of a bank
   // row: the 256/(2*BK) tile rows that share a bank row take one swizzle value.
@@ -75,32 +79,48 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
-// The fragment reads of a 16-wide k slice are issued, one behind each MFMA of the slice before, in the
-// order the MFMAs (row-major over the TM x TN accumulator tiles) first need them: A0, B0..B(TN-1),
-// A1..A(TM-1).  Every read is an assembly statement and so is every wait: the LDS returns in order, so
-// "all but the newest N LDS instructions have returned" is exactly "the fragments MFMA q needs are in
-// their registers", with N counted here from the issue order -- the reads of the slice issued after the
-// later of the two fragments q needs, plus the reads of the next slice issued ahead of q.  (Left to the
-// compiler, every slice starts with a wait for all six reads, the last of which was issued two MFMAs
-// earlier.)  A K-major fragment is two transposing reads.
-template <int TM, int TN, bool QK>
+// Issue order of the fragment reads.  A 32-deep step of a wavefront tile is HALVES halves of sixteen MFMAs
+// (A fragment i = q / 4 against B fragment j = q % 4); a slab is ST steps, i.e. P = HALVES * ST halves.  While
+// the MFMAs of one half issue, the fragments of the next half are requested behind them:
+//   next half starts a step:   A0 B0 B1 B2 B3 A1 A2 A3 of that step, read r behind MFMA r, the order in
+//                              which the MFMAs first need them;
+//   next half is a second half: its A fragments 4..7, read r behind MFMA 4 r + 1 (B stays).
+// Every fragment is requested fifteen or more MFMAs before its first use.  Every read is an assembly
+// statement and so is every wait: the LDS returns in order, so "all but the newest N LDS instructions have
+// returned" is exactly "the fragments MFMA q needs are in their registers", with N counted here from the
+// issue order -- the LDS instructions issued after the later of the two fragments q needs.  (Left to the
+// compiler, every group of MFMAs starts with a wait for all outstanding reads, the last of which was
+// issued two MFMAs earlier.)  A K-major B fragment is two transposing reads.
+template <int HALVES, int ST, bool QK>
 struct FragSched {
-  static constexpr int NR = TM + TN, NM = TM * TN;
-  static constexpr int RPM = (NR + NM - 1) / NM;  // reads slotted behind each MFMA
-  static constexpr int instrs(int r) { return (QK && r >= 1 && r <= TN) ? 2 : 1; }
-  static constexpr int pos_a(int i) { return i == 0 ? 0 : TN + i; }
-  static constexpr int pos_b(int j) { return 1 + j; }
-  // LDS instructions that may still be outstanding when MFMA q of a slice issues
-  static constexpr int allowed(int q) {
-    const int i = q / TN, j = q % TN;
-    const int need = pos_a(i) > pos_b(j) ? pos_a(i) : pos_b(j);
-    int n = 0;
-    for (int r = need + 1; r < NR; ++r) n += instrs(r);
-    const int issued = q * RPM < NR ? q * RPM : NR;
-    for (int r = 0; r < issued; ++r) n += instrs(r);
-    return n;
+  static constexpr int P = HALVES * ST, NM = 16;
+  static constexpr bool issues_full(int hp) { return (hp + 1) % HALVES == 0; }
+  static constexpr int read_behind(int hp, int q) {
+    if (issues_full(hp)) return q < 8 ? q : -1;
+    return (q % 4 == 1) ? q / 4 : -1;
   }
-  static_assert(allowed(NM - 1) < 16, "lgkmcnt is a four-bit field");
+  static constexpr int instrs_full(int r) { return (QK && r >= 1 && r <= 4) ? 2 : 1; }
+  static constexpr int lds_behind(int hp, int q) {
+    const int r = read_behind(hp, q);
+    if (r < 0) return 0;
+    return issues_full(hp) ? instrs_full(r) : 1;
+  }
+  // LDS instructions that may still be outstanding when MFMA q of half hp issues
+  static constexpr int allowed(int hp, int q) {
+    const int i = q / 4, j = q % 4;
+    const int prev = (hp + P - 1) % P;
+    int need_q = 0;  // MFMA of the half before behind which the later of q's two fragments was requested
+    if (hp % HALVES == 0) {
+      const int ra = i == 0 ? 0 : 4 + i, rb = 1 + j;
+      need_q = ra > rb ? ra : rb;
+    } else {
+      need_q = 4 * i + 1;  // A fragment 4 + i; the B fragments arrived a half earlier
+    }
+    int n = 0;
+    for (int qq = need_q + 1; qq < NM; ++qq) n += lds_behind(prev, qq);
+    for (int qq = 0; qq < q; ++qq) n += lds_behind(hp, qq);
+    return n < 15 ? n : 15;  // lgkmcnt is a four-bit field; waiting for more than needed is harmless
+  }
 };
 
 // Fragment wait: an asm statement that takes the fragments it guards as read-write operands, so that to
@@ -187,6 +207,16 @@ __device__ __forceinline__ void pipeline_barrier() {
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
+// A pointer every lane holds the same value of, moved to scalar registers (where the compiler cannot
+// prove uniformity it wraps each buffer access in a loop over the distinct values).
+template <typename T>
+__device__ __forceinline__ T* uniform_ptr(T* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (T*)(((uint64_t)hi << 32) | lo);
+}
+
 // Parameter accesses of the fused update go through buffer instructions: a descriptor based at the
 // wavefront's tile of X (wave-uniform, scalar registers), a wave-uniform byte offset per instruction
 // (scalar) and one per-lane byte offset shared by all accesses -- no 64-bit address per row in vector
@@ -258,13 +288,11 @@ struct PostSel<2> {
 template <class Cfg, bool HAS_D, bool HAS_C, bool HAS_CT, bool QK = false, int POST = 0>
 __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, const typename PostSel<POST>::arg post) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
-  constexpr int TM = Cfg::TM, TN = Cfg::TN, KK = Cfg::KK, NSTAGE = Cfg::NSTAGE;
-  constexpr int NM = TM * TN;  // MFMAs per 16-wide k slice
-  constexpr int NR = TM + TN;  // fragment reads per slice
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, ST = Cfg::ST, HALVES = Cfg::HALVES, NSTAGE = Cfg::NSTAGE;
+  constexpr int HP = HALVES * ST;  // halves (sixteen MFMAs each) per slab
+  constexpr int NM = 16;
   constexpr int LPS = Cfg::LOADS_PER_STAGE;
-  static_assert(KK % 2 == 0, "fragment double buffer needs an even slice count per stage");
-  constexpr int RPM = (NR + NM - 1) / NM;    // fragment reads slotted behind each MFMA
-  constexpr int LPM = (LPS + NM - 1) / NM;   // refill loads slotted behind each MFMA
+  static_assert(LPS <= NM / 2, "one refill load behind every second MFMA of a slab's last half");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int tid = threadIdx.x;
@@ -328,8 +356,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   const int qk_chunk = ((((tid % QCPR) >> 2) ^ (qk_row & 3)) << 2) | (tid & 3);
   const char* gQ = QK ? (const char*)(p.Q + (int64_t)b * p.strideQ + tj * BN)
                       : (const char*)(p.Q + (int64_t)b * p.strideQ + (int64_t)(tj * BN) * p.ldq);
-  const uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
-  const uint32_t offQ = QK ? (uint32_t)(qk_row * p.ldq + qk_chunk * 8) * 2u
+  uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
+  uint32_t offQ = QK ? (uint32_t)(qk_row * p.ldq + qk_chunk * 8) * 2u
                            : (uint32_t)(ld_row * p.ldq + ld_chunk * 8) * 2u;
   const uint32_t stepP = (uint32_t)(Cfg::ROWS_PER_LOAD * p.ldp) * 2u;
   const uint32_t stepQ = (uint32_t)((QK ? QROWS_PER_LOAD : Cfg::ROWS_PER_LOAD) * p.ldq) * 2u;
@@ -351,70 +379,79 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
     if (one_operand && j >= Cfg::P_LOADS) return;
     const int k = kt < KT ? kt : KT - 1;
     char* l = lds + buf * Cfg::P_BYTES + wave * (64 * 16);
+    // Address = wave-uniform 64-bit base (scalar registers; slab and load index folded in) + one 32-bit
+    // per-lane offset per operand.  The empty asm (re)defines both right at the load, so that the
+    // instruction is selected in its scalar-base form: left to the compiler, base and offset are
+    // folded and hoisted out of the loop as a 64-bit address in vector registers per load.
     if (j < Cfg::P_LOADS) {
-      const char* src = gP + (int64_t)k * (BK * 2) + (offP + j * stepP);
-      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
+      const char* src = gP + (int64_t)k * (BK * 2) + (uint64_t)j * stepP;
+      asm volatile("" : "+s"(src), "+v"(offP));
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src + offP), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
     } else {
       const int jq = j - Cfg::P_LOADS;
-      const char* src = gQ + k * slabQ + (offQ + jq * stepQ);
-      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + NSTAGE * Cfg::P_BYTES + jq * (Cfg::NT * 16)),
+      const char* src = gQ + k * slabQ + (uint64_t)jq * stepQ;
+      asm volatile("" : "+s"(src), "+v"(offQ));
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src + offQ), LDS_PTR(l + NSTAGE * Cfg::P_BYTES + jq * (Cfg::NT * 16)),
                                        16, 0, 0);
     }
   };
 
-  // ---- LDS -> register fragment addressing (per lane, per 16-wide k slice).
+  // ---- LDS -> register fragment addressing.  A fragment of v_mfma_f32_16x16x32_bf16: lane l holds row (or
+  // column) l % 16 and the eight reduction indices 8 * (l / 16) .. + 7 of a 32-deep step -- one 16-byte chunk.
   const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
-  const int frow = lane & 31;
-  const int fhalf = lane >> 5;
-  const int fswz = (frow / Cfg::SWZ_DIV) % Cfg::CPR;
-  uint32_t aoff[KK], boff[KK];
+  const int l16 = lane & 15, quad = lane >> 4;
+  const int fswz = (l16 / Cfg::SWZ_DIV) % Cfg::CPR;  // (every fragment's first row is a multiple of 16)
+  uint32_t aoff[ST], boff[ST];
 #pragma unroll
-  for (int kk = 0; kk < KK; ++kk) {
-    const int chunk = ((kk * 2 + fhalf) ^ fswz) * 16;
-    aoff[kk] = lds_base + (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + chunk);
-    boff[kk] = lds_base + (uint32_t)((one_operand ? 0 : NSTAGE * Cfg::P_BYTES) + (wn * Cfg::WTN + frow) * (BK * 2) + chunk);
+  for (int st = 0; st < ST; ++st) {
+    const int chunk = ((st * 4 + quad) ^ fswz) * 16;
+    aoff[st] = lds_base + (uint32_t)((wm * Cfg::WTM + l16) * (BK * 2) + chunk);
+    boff[st] = lds_base + (uint32_t)((one_operand ? 0 : NSTAGE * Cfg::P_BYTES) + (wn * Cfg::WTN + l16) * (BK * 2) + chunk);
   }
 
-  // QK fragments: within a 16-lane group, lane 4r+q addresses row r / 4-element piece q of a 4x16
-  // block; the transposing read hands lane i column i.  Lanes 0-31 take k 0..7 of the slice (two
-  // reads of 4 rows), lanes 32-63 k 8..15; column = lane % 32.
+  // QK fragments: a transposing read hands each 16-lane group a 4 (reduction index) x 16 (column) block, lane i
+  // its column i; within the group, lane 4r+q addresses row r / 4-element piece q of the block.  Group g takes
+  // reduction indices 8 g .. 8 g + 7 of the step (two reads of 4 rows); the 16 columns of fragment j are half
+  // of a 64-byte group of the tile row, which the swizzle keys on the row's index modulo 4.
   uint32_t qoff[TN];
   if (QK) {
-    const int g16 = lane >> 4, t16 = lane & 15;
+    const int t16 = lane & 15;
 #pragma unroll
-    for (int r = 0; r < TN; ++r)
-      qoff[r] = lds_base + (uint32_t)(NSTAGE * Cfg::P_BYTES + (8 * (g16 >> 1) + (t16 >> 2)) * (BN * 2) +
-                                      ((((wn * Cfg::WTN + r * 32) >> 5) ^ (t16 >> 2)) << 6) + (g16 & 1) * 32 +
+    for (int j = 0; j < TN; ++j)
+      qoff[j] = lds_base + (uint32_t)(NSTAGE * Cfg::P_BYTES + (8 * quad + (t16 >> 2)) * (BN * 2) +
+                                      ((((wn * Cfg::WTN + j * 16) >> 5) ^ (t16 >> 2)) << 6) + (j & 1) * 32 +
                                       (t16 & 3) * 8);
   }
 
-  typedef FragSched<TM, TN, QK> FS;
-  bf16x8 fa[2][TM], fb[2][TN];
-  // Fragment read r (0..NR-1, order A0, B0..B(TN-1), A1..A(TM-1)) of slice kk of ring slot buf into
-  // fragment set f; all four are compile-time constants and end up in the instruction's offset field.
-  auto read_frag = [&](auto bufc, auto kkc, auto fc, auto rc) {
-    constexpr int buf = decltype(bufc)::value, kk = decltype(kkc)::value, f = decltype(fc)::value,
-                  r = decltype(rc)::value;
-    if constexpr (r == 0 || r > TN) {
-      constexpr int i = r == 0 ? 0 : r - TN;
-      lds_read16<buf * Cfg::P_BYTES + i * (32 * BK * 2)>(fa[f][i], aoff[kk]);
+  typedef FragSched<HALVES, ST, QK> FS;
+  // A fragments: two sets of four, alternating by half; B fragments: two sets of TN, alternating by step
+  bf16x8 fa[2][4], fb[2][TN];
+  // Read r of the fragments half hn (0..HP-1) of ring slot buf needs: the first half of a step takes
+  // A0 B0 B1 B2 B3 A1 A2 A3 (r = 0..7), a second half its A fragments 4..7 (r = 0..3).  All compile-time
+  // constants, which end up in the instruction's offset field.
+  auto read_frag = [&](auto bufc, auto hnc, auto rc) {
+    constexpr int buf = decltype(bufc)::value, hn = decltype(hnc)::value, r = decltype(rc)::value;
+    constexpr int st = hn / HALVES, part = hn % HALVES, fs = hn & 1, bs = st & 1;
+    if constexpr (part != 0) {
+      lds_read16<buf * Cfg::P_BYTES + (4 + r) * (16 * BK * 2)>(fa[fs][r], aoff[st]);
+    } else if constexpr (r == 0 || r > 4) {
+      constexpr int i = r == 0 ? 0 : r - 4;
+      lds_read16<buf * Cfg::P_BYTES + i * (16 * BK * 2)>(fa[fs][i], aoff[st]);
     } else if constexpr (QK) {
       constexpr int j = r - 1;
-      lds_read_tr<buf * Cfg::Q_BYTES + kk * (16 * BN * 2), 4 * BN * 2>(fb[f][j], qoff[j]);
+      lds_read_tr<buf * Cfg::Q_BYTES + st * (32 * BN * 2), 4 * BN * 2>(fb[bs][j], qoff[j]);
     } else {
       constexpr int j = r - 1;
-      lds_read16<buf * Cfg::Q_BYTES + j * (32 * BK * 2)>(fb[f][j], boff[kk]);
+      lds_read16<buf * Cfg::Q_BYTES + j * (16 * BK * 2)>(fb[bs][j], boff[st]);
     }
   };
   typedef std::integral_constant<int, 0> ic0;
 
-  f32x16 acc[TM][TN];
+  f32x4 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // ---- prologue: fill NSTAGE-1 ring slots, wait for slab 0, read its first fragments, start the
   // last free slot.
@@ -423,44 +460,40 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 #pragma unroll
     for (int j = 0; j < LPS; ++j) issue_load(s, s, j);
   pipeline_barrier<(NSTAGE - 2) * LPS>();
-  static_for<0, NR>([&](auto rc) { read_frag(ic0(), ic0(), ic0(), rc); });
+  static_for<0, 8>([&](auto rc) { read_frag(ic0(), ic0(), rc); });
 #pragma unroll
   for (int j = 0; j < LPS; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
   __builtin_amdgcn_sched_barrier(0);
 
-  // ---- main loop.  Slices run back to back across slab boundaries: while the MFMAs of one slice
-  // issue, the fragment reads of the next slice (and, on the last slice of a slab, the refill of
-  // the slot that slab occupied) are slotted one behind each MFMA.  sched_barrier pins that order.
-  // KT is a multiple of NSTAGE (launcher checks) so ring slots are compile-time constants.
+  // ---- main loop.  Halves run back to back across slab boundaries: while the MFMAs of one half issue, the
+  // fragment reads of the next half (and, in the last half of a slab, the refill of the slot that slab
+  // occupied) are slotted behind them.  sched_barrier pins that order.  KT is a multiple of NSTAGE
+  // (launcher checks) so ring slots are compile-time constants.
   for (int kt0 = 0; kt0 < KT; kt0 += NSTAGE) {
-    static_for<0, NSTAGE * KK>([&](auto skc) {
-      constexpr int s = decltype(skc)::value / KK, kk = decltype(skc)::value % KK;
-      constexpr int cur = kk & 1, nxt = cur ^ 1;
-      constexpr bool last = (kk == KK - 1);
+    static_for<0, NSTAGE * HP>([&](auto shc) {
+      constexpr int s = decltype(shc)::value / HP, hp = decltype(shc)::value % HP;
+      constexpr int st = hp / HALVES, part = hp % HALVES, fs = hp & 1, bs = st & 1;
+      constexpr bool last = (hp == HP - 1);
       // slab kt+1 landed, slab kt fully read
       if constexpr (last) pipeline_barrier<(NSTAGE - 2) * LPS>();
       static_for<0, NM>([&](auto qc) {
-        constexpr int q = decltype(qc)::value, i = q / TN, j = q % TN;
-        frag_wait<FS::allowed(q)>(fa[cur][i], fb[cur][j]);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+        constexpr int q = decltype(qc)::value, i = q / 4, j = q % 4;
+        frag_wait<FS::allowed(hp, q)>(fa[fs][i], fb[bs][j]);
+        acc[part * 4 + i][j] =
+            __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[fs][i], fb[bs][j], acc[part * 4 + i][j], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        static_for<q * RPM, ((q + 1) * RPM < NR ? (q + 1) * RPM : NR)>([&](auto rc) {
-          if constexpr (last)
-            read_frag(std::integral_constant<int, (s + 1) % NSTAGE>(), ic0(), std::integral_constant<int, nxt>(), rc);
-          else
-            read_frag(std::integral_constant<int, s>(), std::integral_constant<int, kk + 1>(),
-                      std::integral_constant<int, nxt>(), rc);
-        });
-        if constexpr (last) {
-#pragma unroll
-          for (int jl = q * LPM; jl < (q + 1) * LPM && jl < LPS; ++jl) issue_load(kt0 + s + NSTAGE, s, jl);
+        if constexpr (FS::read_behind(hp, q) >= 0) {
+          typedef std::integral_constant<int, FS::read_behind(hp, q)> rc;
+          if constexpr (last) read_frag(std::integral_constant<int, (s + 1) % NSTAGE>(), ic0(), rc());
+          else read_frag(std::integral_constant<int, s>(), std::integral_constant<int, hp + 1>(), rc());
         }
+        if constexpr (last && (q & 1) && q / 2 < LPS) issue_load(kt0 + s + NSTAGE, s, q / 2);
         __builtin_amdgcn_sched_barrier(0);
       });
     });
   }
   wait_vmcnt<0>();  // drain the redundant tail refills before LDS is reused / the wave exits
-  // The read-ahead of the last slice issued reads whose results nobody uses.  The compiler does not know
+  // The read-ahead of the last half issued reads whose results nobody uses.  The compiler does not know
   // they are in flight; were their destination registers dead here, it would hand them to whatever comes
   // next (the lane index, store addresses) and a read landing late would overwrite that.  So: wait for the
   // LDS queue to drain, and only then let go of the fragment registers -- the empty asm statements below
@@ -469,26 +502,26 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 #pragma unroll
   for (int f = 0; f < 2; ++f) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) asm volatile("" ::"v"(fa[f][i]));
+    for (int i = 0; i < 4; ++i) asm volatile("" ::"v"(fa[f][i]));
 #pragma unroll
     for (int j = 0; j < TN; ++j) asm volatile("" ::"v"(fb[f][j]));
   }
 
-  // ---- epilogue.  Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4,
-  // column l%32 of its 32x32 tile.  Whole tiles are stored: destinations are padded to the tile.
-  // C goes out straight from registers (32 lanes x 2 B = one 64-byte run per row).  The transposed
-  // copy would be 8-byte pieces scattered over 32 rows per instruction, so it is staged through
-  // LDS ([column][row], this wavefront's private slice) and stored as 16 bytes per lane with
+  // ---- epilogue.  Accumulator element e of lane l holds row 4 * (l / 16) + e, column l % 16 of its 16 x 16
+  // tile.  Whole tiles are stored: destinations are padded to the tile.  C goes out straight from registers
+  // (16 lanes x 2 B = one 32-byte run per row and instruction, neighbouring tiles completing the lines).
+  // The transposed copy would be 8-byte pieces scattered over 16 rows per instruction, so it is staged
+  // through LDS ([column][row], this wavefront's private slice) and stored as 16 bytes per lane with
   // 256-byte runs per row.
   const float alpha = gemm_alpha(p, b), beta = p.beta;
   const int row_base = ti * BM + wm * Cfg::WTM;
   const int col_base = tj * BN + wn * Cfg::WTN;
   const bool mirror = HAS_CT && !(p.tri && ti == tj);  // a diagonal tile is its own mirror
-  const bf16_t* Dp = HAS_D ? p.D + (int64_t)b * p.strideD + (int64_t)(row_base + 4 * fhalf) * p.ldd +
-                                 col_base + frow
+  const bf16_t* Dp = HAS_D ? p.D + (int64_t)b * p.strideD + (int64_t)(row_base + 4 * quad) * p.ldd +
+                                 col_base + l16
                            : nullptr;
   bf16_t* Cp = (HAS_C && POST == 0) ? p.C + (int64_t)b * p.strideC +
-                                           (int64_t)(row_base + 4 * fhalf) * p.ldc + col_base + frow
+                                           (int64_t)(row_base + 4 * quad) * p.ldc + col_base + l16
                                      : nullptr;
   const int ldd = p.ldd, ldc = p.ldc, ldct = p.ldct;
   typedef typename PostSel<POST>::xt XT;
@@ -511,42 +544,41 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   if constexpr (POST != 0 && HAS_C) {
     // Update X[row][col] from registers.  The products are rounded to bf16 first, two per register,
     // which frees half of the accumulator registers: the parameter values of half a wavefront tile
-    // are then loaded in one go (one round trip to memory per half, not one per 32x32 tile).
-    // 32 lanes x one element: a 128-byte (fp32) or 64-byte (bf16) run of X per row.
-    uint32_t pk[TM][TN][8];
+    // are then loaded in one go (one round trip to memory per half, not one per tile).
+    // 16 lanes x one element: a 64-byte (fp32) or 32-byte (bf16) run of X per row.
+    uint32_t pk[TM][TN][2];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int q = 0; q < 8; ++q)
+        for (int q = 0; q < 2; ++q)
           pk[i][j][q] = pack_bf16x2(alpha * acc[i][j][2 * q], alpha * acc[i][j][2 * q + 1]);
-    const __amdgpu_buffer_rsrc_t xr = bx_resource(xmat + (int64_t)row_base * ldc + col_base);
-    const int xl = (4 * fhalf * ldc + frow) * (int)sizeof(XT);  // per lane
-    constexpr int HM = TM >= 2 ? TM / 2 : 1;
+    const __amdgpu_buffer_rsrc_t xr = bx_resource(uniform_ptr(xmat + (int64_t)row_base * ldc + col_base));
+    const int xl = (4 * quad * ldc + l16) * (int)sizeof(XT);  // per lane
+    constexpr int HM = TM / 2;
     auto run = [&](auto caut) {
       constexpr int CAUT = decltype(caut)::value;
 #pragma unroll
       for (int i0 = 0; i0 < TM; i0 += HM) {
-        float xv[HM][TN][16];
+        float xv[HM][TN][4];
 #pragma unroll
         for (int ii = 0; ii < HM; ++ii)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-              xv[ii][j][r] = bx_load<XT>(
-                  xr, xl, (((i0 + ii) * 32 + (r >> 2) * 8 + (r & 3)) * ldc + j * 32) * (int)sizeof(XT));
+            for (int e = 0; e < 4; ++e)
+              xv[ii][j][e] = bx_load<XT>(xr, xl, (((i0 + ii) * 16 + e) * ldc + j * 16) * (int)sizeof(XT));
 #pragma unroll
         for (int ii = 0; ii < HM; ++ii)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const uint32_t w = pk[i0 + ii][j][r >> 1];
-              const float u = __uint_as_float((r & 1) ? (w & 0xffff0000u) : (w << 16));
-              bx_store<XT>(xr, xl, (((i0 + ii) * 32 + (r >> 2) * 8 + (r & 3)) * ldc + j * 32) * (int)sizeof(XT),
-                           muon_post_one(xv[ii][j][r], u, pa, pcoeff, pb, CAUT));
+            for (int e = 0; e < 4; ++e) {
+              const uint32_t w = pk[i0 + ii][j][e >> 1];
+              const float u = __uint_as_float((e & 1) ? (w & 0xffff0000u) : (w << 16));
+              bx_store<XT>(xr, xl, (((i0 + ii) * 16 + e) * ldc + j * 16) * (int)sizeof(XT),
+                           muon_post_one(xv[ii][j][e], u, pa, pcoeff, pb, CAUT));
             }
         asm volatile("" ::: "memory");  // the next batch of loads stays behind these stores
       }
@@ -556,56 +588,47 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
     return;
   }
 
-  // The addend is loaded two 32x32 tiles at a time, one pair ahead: the loads of a pair are issued before the
-  // stores of the pair before it, so they neither wait for those stores (the memory counter retires in order)
-  // nor cost a round trip to memory per tile.
-  constexpr int GS = 2, NG = (TM * TN) / GS;
-  static_assert((TM * TN) % GS == 0, "addend pairs");
-  bf16_t dreg[HAS_D ? 2 : 1][GS][16];
-  auto load_addend = [&](int g) {
+  // The addend is loaded one row of tiles (TN tiles) at a time, one row ahead: the loads of a row are issued
+  // before the stores of the row before it, so they neither wait for those stores (the memory counter retires
+  // in order) nor cost a round trip to memory per tile.
+  bf16_t dreg[HAS_D ? 2 : 1][TN][4];
+  auto load_addend = [&](int i) {
 #pragma unroll
-    for (int s = 0; s < GS; ++s) {
-      const int i = (g * GS + s) / TN, j = (g * GS + s) % TN;
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        dreg[g & 1][s][r] = Dp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldd + j * 32];
-    }
+      for (int e = 0; e < 4; ++e) dreg[i & 1][j][e] = Dp[(int64_t)(i * 16 + e) * ldd + j * 16];
   };
   if (HAS_D) load_addend(0);
 
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
+    if (HAS_D && i + 1 < TM) load_addend(i + 1);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      float v[16];
+      float v[4];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) v[r] = alpha * acc[i][j][r];
+      for (int e = 0; e < 4; ++e) v[e] = alpha * acc[i][j][e];
       if (HAS_D) {
-        const int n = i * TN + j;
-        if (n % GS == 0 && n / GS + 1 < NG) load_addend(n / GS + 1);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) v[r] += beta * bf16_to_f32(dreg[(n / GS) & 1][n % GS][r]);
+        for (int e = 0; e < 4; ++e) v[e] += beta * bf16_to_f32(dreg[i & 1][j][e]);
       }
       if (on_diag) {
-        // element (row, col) of this 32x32 tile sits on the global diagonal
-        const int dcol = col_base + j * 32 + frow - (row_base + i * 32 + 4 * fhalf);
+        // element (row, col) of this tile sits on the global diagonal
+        const int dcol = col_base + j * 16 + l16 - (row_base + i * 16 + 4 * quad);
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (dcol == (r >> 2) * 8 + (r & 3)) v[r] += p.diag;
+        for (int e = 0; e < 4; ++e)
+          if (dcol == e) v[e] += p.diag;
       }
       if (HAS_C && POST == 0) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          Cp[(int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * ldc + j * 32] = f32_to_bf16(v[r]);
+        for (int e = 0; e < 4; ++e) Cp[(int64_t)(i * 16 + e) * ldc + j * 16] = f32_to_bf16(v[e]);
       }
       if (HAS_CT) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          uint2 pk;
-          pk.x = pack_bf16x2(v[g * 4 + 0], v[g * 4 + 1]);
-          pk.y = pack_bf16x2(v[g * 4 + 2], v[g * 4 + 3]);
-          *(uint2*)(stg + (j * 32 + frow) * Cfg::STG_PITCH + (i * 32 + g * 8 + 4 * fhalf) * 2) = pk;
-        }
+        // four consecutive rows of column j * 16 + l16: 8 bytes of the staged [column][row] tile
+        uint2 pk;
+        pk.x = pack_bf16x2(v[0], v[1]);
+        pk.y = pack_bf16x2(v[2], v[3]);
+        *(uint2*)(stg + (j * 16 + l16) * Cfg::STG_PITCH + (i * 16 + 4 * quad) * 2) = pk;
       }
     }
   }
@@ -626,7 +649,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
         static_assert(64 % PCH == 0 && Cfg::WTN % PRPI == 0 && NIT % BI == 0, "staged rows per wavefront");
         const int prow = lane / PCH, pchunk = lane % PCH;
         const char* pp = stg + prow * Cfg::STG_PITCH + pchunk * (EPL * 2);
-        const __amdgpu_buffer_rsrc_t xr = bx_resource(xmat + (int64_t)col_base * ldct + row_base);
+        const __amdgpu_buffer_rsrc_t xr = bx_resource(uniform_ptr(xmat + (int64_t)col_base * ldct + row_base));
         const int xl = (prow * ldct + pchunk * EPL) * (int)sizeof(XT);  // per lane
         auto run = [&](auto caut) {
           constexpr int CAUT = decltype(caut)::value;
@@ -696,18 +719,17 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
 //     lane, each instruction writing whole 128-byte lines.  Sixteen outstanding stores also stay countable
 //     next to the ring's loads (the wait counter has six bits), and their acknowledgements come back
 //     under the next tile's first slab.
-// OUT_T false stores C[row][col]: the MFMA operands are swapped, so that a lane's four consecutive
-// accumulator registers are four consecutive columns of one output row (8 bytes of a C row).
+// OUT_T false stores C[row][col]: the MFMA operands are swapped, so that a lane's four accumulator
+// elements are four consecutive columns of one output row (8 bytes of a C row).
 // OUT_T true stores Ct[col][row] (the product of a tall input, kept in the wide layout): operands
-// in the usual order, four consecutive registers are four consecutive rows = 8 bytes of a Ct row.
-// Either way a staged chunk is 32 lines x 128 bytes from two 32x32 accumulator tiles.
+// in the usual order, the four elements are four consecutive rows = 8 bytes of a Ct row.
+// Either way a staged chunk is 32 lines x 128 bytes from eight 16x16 accumulator tiles.
 template <class Cfg, bool OUT_T>
 __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams p, const int total_tiles) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
-  constexpr int TM = Cfg::TM, TN = Cfg::TN, KK = Cfg::KK, NSTAGE = Cfg::NSTAGE;
-  constexpr int NM = TM * TN, NR = TM + TN, LPS = Cfg::LOADS_PER_STAGE;
-  constexpr int RPM = (NR + NM - 1) / NM, LPM = (LPS + NM - 1) / NM;
-  static_assert(NSTAGE == 2 && TM == 4 && TN == 2 && KK % 2 == 0, "written for 128x64 wavefront tiles, two-slot ring");
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, ST = Cfg::ST, HALVES = Cfg::HALVES, NSTAGE = Cfg::NSTAGE;
+  constexpr int HP = HALVES * ST, NM = 16, LPS = Cfg::LOADS_PER_STAGE;
+  static_assert(NSTAGE == 2 && TM == 8 && TN == 4 && LPS <= NM / 2, "written for 128x64 wavefront tiles, two-slot ring");
   constexpr int STG_WAVE = 32 * 128;  // staging bytes per wavefront: 32 lines of 128 bytes
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -755,8 +777,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
   static_assert(BK % QROWS_PER_LOAD == 0 && QROWS_PER_LOAD % 4 == 0, "K-major tile/threads");
   const int qk_row = tid / QCPR;
   const int qk_chunk = ((((tid % QCPR) >> 2) ^ (qk_row & 3)) << 2) | (tid & 3);
-  const uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
-  const uint32_t offQ = (uint32_t)(qk_row * p.ldq + qk_chunk * 8) * 2u;
+  uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
+  uint32_t offQ = (uint32_t)(qk_row * p.ldq + qk_chunk * 8) * 2u;
   const uint32_t stepP = (uint32_t)(Cfg::ROWS_PER_LOAD * p.ldp) * 2u;
   const uint32_t stepQ = (uint32_t)(QROWS_PER_LOAD * p.ldq) * 2u;
   const int64_t slabQ = (int64_t)BK * p.ldq * 2;
@@ -790,63 +812,62 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
     const bool nx = kt >= KT;
     const int k = nx ? kt - KT : kt;
     char* l = lds + buf * Cfg::P_BYTES + wave * (64 * 16);
+    // wave-uniform base in scalar registers + one per-lane offset per operand (see the kernel above)
     if (j < Cfg::P_LOADS) {
-      const char* src = (nx ? gP_n : gP_c) + (int64_t)k * (BK * 2) + (offP + j * stepP);
-      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
+      const char* src = (nx ? gP_n : gP_c) + (int64_t)k * (BK * 2) + (uint64_t)j * stepP;
+      asm volatile("" : "+s"(src), "+v"(offP));
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src + offP), LDS_PTR(l + j * (Cfg::NT * 16)), 16, 0, 0);
     } else {
       const int jq = j - Cfg::P_LOADS;
-      const char* src = (nx ? gQ_n : gQ_c) + k * slabQ + (offQ + jq * stepQ);
-      __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(l + NSTAGE * Cfg::P_BYTES + jq * (Cfg::NT * 16)), 16, 0, 0);
+      const char* src = (nx ? gQ_n : gQ_c) + k * slabQ + (uint64_t)jq * stepQ;
+      asm volatile("" : "+s"(src), "+v"(offQ));
+      __builtin_amdgcn_global_load_lds(GLB_PTR(src + offQ), LDS_PTR(l + NSTAGE * Cfg::P_BYTES + jq * (Cfg::NT * 16)), 16, 0, 0);
     }
   };
 
   // ---- LDS -> register fragments (see the kernel above)
   const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
-  const int frow = lane & 31;
-  const int fhalf = lane >> 5;
-  const int fswz = (frow / Cfg::SWZ_DIV) % Cfg::CPR;
-  uint32_t aoff[KK];
+  const int l16 = lane & 15, quad = lane >> 4;
+  const int fswz = (l16 / Cfg::SWZ_DIV) % Cfg::CPR;
+  uint32_t aoff[ST];
 #pragma unroll
-  for (int kk = 0; kk < KK; ++kk)
-    aoff[kk] = lds_base + (uint32_t)((wm * Cfg::WTM + frow) * (BK * 2) + ((kk * 2 + fhalf) ^ fswz) * 16);
+  for (int st = 0; st < ST; ++st)
+    aoff[st] = lds_base + (uint32_t)((wm * Cfg::WTM + l16) * (BK * 2) + ((st * 4 + quad) ^ fswz) * 16);
   uint32_t qoff[TN];
-  {
-    const int g16 = lane >> 4, t16 = lane & 15;
 #pragma unroll
-    for (int r = 0; r < TN; ++r)
-      qoff[r] = lds_base + (uint32_t)(NSTAGE * Cfg::P_BYTES + (8 * (g16 >> 1) + (t16 >> 2)) * (BN * 2) +
-                                      ((((wn * Cfg::WTN + r * 32) >> 5) ^ (t16 >> 2)) << 6) + (g16 & 1) * 32 +
-                                      (t16 & 3) * 8);
-  }
-  typedef FragSched<TM, TN, true> FS;
-  bf16x8 fa[2][TM], fb[2][TN];
-  auto read_frag = [&](auto bufc, auto kkc, auto fc, auto rc) {
-    constexpr int buf = decltype(bufc)::value, kk = decltype(kkc)::value, f = decltype(fc)::value,
-                  r = decltype(rc)::value;
-    if constexpr (r == 0 || r > TN) {
-      constexpr int i = r == 0 ? 0 : r - TN;
-      lds_read16<buf * Cfg::P_BYTES + i * (32 * BK * 2)>(fa[f][i], aoff[kk]);
+  for (int j = 0; j < TN; ++j)
+    qoff[j] = lds_base + (uint32_t)(NSTAGE * Cfg::P_BYTES + (8 * quad + (l16 >> 2)) * (BN * 2) +
+                                    ((((wn * Cfg::WTN + j * 16) >> 5) ^ (l16 >> 2)) << 6) + (j & 1) * 32 +
+                                    (l16 & 3) * 8);
+  typedef FragSched<HALVES, ST, true> FS;
+  bf16x8 fa[2][4], fb[2][TN];
+  auto read_frag = [&](auto bufc, auto hnc, auto rc) {
+    constexpr int buf = decltype(bufc)::value, hn = decltype(hnc)::value, r = decltype(rc)::value;
+    constexpr int st = hn / HALVES, part = hn % HALVES, fs = hn & 1, bs = st & 1;
+    if constexpr (part != 0) {
+      lds_read16<buf * Cfg::P_BYTES + (4 + r) * (16 * BK * 2)>(fa[fs][r], aoff[st]);
+    } else if constexpr (r == 0 || r > 4) {
+      constexpr int i = r == 0 ? 0 : r - 4;
+      lds_read16<buf * Cfg::P_BYTES + i * (16 * BK * 2)>(fa[fs][i], aoff[st]);
     } else {
       constexpr int j = r - 1;
-      lds_read_tr<buf * Cfg::Q_BYTES + kk * (16 * BN * 2), 4 * BN * 2>(fb[f][j], qoff[j]);
+      lds_read_tr<buf * Cfg::Q_BYTES + st * (32 * BN * 2), 4 * BN * 2>(fb[bs][j], qoff[j]);
     }
   };
   typedef std::integral_constant<int, 0> ic0;
 
-  f32x16 acc[TM][TN];
+  f32x4 acc[TM][TN];
   auto clear_acc = [&]() {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+      for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   };
   clear_acc();
 
-  // ---- epilogue addressing: lane = (line wl, half wh) when staging, (line rl, 16-byte piece rq) when storing
+  // ---- epilogue addressing: lane = (line l16 of a tile, 8-byte piece quad) when staging, (line rl, 16-byte
+  // piece rq) when storing
   char* stg = lds + Cfg::RING_BYTES + wave * STG_WAVE;
-  const int wl = lane & 31, wh = lane >> 5;
   const int rl = lane >> 3, rq = lane & 7;
   const int ld_out = OUT_T ? p.ldct : p.ldc;
 
@@ -855,40 +876,38 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
     const int col_base = tj * BN + wn * Cfg::WTN;
     bf16_t* out = OUT_T ? p.Ct + (int64_t)b * p.strideCt + (int64_t)col_base * ld_out + row_base
                         : p.C + (int64_t)b * p.strideC + (int64_t)row_base * ld_out + col_base;
-    const __amdgpu_buffer_rsrc_t rs = bx_resource(out);
+    const __amdgpu_buffer_rsrc_t rs = bx_resource(uniform_ptr(out));
     const int lane_bytes = (rl * ld_out + rq * 8) * 2;
     const float alpha = gemm_alpha(p, b);  // 1 unless a per-matrix factor rides on this launch
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      // chunk c: accumulator tiles t2 = 0, 1 side by side along the 128-byte lines
+      // chunk c: 32 output lines of 128 bytes.  OUT_T false: C rows 32 c .. 32 c + 31 of the wavefront tile
+      // (accumulator tiles i = 2 c, 2 c + 1, all j); OUT_T true: Ct lines = C columns 32 (c / 2) .. + 31
+      // (j = 2 (c / 2), + 1) by C rows 64 (c % 2) .. + 63 (i = 4 (c % 2) .. + 3).
       const int line0 = OUT_T ? (c >> 1) * 32 : c * 32;   // first output line of the chunk (relative)
       const int run0 = OUT_T ? (c & 1) * 64 : 0;          // first element of the chunk within a line
 #pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        const f32x16& a = OUT_T ? acc[(c & 1) * 2 + t2][c >> 1] : acc[c][t2];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          uint2 pk;
-          pk.x = pack_bf16x2(alpha * a[g * 4 + 0], alpha * a[g * 4 + 1]);
-          pk.y = pack_bf16x2(alpha * a[g * 4 + 2], alpha * a[g * 4 + 3]);
-          // 8-byte piece t2*8 + 2g + wh of line wl; XOR with the line pair number spreads the 32 lines of
-          // a half wavefront over all 64 banks
-          *(uint2*)(stg + wl * 128 + (((t2 * 8 + 2 * g + wh) ^ ((wl >> 1) & 15)) << 3)) = pk;
-        }
+      for (int t = 0; t < 8; ++t) {
+        const f32x4& a = OUT_T ? acc[4 * (c & 1) + (t & 3)][2 * (c >> 1) + (t >> 2)] : acc[2 * c + (t >> 2)][t & 3];
+        uint2 pk;
+        pk.x = pack_bf16x2(alpha * a[0], alpha * a[1]);
+        pk.y = pack_bf16x2(alpha * a[2], alpha * a[3]);
+        // 8-byte piece 4 (t % 4) + quad of line 16 (t / 4) + l16; XOR with twice the line pair number spreads
+        // the 16 lines of half a wavefront over all 64 banks and keeps 16-byte pairs together
+        const int line = 16 * (t >> 2) + l16;
+        *(uint2*)(stg + line * 128 + (((4 * (t & 3) + quad) ^ (((line >> 1) & 7) << 1)) << 3)) = pk;
       }
       asm volatile("" ::: "memory");
-      uint2 lo[4], hi[4];
+      uint4 v[4];
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
         const int line = rl + 8 * it;
-        const int sw = (line >> 1) & 15;
-        lo[it] = *(const uint2*)(stg + line * 128 + (((2 * rq) ^ sw) << 3));
-        hi[it] = *(const uint2*)(stg + line * 128 + (((2 * rq + 1) ^ sw) << 3));
+        v[it] = *(const uint4*)(stg + line * 128 + (((2 * rq) ^ (((line >> 1) & 7) << 1)) << 3));
       }
       asm volatile("" ::: "memory");
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
-        const bx_u32x4 o = {lo[it].x, lo[it].y, hi[it].x, hi[it].y};
+        const bx_u32x4 o = {v[it].x, v[it].y, v[it].z, v[it].w};
         __builtin_amdgcn_raw_buffer_store_b128(o, rs, lane_bytes, ((line0 + 8 * it) * ld_out + run0) * 2, 0);
       }
     }
@@ -898,7 +917,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
 #pragma unroll
   for (int j = 0; j < LPS; ++j) issue_load(0, 0, j);
   pipeline_barrier<0>();
-  static_for<0, NR>([&](auto rc) { read_frag(ic0(), ic0(), ic0(), rc); });
+  static_for<0, 8>([&](auto rc) { read_frag(ic0(), ic0(), rc); });
 #pragma unroll
   for (int j = 0; j < LPS; ++j) issue_load(1, 1, j);
   __builtin_amdgcn_sched_barrier(0);
@@ -906,30 +925,27 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
   for (;;) {
     // ---- one tile: the main loop of the kernel above; refills past the tile's last slab fetch the next tile
     for (int kt0 = 0; kt0 < KT; kt0 += NSTAGE) {
-      static_for<0, NSTAGE * KK>([&](auto skc) {
-        constexpr int s = decltype(skc)::value / KK, kk = decltype(skc)::value % KK;
-        constexpr int cur = kk & 1, nxt = cur ^ 1;
-        constexpr bool last = (kk == KK - 1);
+      static_for<0, NSTAGE * HP>([&](auto shc) {
+        constexpr int s = decltype(shc)::value / HP, hp = decltype(shc)::value % HP;
+        constexpr int st = hp / HALVES, part = hp % HALVES, fs = hp & 1, bs = st & 1;
+        constexpr bool last = (hp == HP - 1);
         if constexpr (last) pipeline_barrier<0>();
         static_for<0, NM>([&](auto qc) {
-          constexpr int q = decltype(qc)::value, i = q / TN, j = q % TN;
-          frag_wait<FS::allowed(q)>(fa[cur][i], fb[cur][j]);
+          constexpr int q = decltype(qc)::value, i = q / 4, j = q % 4;
+          frag_wait<FS::allowed(hp, q)>(fa[fs][i], fb[bs][j]);
           if constexpr (OUT_T)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+            acc[part * 4 + i][j] =
+                __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[fs][i], fb[bs][j], acc[part * 4 + i][j], 0, 0, 0);
           else
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+            acc[part * 4 + i][j] =
+                __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[bs][j], fa[fs][i], acc[part * 4 + i][j], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
-          static_for<q * RPM, ((q + 1) * RPM < NR ? (q + 1) * RPM : NR)>([&](auto rc) {
-            if constexpr (last)
-              read_frag(std::integral_constant<int, (s + 1) % NSTAGE>(), ic0(), std::integral_constant<int, nxt>(), rc);
-            else
-              read_frag(std::integral_constant<int, s>(), std::integral_constant<int, kk + 1>(),
-                        std::integral_constant<int, nxt>(), rc);
-          });
-          if constexpr (last) {
-#pragma unroll
-            for (int jl = q * LPM; jl < (q + 1) * LPM && jl < LPS; ++jl) issue_load(kt0 + s + NSTAGE, s, jl);
+          if constexpr (FS::read_behind(hp, q) >= 0) {
+            typedef std::integral_constant<int, FS::read_behind(hp, q)> rc;
+            if constexpr (last) read_frag(std::integral_constant<int, (s + 1) % NSTAGE>(), ic0(), rc());
+            else read_frag(std::integral_constant<int, s>(), std::integral_constant<int, hp + 1>(), rc());
           }
+          if constexpr (last && (q & 1) && q / 2 < LPS) issue_load(kt0 + s + NSTAGE, s, q / 2);
           __builtin_amdgcn_sched_barrier(0);
         });
       });
@@ -937,7 +953,8 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
     // The first fragments of the next tile are on their way into set 0.  Let them land before the epilogue:
     // its register traffic must not meet a transposing read still in flight.
     asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]), "+v"(fb[0][0]), "+v"(fb[0][1]));
+                 : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]), "+v"(fb[0][0]), "+v"(fb[0][1]),
+                   "+v"(fb[0][2]), "+v"(fb[0][3]));
     store_tile(b_c, ti_c, tj_c);
     pid += (int)gridDim.x;
     if (pid >= total_tiles) break;

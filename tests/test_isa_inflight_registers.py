@@ -28,64 +28,81 @@ def _regs(tok):
 
 
 def walk(body):
-    """Returns (number of LDS reads seen, list of hazards) for one kernel's assembly lines."""
+    """Returns (number of LDS reads seen, list of hazards) for one kernel's assembly lines.
+
+    The instruction stream is followed along both outcomes of every conditional branch, each branch
+    outcome once, carrying the queues of outstanding reads as they stand on first arrival (so a loop
+    body is walked a second time with what its first pass left in flight)."""
     labels = {l.split(":")[0].strip(): i for i, l in enumerate(body) if re.match(r"\.L\w+:", l.strip())}
-    taken, queue, vmq, hazards = set(), [], [], []
-    pc = steps = n_tr = 0
-    in_asm = False
-    while pc < len(body) and steps < 500000:
-        steps += 1
-        if "#ASMSTART" in body[pc]:
-            in_asm = True
-        elif "#ASMEND" in body[pc]:
-            in_asm = False
-        cur, s = pc, body[pc].split(";")[0].strip()
-        pc += 1
-        if not s or s.startswith(".") or s.endswith(":"):
-            continue
-        op, *args = s.split()
-        if op == "s_endpgm":
-            break
-        if op.startswith("s_cbranch") or op == "s_branch":
-            tgt = args[0]
-            if tgt in labels and labels[tgt] < cur and cur not in taken:
-                taken.add(cur)
-                pc = labels[tgt]
-            elif op == "s_branch" and tgt in labels and labels[tgt] > cur:
-                pc = labels[tgt]
-            continue
-        if op == "s_waitcnt":
-            m = re.search(r"lgkmcnt\((\d+)\)", s)
-            if m:
-                del queue[: max(0, len(queue) - int(m.group(1)))]
-            m = re.search(r"vmcnt\((\d+)\)", s)
-            if m:
-                del vmq[: max(0, len(vmq) - int(m.group(1)))]
-            continue
-        inflight = set().union(*[q for q in queue + vmq if q]) if queue or vmq else set()
-        if re.match(r"(buffer|global|flat|scratch)_", op):
-            # vector memory: returns in order, counted by vmcnt.  The destination of a load issued from an
-            # assembly statement is in flight until a wait retires it (the compiler guards its own loads)
-            is_load = in_asm and "_load" in op and "_lds_" not in op and not op.endswith("_lds")
-            dest = _regs(args[0]) if is_load else set()
+    in_asm_at, inside = [], False
+    for l in body:
+        if "#ASMSTART" in l:
+            inside = True
+        elif "#ASMEND" in l:
+            inside = False
+        in_asm_at.append(inside)
+    explored, hazards, reads = set(), {}, set()
+    stack = [(0, [], [])]
+    steps = 0
+    while stack and steps < 4000000:
+        pc, queue, vmq = stack.pop()
+        while pc < len(body) and steps < 4000000:
+            steps += 1
+            cur, s = pc, body[pc].split(";")[0].strip()
+            in_asm = in_asm_at[pc]
+            pc += 1
+            if not s or s.startswith(".") or s.endswith(":"):
+                continue
+            op, *args = s.split()
+            if op == "s_endpgm":
+                break
+            if op.startswith("s_cbranch") or op == "s_branch":
+                tgt = labels.get(args[0])
+                if op == "s_branch":
+                    if tgt is None or (cur, True) in explored:
+                        break
+                    explored.add((cur, True))
+                    pc = tgt
+                    continue
+                if tgt is not None and (cur, True) not in explored:
+                    explored.add((cur, True))
+                    stack.append((tgt, list(queue), list(vmq)))
+                if (cur, False) in explored:
+                    break
+                explored.add((cur, False))
+                continue
+            if op == "s_waitcnt":
+                m = re.search(r"lgkmcnt\((\d+)\)", s)
+                if m:
+                    del queue[: max(0, len(queue) - int(m.group(1)))]
+                m = re.search(r"vmcnt\((\d+)\)", s)
+                if m:
+                    del vmq[: max(0, len(vmq) - int(m.group(1)))]
+                continue
+            inflight = set().union(*[q for q in queue + vmq if q]) if queue or vmq else set()
+            if re.match(r"(buffer|global|flat|scratch)_", op):
+                # vector memory: returns in order, counted by vmcnt.  The destination of a load issued from an
+                # assembly statement is in flight until a wait retires it (the compiler guards its own loads)
+                is_load = in_asm and "_load" in op and "_lds_" not in op and not op.endswith("_lds")
+                dest = _regs(args[0]) if is_load else set()
+                touched = set().union(*[_regs(a) for a in args]) if args else set()
+                if touched & inflight:
+                    hazards[cur] = s
+                vmq.append(dest)
+                continue
+            if op.startswith("ds_read"):
+                dest = _regs(args[0])
+                reads.add(cur)
+                if dest & inflight:
+                    hazards[cur] = s
+                queue.append(dest)
+                continue
             touched = set().union(*[_regs(a) for a in args]) if args else set()
             if touched & inflight:
-                hazards.append((cur, s))
-            vmq.append(dest)
-            continue
-        if op.startswith("ds_read"):
-            dest = _regs(args[0])
-            n_tr += 1
-            if dest & inflight:
-                hazards.append((cur, s))
-            queue.append(dest)
-            continue
-        touched = set().union(*[_regs(a) for a in args]) if args else set()
-        if touched & inflight:
-            hazards.append((cur, s))
-        if op.startswith("ds_") or op.startswith("s_load") or op.startswith("s_buffer_load"):
-            queue.append(set())
-    return n_tr, hazards
+                hazards[cur] = s
+            if op.startswith("ds_") or op.startswith("s_load") or op.startswith("s_buffer_load"):
+                queue.append(set())
+    return len(reads), sorted(hazards.items())
 
 
 def test_the_walk_flags_a_register_reused_before_the_wait():
