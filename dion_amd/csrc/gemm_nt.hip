@@ -88,7 +88,9 @@ __device__ __forceinline__ void static_for(F&& f) {
 // Every fragment is requested fifteen or more MFMAs before its first use.  Every read is an assembly
 // statement and so is every wait: the LDS returns in order, so "all but the newest N LDS instructions have
 // returned" is exactly "the fragments MFMA q needs are in their registers", with N counted here from the
-// issue order -- the LDS instructions issued after the later of the two fragments q needs.  (Left to the
+// issue order -- the LDS instructions issued after the later of the two fragments q needs.  Every MFMA
+// carries its wait, also where an earlier one already covers its fragments: dropping those nine of sixteen
+// measured 0.5-1.5 % slower on the polynomial and K-major launches.  (Left to the
 // compiler, every group of MFMAs starts with a wait for all outstanding reads, the last of which was
 // issued two MFMAs earlier.)  A K-major B fragment is two transposing reads.
 template <int HALVES, int ST, bool QK>
@@ -293,6 +295,11 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   constexpr int NM = 16;
   constexpr int LPS = Cfg::LOADS_PER_STAGE;
   static_assert(LPS <= NM / 2, "one refill load behind every second MFMA of a slab's last half");
+  // Refill of the slot a slab occupied: all of it during the slab's last half, or -- the plain product of two
+  // K-contiguous operands on 256-wide tiles, i.e. X X^T -- half then and half during the next slab's first half.
+  // Measured: X X^T 2-3 % faster that way; the polynomial GEMM (addend loads in the epilogue) 1 % slower, the
+  // K-major form (two-instruction fragment reads in the same half) 3 % slower, 128-wide tiles 10 % slower.
+  constexpr bool SPREAD = !QK && !HAS_D && BM == 256;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int tid = threadIdx.x;
@@ -462,11 +469,11 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   pipeline_barrier<(NSTAGE - 2) * LPS>();
   static_for<0, 8>([&](auto rc) { read_frag(ic0(), ic0(), rc); });
 #pragma unroll
-  for (int j = 0; j < LPS; ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
+  for (int j = 0; j < (SPREAD ? LPS / 2 : LPS); ++j) issue_load(NSTAGE - 1, NSTAGE - 1, j);
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- main loop.  Halves run back to back across slab boundaries: while the MFMAs of one half issue, the
-  // fragment reads of the next half (and, in the last half of a slab, the refill of the slot that slab
+  // fragment reads of the next half (and, from the last half of a slab on, the refill of the slot that slab
   // occupied) are slotted behind them.  sched_barrier pins that order.  KT is a multiple of NSTAGE
   // (launcher checks) so ring slots are compile-time constants.
   for (int kt0 = 0; kt0 < KT; kt0 += NSTAGE) {
@@ -487,7 +494,13 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
           if constexpr (last) read_frag(std::integral_constant<int, (s + 1) % NSTAGE>(), ic0(), rc());
           else read_frag(std::integral_constant<int, s>(), std::integral_constant<int, hp + 1>(), rc());
         }
-        if constexpr (last && (q & 1) && q / 2 < LPS) issue_load(kt0 + s + NSTAGE, s, q / 2);
+        if constexpr (SPREAD) {
+          if constexpr (last && q % 4 == 3 && q / 4 < LPS / 2) issue_load(kt0 + s + NSTAGE, s, q / 4);
+          if constexpr (hp == 0 && q % 4 == 3 && LPS / 2 + q / 4 < LPS)
+            issue_load(kt0 + s - 1 + NSTAGE, (s + NSTAGE - 1) % NSTAGE, LPS / 2 + q / 4);
+        } else {
+          if constexpr (last && (q & 1) && q / 2 < LPS) issue_load(kt0 + s + NSTAGE, s, q / 2);
+        }
         __builtin_amdgcn_sched_barrier(0);
       });
     });
