@@ -354,13 +354,14 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   const int ld_chunk = ld_phys ^ ((ld_row / Cfg::SWZ_DIV) % Cfg::CPR);
   const char* gP = (const char*)(p.P + (int64_t)b * p.strideP + (int64_t)(ti * BM) * p.ldp);
   // QK: the Q tile is BK rows (reduction index) of BN bf16; chunk q lands at LDS byte q*16 and holds
-  // logical chunk ((c >> 2) ^ (row & 3)) << 2 | (c & 3), c = q % QCPR, of tile row q / QCPR: the four
-  // rows one transposing read gathers land in four distinct 64-byte bank groups.
+  // logical chunk ((c >> 2) ^ (row & 3)) << 2 | ((c & 3) ^ 2 * ((row >> 3) & 1)), c = q % QCPR, of tile row
+  // q / QCPR: the four rows one transposing read gathers land in four distinct 64-byte bank groups, and
+  // the rows 8 apart that neighbouring 16-lane groups read in the two 32-byte halves of a group.
   constexpr int QCPR = BN / 8;               // 16-byte chunks per K-major tile row
   constexpr int QROWS_PER_LOAD = Cfg::NT / QCPR;
-  static_assert(!QK || (BK % QROWS_PER_LOAD == 0 && QROWS_PER_LOAD % 4 == 0), "K-major tile/threads");
+  static_assert(!QK || (BK % QROWS_PER_LOAD == 0 && QROWS_PER_LOAD % 16 == 0), "K-major tile/threads");
   const int qk_row = tid / QCPR;
-  const int qk_chunk = ((((tid % QCPR) >> 2) ^ (qk_row & 3)) << 2) | (tid & 3);
+  const int qk_chunk = ((((tid % QCPR) >> 2) ^ (qk_row & 3)) << 2) | ((tid & 3) ^ (((qk_row >> 3) & 1) << 1));
   const char* gQ = QK ? (const char*)(p.Q + (int64_t)b * p.strideQ + tj * BN)
                       : (const char*)(p.Q + (int64_t)b * p.strideQ + (int64_t)(tj * BN) * p.ldq);
   uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
@@ -419,14 +420,15 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   // QK fragments: a transposing read hands each 16-lane group a 4 (reduction index) x 16 (column) block, lane i
   // its column i; within the group, lane 4r+q addresses row r / 4-element piece q of the block.  Group g takes
   // reduction indices 8 g .. 8 g + 7 of the step (two reads of 4 rows); the 16 columns of fragment j are half
-  // of a 64-byte group of the tile row, which the swizzle keys on the row's index modulo 4.
+  // of a 64-byte group of the tile row; the swizzle keys the group on the row's index modulo 4 and the half
+  // on bit 3 of the row (= g & 1), so the 32 lanes served together cover all 64 banks once.
   uint32_t qoff[TN];
   if (QK) {
     const int t16 = lane & 15;
 #pragma unroll
     for (int j = 0; j < TN; ++j)
       qoff[j] = lds_base + (uint32_t)(NSTAGE * Cfg::P_BYTES + (8 * quad + (t16 >> 2)) * (BN * 2) +
-                                      ((((wn * Cfg::WTN + j * 16) >> 5) ^ (t16 >> 2)) << 6) + (j & 1) * 32 +
+                                      ((((wn * Cfg::WTN + j * 16) >> 5) ^ (t16 >> 2)) << 6) + ((j ^ quad) & 1) * 32 +
                                       (t16 & 3) * 8);
   }
 
@@ -787,9 +789,9 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
   const int ld_chunk = ld_phys ^ ((ld_row / Cfg::SWZ_DIV) % Cfg::CPR);
   constexpr int QCPR = BN / 8;
   constexpr int QROWS_PER_LOAD = Cfg::NT / QCPR;
-  static_assert(BK % QROWS_PER_LOAD == 0 && QROWS_PER_LOAD % 4 == 0, "K-major tile/threads");
+  static_assert(BK % QROWS_PER_LOAD == 0 && QROWS_PER_LOAD % 16 == 0, "K-major tile/threads");
   const int qk_row = tid / QCPR;
-  const int qk_chunk = ((((tid % QCPR) >> 2) ^ (qk_row & 3)) << 2) | (tid & 3);
+  const int qk_chunk = ((((tid % QCPR) >> 2) ^ (qk_row & 3)) << 2) | ((tid & 3) ^ (((qk_row >> 3) & 1) << 1));
   uint32_t offP = (uint32_t)(ld_row * p.ldp + ld_chunk * 8) * 2u;
   uint32_t offQ = (uint32_t)(qk_row * p.ldq + qk_chunk * 8) * 2u;
   const uint32_t stepP = (uint32_t)(Cfg::ROWS_PER_LOAD * p.ldp) * 2u;
@@ -850,7 +852,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_qk_walk_kernel(const GemmParams 
 #pragma unroll
   for (int j = 0; j < TN; ++j)
     qoff[j] = lds_base + (uint32_t)(NSTAGE * Cfg::P_BYTES + (8 * quad + (l16 >> 2)) * (BN * 2) +
-                                    ((((wn * Cfg::WTN + j * 16) >> 5) ^ (l16 >> 2)) << 6) + (j & 1) * 32 +
+                                    ((((wn * Cfg::WTN + j * 16) >> 5) ^ (l16 >> 2)) << 6) + ((j ^ quad) & 1) * 32 +
                                     (l16 & 3) * 8);
   typedef FragSched<HALVES, ST, true> FS;
   bf16x8 fa[2][4], fb[2][TN];
