@@ -89,7 +89,7 @@ def cpu_baseline(ns: str):
 def measured_traffic():
     """HBM bytes per launch of the dominant kernel, from the committed rocprofv3 --pmc summary
     (profiles/gemm_xprime_traffic.json: FETCH_SIZE + WRITE_SIZE, each scaled by the same counter's
-    reading for muon_post_kernel, a streaming kernel of known traffic in the same run).  None when
+    reading for a streaming kernel of known traffic in the same run).  None when
     the file is absent."""
     path = os.path.join(ROOT, "profiles", "gemm_xprime_traffic.json")
     try:
@@ -392,7 +392,7 @@ def main() -> int:
         achieved = flop3 / (ms3 * 1e-3) * 1e-12
         result["roofline"] = {
             "bound": "mfma",
-            "kernel": "gemm_nt_kernel<256x256x64, 8 waves, direct-to-LDS loads, K-major second operand> (X' = B X)",
+            "kernel": "gemm_nt_kernel<256x256x64, 8 waves, 16x16x32 MFMAs, direct-to-LDS loads, K-major second operand> (X' = B X)",
             "achieved": round(achieved, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
