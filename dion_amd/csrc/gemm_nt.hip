@@ -380,7 +380,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_nt_kernel(const GemmParams p, co
   // two-slot ring the barrier waits for every outstanding load, so the load count per slab is free to vary.)
   const bool one_operand = !QK && p.tri && ti == tj && p.P == p.Q && p.ldp == p.ldq && p.strideP == p.strideQ;
   // LDS layout of the ring: [P slot 0][P slot 1][Q slot 0][Q slot 1].  With the two slots of an operand
-  // side by side, slot, wavefront-tile row block and k slice all fit the offset field of the LDS read
+  // side by side, slot, wavefront-tile row block and k step all fit the offset field of the LDS read
   // instructions: the per-lane address registers below are all the address arithmetic the loop needs.
   static_assert(Cfg::P_BYTES == Cfg::Q_BYTES, "square tiles: a one-operand tile reads Q's fragments from P's slots");
   auto issue_load = [&](int kt, int buf, int j) {
