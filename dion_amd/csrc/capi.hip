@@ -376,57 +376,78 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
 
   const int mp = pl.mp, np = pl.np;
   const int64_t sX = (int64_t)mp * np, sA = (int64_t)mp * mp;
-  if (sumsq) {
-    NsStep s = blank_step(NsStep::kNormFinalize, "frobenius norm from the caller's partial sums");
-    s.batch = batch;
-    s.norm_scale = norm_scale;
-    s.eps = eps;
-    s.partial = const_cast<float*>(sumsq);
-    s.nblk = sumsq_blocks;
-    s.inv = inv;
-    call.push(s);
-  } else {
-    NsStep s = blank_step(NsStep::kNorm, "frobenius norm");
-    s.in = in;
-    s.in_dtype = in_dtype;
-    s.batch = batch;
-    s.R = rows;
-    s.C = cols;
-    s.norm_scale = norm_scale;
-    s.eps = eps;
-    s.partial = partial;
-    s.nblk = pl.nblk;
-    s.inv = inv;
-    call.push(s);
-  }
-  if (!sumsq) {
-    // Only X (short side along rows) is carried between iterations: X' = B X reads X with the
-    // reduction index along rows.  With no iteration at all the result is the prepared input, and
-    // the output copy of a tall input reads X^T: prepare that layout instead.
-    NsStep s = blank_step(NsStep::kPrepare, "prepare");
-    s.in = in;
-    s.in_dtype = in_dtype;
-    s.batch = batch;
-    s.R = rows;
-    s.C = cols;
-    s.inv = inv;
-    if (pl.tall) {
-      s.Rp = np;
-      s.Cp = mp;
-      s.same = n_iters > 0 ? nullptr : Xt;
-      s.ld_same = mp;
-      s.stride_same = sX;
-      s.trans = n_iters > 0 ? X[0] : nullptr;
-      s.ld_trans = np;
-      s.stride_trans = sX;
+  // An input that fills whole tiles is not scaled on its way in either: a wide bf16 one is read by the first
+  // GEMMs where it lies, any other is copied (rounded to bf16, transposed if tall) value for value, and the
+  // normalisation rides on the first two GEMMs as for a prepared input -- one pass over a wide bf16 input instead
+  // of two, and the same arithmetic whichever way (orientation, fp32 or bf16) a matrix is handed over.
+  const bool self_prep = !sumsq && aligned16((uint64_t)(uintptr_t)in) &&
+                         ns_accepts_prepared(batch, rows, cols, flags, n_iters);
+  const bool in_place = self_prep && !pl.tall && in_dtype == DION_BF16;
+  const bool copy_first = self_prep && pl.tall;
+  auto plan_norm = [&]() {
+    if (sumsq) {
+      NsStep s = blank_step(NsStep::kNormFinalize, "frobenius norm from the caller's partial sums");
+      s.batch = batch;
+      s.norm_scale = norm_scale;
+      s.eps = eps;
+      s.partial = const_cast<float*>(sumsq);
+      s.nblk = sumsq_blocks;
+      s.inv = inv;
+      call.push(s);
     } else {
-      s.Rp = mp;
-      s.Cp = np;
-      s.same = X[0];
-      s.ld_same = np;
-      s.stride_same = sX;
+      // (over the transposed copy of a tall input that is copied unscaled: the sum then runs in the order it
+      // runs in for the same matrix handed over wide, and the two calls agree bit for bit)
+      NsStep s = blank_step(NsStep::kNorm, "frobenius norm");
+      s.in = copy_first ? (const void*)X[0] : in;
+      s.in_dtype = copy_first ? DION_BF16 : in_dtype;
+      s.batch = batch;
+      s.R = copy_first ? mp : rows;
+      s.C = copy_first ? np : cols;
+      s.norm_scale = norm_scale;
+      s.eps = eps;
+      s.partial = partial;
+      s.nblk = pl.nblk;
+      s.inv = inv;
+      call.push(s);
     }
-    call.push(s);
+  };
+  auto plan_prepare = [&]() {
+    if (!sumsq && !in_place) {
+      // Only X (short side along rows) is carried between iterations: X' = B X reads X with the
+      // reduction index along rows.  With no iteration at all the result is the prepared input, and
+      // the output copy of a tall input reads X^T: prepare that layout instead.
+      NsStep s = blank_step(NsStep::kPrepare, "prepare");
+      s.in = in;
+      s.in_dtype = in_dtype;
+      s.batch = batch;
+      s.R = rows;
+      s.C = cols;
+      s.inv = self_prep ? nullptr : inv;  // null: plain copy
+      if (pl.tall) {
+        s.Rp = np;
+        s.Cp = mp;
+        s.same = n_iters > 0 ? nullptr : Xt;
+        s.ld_same = mp;
+        s.stride_same = sX;
+        s.trans = n_iters > 0 ? X[0] : nullptr;
+        s.ld_trans = np;
+        s.stride_trans = sX;
+      } else {
+        s.Rp = mp;
+        s.Cp = np;
+        s.same = X[0];
+        s.ld_same = np;
+        s.stride_same = sX;
+      }
+      call.push(s);
+    }
+  };
+  if (copy_first) {
+    plan_prepare();
+    plan_norm();
+  } else {
+    plan_norm();
+    plan_prepare();
   }
 
   const bool direct = (mp == pl.m && np == pl.n);
@@ -458,9 +479,10 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
   };
   // A prepared input is the unnormalised X_0: every GEMM that reads it carries the factor 1/(||X_0|| s + eps)
   // (squared for X_0 X_0^T); products of these GEMMs are normalised, and so is every later X.
-  const bf16_t* const x_raw = sumsq ? (const bf16_t*)in : nullptr;
+  const bf16_t* const x_raw = (sumsq || in_place) ? (const bf16_t*)in : self_prep ? X[0] : nullptr;
+  bool x_written = false;  // an X' has been written: from then on every X is normalised
   auto scaled = [&](GemmParams& p, const bf16_t* Xc, int pow) {
-    if (x_raw && Xc == x_raw) {
+    if (x_raw && Xc == x_raw && !x_written) {
       p.scale_vec = inv;
       p.scale_pow = pow;
     }
@@ -555,8 +577,7 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
 
   int cur = 0;
   bool wrote_out = false;
-  // the matrix the next GEMM reads as X: the caller's prepared input until the first X' is written
-  bool x_written = false;
+  // the matrix the next GEMM reads as X: the unnormalised input until the first X' is written
   auto xc = [&]() -> const bf16_t* { return (x_raw && !x_written) ? x_raw : X[cur]; };
   if (!pl.gram) {
     for (int it = 0; it < n_iters; ++it) {
@@ -685,7 +706,7 @@ int ns_audit(const NsCall& call) {
         const size_t es = s.in_dtype == DION_BF16 ? 2 : 4;
         if (s.Rp % 64 || s.Cp % 64 || s.Rp < s.R || s.Cp < s.C) bad = "padded extents";
         else if (!rd(s.in, (size_t)s.batch * s.R * s.C * es)) bad = "input";
-        else if (!rd(s.inv, (size_t)s.batch * 4)) bad = "reciprocal norms";
+        else if (s.inv && !rd(s.inv, (size_t)s.batch * 4)) bad = "reciprocal norms";
         else if (s.same && !wr(s.same, span_bytes(s.batch, s.stride_same, s.Rp, s.ld_same, s.Cp, 2))) bad = "X";
         else if (s.trans && !wr(s.trans, span_bytes(s.batch, s.stride_trans, s.Cp, s.ld_trans, s.Rp, 2)))
           bad = "X^T";

@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void ns_prepare_kernel(const T* __restrict__ i
   __shared__ bf16_t tile[64][66];
   const int b = blockIdx.z;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  const float sc = inv_norm[b];
+  const float sc = inv_norm ? inv_norm[b] : 1.0f;  // (no factor: the values are copied as they are)
   const T* src = in + (int64_t)b * R * C;
   bf16_t* ds = same + (int64_t)b * stride_same;
   bf16_t* dt = trans + (int64_t)b * stride_trans;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256) void ns_prepare_vec_kernel(const T* __restrict
   __shared__ __attribute__((aligned(16))) bf16_t tile[64][72];
   const int b = blockIdx.z;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  const float sc = inv_norm[b];
+  const float sc = inv_norm ? inv_norm[b] : 1.0f;  // (no factor: the values are copied as they are)
   const T* src = in + (int64_t)b * R * C;
   bf16_t* ds = same + (int64_t)b * stride_same;
   bf16_t* dt = trans + (int64_t)b * stride_trans;

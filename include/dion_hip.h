@@ -71,6 +71,8 @@ int dion_ns_line_3(const void* B, const void* X, void* C, int batch, int m, int 
  *   coeffs  host array of n_iters*3 floats (a,b,c per iteration)
  *   X0 = bf16(in) / (||bf16(in)||_F * norm_scale + eps)  per matrix, then n_iters times
  *   A = X X^T; B = b A + c A A; X = a X + B X   on the orientation with rows <= cols.
+ *   (For matrices that fill whole GEMM tiles the division is not a pass of its own: the factor is applied
+ *   in the fp32 epilogue of the first two GEMMs, and a wide bf16 `in` is read where it lies.)
  *   flags: DION_NS_GRAM selects the Gram-matrix recurrence (call site
  *   dion/megabatch_base.py:77-94) with a restart at iteration `gram_reset` (<=0: none).  Both forms
  *   apply the same polynomial; the recurrence only saves work for long matrices, so it is used
