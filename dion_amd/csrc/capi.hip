@@ -382,7 +382,9 @@ int ns_build(const void* in, int in_dtype, void* out, int batch, int rows, int c
   // of two, and the same arithmetic whichever way (orientation, fp32 or bf16) a matrix is handed over.
   const bool self_prep = !sumsq && aligned16((uint64_t)(uintptr_t)in) &&
                          ns_accepts_prepared(batch, rows, cols, flags, n_iters);
-  const bool in_place = self_prep && !pl.tall && in_dtype == DION_BF16;
+  // (not when `out` overlaps `in`: the copy is then what keeps a caller's in-place call working)
+  const bool aliased = out && call.out_lo < call.in_hi && call.in_lo < call.out_hi;
+  const bool in_place = self_prep && !pl.tall && in_dtype == DION_BF16 && !aliased;
   const bool copy_first = self_prep && pl.tall;
   auto plan_norm = [&]() {
     if (sumsq) {
